@@ -1,0 +1,157 @@
+/*
+ * tpamd.h - C ABI of the MI355X (gfx950) hot path of a tensor-parallel transformer layer:
+ * state-dict slicing, rank-shard Linears and the single-device partial-sum reduction.
+ *
+ * The reference implementation (BlackSamorez/tensor_parallel) is pure Python and has no FFI.
+ * Each entry point below names the Python call of the reference whose work it performs.
+ *
+ * Conventions
+ *   - every pointer named *_dev is device memory of the current HIP device; everything else is host memory;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); all work is enqueued on it
+ *     and the call returns without waiting for it;
+ *   - matrices are row-major with an explicit leading dimension in ELEMENTS;
+ *   - return value: 0 on success, a negative tpamd_status otherwise; tpamd_last_error() then returns a
+ *     message for the calling thread;
+ *   - the library keeps no mutable global state besides that thread-local message: every entry point
+ *     may be called concurrently from several host threads.
+ */
+#ifndef TPAMD_H
+#define TPAMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPAMD_ABI_VERSION 1
+
+typedef enum tpamd_status {
+    TPAMD_OK = 0,
+    TPAMD_ERR_INVALID = -1,     /* bad argument (shape, alignment, dtype, null pointer) */
+    TPAMD_ERR_UNSUPPORTED = -2, /* legal request this build has no kernel for */
+    TPAMD_ERR_HIP = -3,         /* a HIP runtime call failed */
+    TPAMD_ERR_NOMEM = -4        /* host or device allocation failed */
+} tpamd_status;
+
+typedef enum tpamd_dtype {
+    TPAMD_BF16 = 0,
+    TPAMD_F16 = 1,
+    TPAMD_F32 = 2
+} tpamd_dtype;
+
+/* How tpamd_reduce_partials accumulates. */
+typedef enum tpamd_accum {
+    /* ((p0 + p1) + p2) + ... with the running sum rounded to the tensor dtype after every add:
+     * the arithmetic of the reference's CPU reduction, `sum([...])` over same-dtype tensors
+     * (src/tensor_parallel/cross_device_ops.py:49), taken in rank order. */
+    TPAMD_ACCUM_STEPWISE = 0,
+    /* fp32 running sum over ranks 0..W-1, one rounding at the store. */
+    TPAMD_ACCUM_F32 = 1
+} tpamd_accum;
+
+/* Epilogue applied by the shard Linears before the store. */
+typedef enum tpamd_act {
+    TPAMD_ACT_NONE = 0,
+    TPAMD_ACT_GELU = 1 /* exact erf GELU */
+} tpamd_act;
+
+int tpamd_abi_version(void);
+const char *tpamd_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Slicing engine.
+ *
+ * One job moves a 2-D byte region: `rows` rows of `row_bytes` bytes, row i read at
+ * src_dev + i*src_pitch and written at dst_dev + i*dst_pitch. A rank shard of a tensor split on
+ * axis d is one such region (rows = prod(shape[:d]), row_bytes = len*prod(shape[d+1:])*itemsize,
+ * src_pitch = shape[d]*prod(shape[d+1:])*itemsize); a grouped split is one region per group; the
+ * inverse (undo / gather) swaps the roles of the pitches.
+ *
+ * Replaces, for device-resident tensors, the strided copies behind
+ *   Split.__call__ / SplitInChunks.__call__ / SplitInGroupedChunks.__call__
+ *     (src/tensor_parallel/state_actions.py:47-48, :76-87, :101-109) followed by `.clone()`
+ *     (src/tensor_parallel/shard.py:160), applied to every tensor of a state dict by
+ *   process_state_ (src/tensor_parallel/shard.py:132-166) and
+ *   convert_state_dict (src/tensor_parallel/dispatch.py:75-131),
+ * and their inverses Split.undo / SplitInGroupedChunks.undo (state_actions.py:50-51, :111-119) and
+ * the "gather d" concatenation (src/tensor_parallel/cross_device_ops.py:39).
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct tpamd_copy_job {
+    const void *src_dev;
+    void *dst_dev;
+    uint64_t rows;
+    uint64_t row_bytes;
+    uint64_t src_pitch; /* bytes between consecutive source rows (ignored when rows == 1) */
+    uint64_t dst_pitch; /* bytes between consecutive destination rows */
+} tpamd_copy_job;
+
+typedef struct tpamd_copy_plan tpamd_copy_plan; /* opaque: device-resident job table */
+
+/* Validates the jobs, uploads the table (synchronously) and returns a plan that can be run any
+ * number of times. Regions of different jobs must not overlap in the destination. Zero-size jobs
+ * are legal and skipped. n_jobs == 0 gives a valid empty plan. */
+int tpamd_copy_plan_create(const tpamd_copy_job *jobs, size_t n_jobs, tpamd_copy_plan **plan_out);
+/* Enqueues the whole plan as ONE kernel launch on `stream`. */
+int tpamd_copy_plan_run(const tpamd_copy_plan *plan, void *stream);
+/* Bytes read (== bytes written) by one run of the plan. */
+uint64_t tpamd_copy_plan_bytes(const tpamd_copy_plan *plan);
+int tpamd_copy_plan_destroy(tpamd_copy_plan *plan);
+
+/* Scale state action: out[i] = in[i] / world_size in the tensor's dtype
+ * (Scale.__call__, src/tensor_parallel/state_actions.py:59-60). For bf16/f16 the quotient of the
+ * fp32-widened value is rounded to nearest even, as torch does. `mul != 0` multiplies instead
+ * (Scale.undo, state_actions.py:62-63). */
+int tpamd_scale(const void *in_dev, void *out_dev, uint64_t n_elems, int dtype, int world_size, int mul,
+                void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Partial-sum reduction: out = sum over r < world_size of parts[r], all W partials on this device.
+ * Replaces the "sum" output rule of a row-parallel module: AllReduce.__call__
+ * (src/tensor_parallel/communications.py:114-116) = ScatterReduce (:119-139) + AllGather (:142-171),
+ * whose arithmetic is reduce_add's `sum([...])` (src/tensor_parallel/cross_device_ops.py:43-50).
+ * `parts_dev` is a HOST array of `world_size` device pointers (1 <= world_size <= 16); `out_dev`
+ * may alias parts_dev[0]. `accum` is a tpamd_accum.
+ * ---------------------------------------------------------------------------------------------- */
+int tpamd_reduce_partials(const void *const *parts_dev, int world_size, void *out_dev, uint64_t n_elems,
+                          int dtype, int accum, void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Rank-shard Linears. y[M,N] = act(x[M,K] . w[N,K]^T + bias[N]); fp32 accumulation, one rounding to
+ * `dtype` at the store. This is the torch.nn.Linear call made by the wrapped module inside
+ * TensorParallelWrapper.forward (src/tensor_parallel/wrapper.py:69-72) on the sliced weight that
+ * process_state_ installed (src/tensor_parallel/shard.py:160, features fixed at :184-187):
+ *   column-parallel shard: w = rows ts(N,W,r) of the full weight, bias sliced alike;
+ *   row-parallel shard:    w = columns ts(K,W,r), x = the matching columns, bias NULL or pre-scaled;
+ *                          the result is a partial sum for tpamd_reduce_partials.
+ * bias_dev may be NULL. x, w, y must be 16-byte aligned; for bf16/f16 K, ldx and ldw must be
+ * multiples of 8 and N, ldy multiples of 4 (every shape the slicing rules above produce from
+ * head-aligned models satisfies this).
+ * ---------------------------------------------------------------------------------------------- */
+int tpamd_linear(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
+                 int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, void *stream);
+
+/* h[M,N] = silu(x . wg^T) * (x . wu^T): the gate/up pair of a SiLU-gated MLP shard in one pass over x
+ * (two column-parallel torch.nn.Linear calls, a SiLU and a product in the reference's wrapped module;
+ * weights sliced by `Split(world_size, dim=0)`, src/tensor_parallel/slicing_configs.py:376-378).
+ * The gate and up products are each rounded to `dtype`, then silu and the product are each rounded
+ * again, which is what the three separate torch ops of the reference produce. */
+int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void *wu_dev, void *h_dev, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldh, int dtype, void *stream);
+
+/* Weight-only int8 shard Linear with fp16/bf16 outlier columns:
+ *   y[m,n] = act( scale[n] * sum_k x[m,k]*wq[n,k]  +  sum_j x[m,outlier_idx[j]] * w_out[n,j]  + bias[n] )
+ * wq is int8 [N,K] (zero in the outlier columns), scale fp32 [N], outlier_idx int32 [n_out] (sorted,
+ * distinct, < K), w_out [N,n_out] in `dtype` with leading dimension ld_wout. Not part of the reference
+ * (its README points to LLM.int8 notebooks); defined here in closed form.
+ * Requirements: dtype is F16 or BF16; K % 16 == 0; ldw (int8 elements) % 16 == 0. */
+int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,
+                    const void *w_out_dev, int64_t n_out, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ld_wout, int64_t ldy, int dtype, int act,
+                    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPAMD_H */

@@ -1,0 +1,27 @@
+"""CPU restatement of the reference's per-rank hot path (BlackSamorez/tensor_parallel v2.0.0).
+
+TEST INFRASTRUCTURE ONLY. Nothing under `tensor_parallel_amd/` imports this package; only `tests/`, the smoke
+check and the benchmark's CPU-baseline leg do, and only as the checker or the baseline being timed.
+
+Modules and the reference code each one follows:
+  slicing.py        Split / SplitInChunks / SplitInGroupedChunks / Scale and their undo
+                    (src/tensor_parallel/state_actions.py:39-119), split_heads and the integer attribute
+                    rules (src/tensor_parallel/aux_actions.py:18-40), numpy on raw element arrays
+  naming.py         get_parameter_name_mapping (src/tensor_parallel/config.py:157-191) and
+                    convert_state_dict (src/tensor_parallel/dispatch.py:75-131) over the oracle's actions
+  reduce.py         the "sum" rule's arithmetic (src/tensor_parallel/cross_device_ops.py:49), bit-level
+  shard_forward.py  rank-shard Linears, the SiLU-gated MLP shard and the W-thread forward
+                    (src/tensor_parallel/wrapper.py:69-72, tensor_parallel.py:237-287), torch on CPU
+  quant.py          int8 weight-only quantisation with outlier columns - NOT in the reference: parity
+                    unpinned against it; defined in closed form and checked against fp64 matmul
+
+How each function is pinned (tests/test_oracle_*.py):
+  slicing      the reference's three docstring vectors (state_actions.py:40,67,94); torch.tensor_split on
+               every (n, W) with n < 40, W <= 9; brute-force index enumeration on small tensors;
+               undo(split) == identity; the shapes SURVEY lists for Llama-2-7B and Falcon-40B
+  naming       hand-derived Llama names; golden vectors written by tests/golden/make_golden.py
+  reduce       torch CPU bf16/fp16 addition (a third-party routine), W = 2 and chained W = 3..8
+  forward      sum of row-parallel partials == unsplit Linear, concat of column-parallel == unsplit Linear,
+               both in fp64
+  quant        dequantised weights within scale/2 of the originals; fp64 matmul of the definition
+"""

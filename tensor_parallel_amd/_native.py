@@ -1,0 +1,308 @@
+"""ctypes binding of `libtpamd.so` (include/tpamd.h).
+
+The library is loaded when this module is imported. If it cannot be loaded, importing still succeeds (so
+that rule tables and shape arithmetic can be used on a machine without the build), but every compute
+entry point raises `NativeLibraryError`: there is no other implementation to fall back to.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from pathlib import Path
+from typing import Optional, Sequence
+
+import torch  # imported first on purpose: the library binds to the HIP runtime torch has loaded
+
+LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libtpamd.so"
+
+EXPORTS = (
+    "tpamd_abi_version",
+    "tpamd_last_error",
+    "tpamd_copy_plan_create",
+    "tpamd_copy_plan_run",
+    "tpamd_copy_plan_bytes",
+    "tpamd_copy_plan_destroy",
+    "tpamd_scale",
+    "tpamd_reduce_partials",
+    "tpamd_linear",
+    "tpamd_swiglu_up",
+    "tpamd_linear_w8",
+)
+
+ABI_VERSION = 1
+
+BF16, F16, F32 = 0, 1, 2
+ACCUM_STEPWISE, ACCUM_F32 = 0, 1
+ACT_NONE, ACT_GELU = 0, 1
+
+_DTYPES = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}
+
+
+class NativeLibraryError(RuntimeError):
+    pass
+
+
+class CopyJob(ctypes.Structure):
+    _fields_ = [
+        ("src", ctypes.c_void_p),
+        ("dst", ctypes.c_void_p),
+        ("rows", ctypes.c_uint64),
+        ("row_bytes", ctypes.c_uint64),
+        ("src_pitch", ctypes.c_uint64),
+        ("dst_pitch", ctypes.c_uint64),
+    ]
+
+
+_lib: Optional[ctypes.CDLL] = None
+_load_error: Optional[str] = None
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    c = ctypes
+    i64, u64, vp, ci = c.c_int64, c.c_uint64, c.c_void_p, c.c_int
+    lib.tpamd_abi_version.restype = ci
+    lib.tpamd_abi_version.argtypes = []
+    lib.tpamd_last_error.restype = c.c_char_p
+    lib.tpamd_last_error.argtypes = []
+    lib.tpamd_copy_plan_create.restype = ci
+    lib.tpamd_copy_plan_create.argtypes = [c.POINTER(CopyJob), c.c_size_t, c.POINTER(vp)]
+    lib.tpamd_copy_plan_run.restype = ci
+    lib.tpamd_copy_plan_run.argtypes = [vp, vp]
+    lib.tpamd_copy_plan_bytes.restype = u64
+    lib.tpamd_copy_plan_bytes.argtypes = [vp]
+    lib.tpamd_copy_plan_destroy.restype = ci
+    lib.tpamd_copy_plan_destroy.argtypes = [vp]
+    lib.tpamd_scale.restype = ci
+    lib.tpamd_scale.argtypes = [vp, vp, u64, ci, ci, ci, vp]
+    lib.tpamd_reduce_partials.restype = ci
+    lib.tpamd_reduce_partials.argtypes = [c.POINTER(vp), ci, vp, u64, ci, ci, vp]
+    lib.tpamd_linear.restype = ci
+    lib.tpamd_linear.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
+    lib.tpamd_swiglu_up.restype = ci
+    lib.tpamd_swiglu_up.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+    lib.tpamd_linear_w8.restype = ci
+    lib.tpamd_linear_w8.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, i64, i64, i64, i64, i64, i64, i64, ci, ci, vp]
+
+
+def _load() -> None:
+    global _lib, _load_error
+    path = Path(os.environ.get("TPAMD_LIB", str(LIB_PATH)))
+    if not path.exists():
+        _load_error = f"{path} does not exist; build it with `python -m tensor_parallel_amd.build`"
+        return
+    try:
+        lib = ctypes.CDLL(str(path))
+        for name in EXPORTS:
+            getattr(lib, name)
+        _declare(lib)
+        got = lib.tpamd_abi_version()
+        if got != ABI_VERSION:
+            raise OSError(f"ABI version {got}, expected {ABI_VERSION}")
+        _lib = lib
+    except (OSError, AttributeError) as e:  # pragma: no cover - depends on the machine
+        _load_error = f"cannot load {path}: {e}"
+
+
+_load()
+
+
+def available() -> bool:
+    return _lib is not None
+
+
+def load_error() -> Optional[str]:
+    return _load_error
+
+
+def lib() -> ctypes.CDLL:
+    if _lib is None:
+        raise NativeLibraryError(f"the HIP library of tensor_parallel_amd is not available: {_load_error}")
+    return _lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().tpamd_last_error().decode("utf-8", "replace")
+        if rc == -1:
+            raise ValueError(f"{what}: {msg}")
+        raise RuntimeError(f"{what} failed (status {rc}): {msg}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError(f"tensor_parallel_amd kernels support bfloat16, float16 and float32, got {dtype}") from None
+
+
+def require_device(t: torch.Tensor, what: str) -> None:
+    if t.device.type != "cuda":
+        raise NativeLibraryError(
+            f"{what}: expected a tensor on a HIP device, got {t.device}. tensor_parallel_amd computes on the GPU only."
+        )
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class CopyPlan:
+    """A device-resident table of 2-D byte-region copies, run as one kernel launch."""
+
+    def __init__(self, jobs: Sequence[tuple], device: torch.device):
+        # jobs: (src_ptr, dst_ptr, rows, row_bytes, src_pitch, dst_pitch)
+        self._handle = ctypes.c_void_p()
+        self.device = device
+        arr = (CopyJob * max(len(jobs), 1))()
+        for i, j in enumerate(jobs):
+            arr[i] = CopyJob(*j)
+        with torch.cuda.device(device):
+            _check(lib().tpamd_copy_plan_create(arr, len(jobs), ctypes.byref(self._handle)), "tpamd_copy_plan_create")
+        self.n_jobs = len(jobs)
+
+    @property
+    def nbytes(self) -> int:
+        return int(lib().tpamd_copy_plan_bytes(self._handle))
+
+    def run(self, stream_ptr: Optional[int] = None) -> None:
+        with torch.cuda.device(self.device):
+            if stream_ptr is None:
+                stream_ptr = current_stream_ptr(self.device)
+            _check(lib().tpamd_copy_plan_run(self._handle, ctypes.c_void_p(stream_ptr)), "tpamd_copy_plan_run")
+
+    def close(self) -> None:
+        if self._handle:
+            h, self._handle = self._handle, ctypes.c_void_p()
+            if _lib is not None:
+                _lib.tpamd_copy_plan_destroy(h)
+
+    def __del__(self):  # noqa: D105
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def scale(inp: torch.Tensor, world_size: int, multiply: bool = False) -> torch.Tensor:
+    require_device(inp, "scale")
+    src = inp.contiguous()
+    out = torch.empty_like(src)
+    with torch.cuda.device(src.device):
+        _check(
+            lib().tpamd_scale(src.data_ptr(), out.data_ptr(), src.numel(), dtype_code(src.dtype), world_size,
+                              1 if multiply else 0, ctypes.c_void_p(current_stream_ptr(src.device))),
+            "tpamd_scale",
+        )
+    return out
+
+
+def reduce_partials(parts: Sequence[torch.Tensor], accum: int = ACCUM_STEPWISE, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if len(parts) == 0:
+        raise ValueError("reduce_partials: no partials")
+    first = parts[0]
+    require_device(first, "reduce_partials")
+    keep = []
+    for p in parts:
+        if p.shape != first.shape or p.dtype != first.dtype or p.device != first.device:
+            raise ValueError("reduce_partials: partials must agree in shape, dtype and device")
+        keep.append(p.contiguous())
+    if out is None:
+        out = torch.empty_like(keep[0])
+    ptrs = (ctypes.c_void_p * len(keep))(*[p.data_ptr() for p in keep])
+    with torch.cuda.device(first.device):
+        _check(
+            lib().tpamd_reduce_partials(ptrs, len(keep), out.data_ptr(), first.numel(), dtype_code(first.dtype), accum,
+                                        ctypes.c_void_p(current_stream_ptr(first.device))),
+            "tpamd_reduce_partials",
+        )
+    return out
+
+
+def _as_2d(x: torch.Tensor) -> torch.Tensor:
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+        x2 = x2.contiguous()
+    return x2
+
+
+def _ld(t: torch.Tensor) -> int:
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, act: int = ACT_NONE) -> torch.Tensor:
+    """y = act(x @ w.T + bias) with w of shape [N, K]; leading dimensions of x are kept."""
+    require_device(x, "linear")
+    require_device(w, "linear")
+    if x.dtype != w.dtype:
+        raise TypeError(f"linear: x is {x.dtype} but w is {w.dtype}")
+    if x.shape[-1] != w.shape[1]:
+        raise ValueError(f"linear: x has {x.shape[-1]} input features, w expects {w.shape[1]}")
+    x2, w2 = _as_2d(x), _as_2d(w)
+    M, K = x2.shape
+    N = w2.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    b = None
+    if bias is not None:
+        b = bias.contiguous()
+        if b.shape != (N,) or b.dtype != x.dtype:
+            raise ValueError("linear: bias must have shape [N] and the dtype of x")
+    with torch.cuda.device(x.device):
+        _check(
+            lib().tpamd_linear(x2.data_ptr(), w2.data_ptr(), b.data_ptr() if b is not None else None, y.data_ptr(),
+                               M, N, K, _ld(x2), _ld(w2), N, dtype_code(x.dtype), act,
+                               ctypes.c_void_p(current_stream_ptr(x.device))),
+            "tpamd_linear",
+        )
+    return y.view(*x.shape[:-1], N)
+
+
+def swiglu_up(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor) -> torch.Tensor:
+    """h = silu(x @ wg.T) * (x @ wu.T)."""
+    require_device(x, "swiglu_up")
+    if not (x.dtype == wg.dtype == wu.dtype):
+        raise TypeError("swiglu_up: x, wg, wu must share one dtype")
+    if wg.shape != wu.shape or x.shape[-1] != wg.shape[1]:
+        raise ValueError("swiglu_up: shape mismatch")
+    x2, g2, u2 = _as_2d(x), _as_2d(wg), _as_2d(wu)
+    if _ld(g2) != _ld(u2):
+        u2 = u2.contiguous()
+        g2 = g2.contiguous()
+    M, K = x2.shape
+    N = g2.shape[0]
+    h = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(
+            lib().tpamd_swiglu_up(x2.data_ptr(), g2.data_ptr(), u2.data_ptr(), h.data_ptr(), M, N, K, _ld(x2), _ld(g2), N,
+                                  dtype_code(x.dtype), ctypes.c_void_p(current_stream_ptr(x.device))),
+            "tpamd_swiglu_up",
+        )
+    return h.view(*x.shape[:-1], N)
+
+
+def linear_w8(x: torch.Tensor, wq: torch.Tensor, scale_: torch.Tensor, outlier_idx: Optional[torch.Tensor],
+              w_out: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None, act: int = ACT_NONE) -> torch.Tensor:
+    """Weight-only int8 Linear with outlier columns kept in the activation dtype."""
+    require_device(x, "linear_w8")
+    if wq.dtype != torch.int8 or scale_.dtype != torch.float32:
+        raise TypeError("linear_w8: wq must be int8 and scale float32")
+    x2 = _as_2d(x)
+    wq = wq.contiguous()
+    M, K = x2.shape
+    N = wq.shape[0]
+    n_out = 0 if outlier_idx is None else int(outlier_idx.numel())
+    if n_out:
+        if outlier_idx.dtype != torch.int32 or w_out is None or w_out.shape != (N, n_out) or w_out.dtype != x.dtype:
+            raise ValueError("linear_w8: outlier_idx must be int32 [n_out] and w_out [N, n_out] in the dtype of x")
+        w_out = w_out.contiguous()
+        outlier_idx = outlier_idx.contiguous()
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    b = bias.contiguous() if bias is not None else None
+    with torch.cuda.device(x.device):
+        _check(
+            lib().tpamd_linear_w8(x2.data_ptr(), wq.data_ptr(), scale_.contiguous().data_ptr(),
+                                  outlier_idx.data_ptr() if n_out else None, w_out.data_ptr() if n_out else None, n_out,
+                                  b.data_ptr() if b is not None else None, y.data_ptr(), M, N, K, _ld(x2), K, max(n_out, 1), N,
+                                  dtype_code(x.dtype), act, ctypes.c_void_p(current_stream_ptr(x.device))),
+            "tpamd_linear_w8",
+        )
+    return y.view(*x.shape[:-1], N)

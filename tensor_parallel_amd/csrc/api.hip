@@ -1,0 +1,112 @@
+// C ABI entry points for the shard Linears, plus the library's error plumbing.
+#include "common.h"
+
+#include <string.h>
+
+namespace tpamd {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias, void *y, int64_t M, int64_t N,
+                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu, hipStream_t s);
+int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *scale,
+                    const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N, int64_t K,
+                    int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
+                    hipStream_t s);
+
+namespace {
+
+// Largest M served by the weight-streaming kernel; above it the tiled MFMA kernel takes over.
+constexpr int64_t SKINNY_MAX_M = 32;
+constexpr int64_t SKINNY_W8_SLAB = 64;
+
+int check_common(const char *who, const void *x, const void *w, const void *y, int64_t M, int64_t N, int64_t K,
+                 int64_t ldx, int64_t ldw, int64_t ldy, int dtype) {
+    TPAMD_REQUIRE(M >= 0 && N >= 0 && K >= 0, "%s: negative dimension (M=%lld N=%lld K=%lld)", who, (long long)M,
+                  (long long)N, (long long)K);
+    TPAMD_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "%s: dimension over 2^31", who);
+    TPAMD_REQUIRE(dtype == TPAMD_BF16 || dtype == TPAMD_F16 || dtype == TPAMD_F32, "%s: unknown dtype %d", who, dtype);
+    if (M == 0 || N == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(x && w && y, "%s: null pointer", who);
+    TPAMD_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "%s: leading dimension smaller than the row (ldx=%lld ldw=%lld ldy=%lld)",
+                  who, (long long)ldx, (long long)ldw, (long long)ldy);
+    if (dtype != TPAMD_F32) {
+        TPAMD_REQUIRE(aligned(x, 16) && aligned(w, 16) && aligned(y, 8), "%s: x/w must be 16-byte and y 8-byte aligned", who);
+        TPAMD_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "%s: K, ldx, ldw must be multiples of 8 (K=%lld ldx=%lld ldw=%lld)",
+                      who, (long long)K, (long long)ldx, (long long)ldw);
+        TPAMD_REQUIRE(N % 4 == 0 && ldy % 4 == 0, "%s: N and ldy must be multiples of 4 (N=%lld ldy=%lld)", who,
+                      (long long)N, (long long)ldy);
+    }
+    return TPAMD_OK;
+}
+
+}  // namespace
+}  // namespace tpamd
+
+using namespace tpamd;
+
+extern "C" int tpamd_abi_version(void) { return TPAMD_ABI_VERSION; }
+extern "C" const char *tpamd_last_error(void) { return g_err; }
+
+extern "C" int tpamd_linear(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
+                            int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, void *stream) {
+    int rc = check_common("tpamd_linear", x_dev, w_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype);
+    if (rc != TPAMD_OK) return rc;
+    TPAMD_REQUIRE(act == TPAMD_ACT_NONE || act == TPAMD_ACT_GELU, "tpamd_linear: unknown activation %d", act);
+    if (M == 0 || N == 0) return TPAMD_OK;
+    if (bias_dev && dtype != TPAMD_F32) TPAMD_REQUIRE(aligned(bias_dev, 8), "tpamd_linear: bias must be 8-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype != TPAMD_F32 && M <= SKINNY_MAX_M)
+        return skinny_dispatch(x_dev, w_dev, nullptr, bias_dev, nullptr, nullptr, nullptr, 0, y_dev, M, N, K, ldx, ldw, ldy, 0,
+                               dtype, act, false, false, s);
+    return gemm_dispatch(x_dev, w_dev, nullptr, bias_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, false, s);
+}
+
+extern "C" int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void *wu_dev, void *h_dev, int64_t M, int64_t N,
+                               int64_t K, int64_t ldx, int64_t ldw, int64_t ldh, int dtype, void *stream) {
+    int rc = check_common("tpamd_swiglu_up", x_dev, wg_dev, h_dev, M, N, K, ldx, ldw, ldh, dtype);
+    if (rc != TPAMD_OK) return rc;
+    TPAMD_REQUIRE(dtype != TPAMD_F32, "tpamd_swiglu_up: fp32 is not supported, use tpamd_linear twice");
+    if (M == 0 || N == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(wu_dev && aligned(wu_dev, 16), "tpamd_swiglu_up: wu must be non-null and 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (M <= SKINNY_MAX_M)
+        return skinny_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw, ldh, 0,
+                               dtype, TPAMD_ACT_NONE, true, false, s);
+    return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true, s);
+}
+
+extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,
+                               const void *w_out_dev, int64_t n_out, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
+                               int64_t K, int64_t ldx, int64_t ldw, int64_t ld_wout, int64_t ldy, int dtype, int act,
+                               void *stream) {
+    const char *who = "tpamd_linear_w8";
+    TPAMD_REQUIRE(dtype == TPAMD_BF16 || dtype == TPAMD_F16, "%s: dtype must be BF16 or F16", who);
+    TPAMD_REQUIRE(M >= 0 && N >= 0 && K >= 0 && n_out >= 0, "%s: negative dimension", who);
+    TPAMD_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "%s: dimension over 2^31", who);
+    TPAMD_REQUIRE(act == TPAMD_ACT_NONE || act == TPAMD_ACT_GELU, "%s: unknown activation %d", who, act);
+    if (M == 0 || N == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(x_dev && wq_dev && scale_dev && y_dev, "%s: null pointer", who);
+    TPAMD_REQUIRE(n_out == 0 || (outlier_idx_dev && w_out_dev && ld_wout >= n_out), "%s: outlier arguments inconsistent", who);
+    TPAMD_REQUIRE(n_out <= K, "%s: more outlier columns (%lld) than K", who, (long long)n_out);
+    TPAMD_REQUIRE(aligned(x_dev, 16) && aligned(wq_dev, 16), "%s: x and wq must be 16-byte aligned", who);
+    TPAMD_REQUIRE(K % 16 == 0 && ldw % 16 == 0 && ldx % 8 == 0, "%s: K, ldw multiples of 16 and ldx of 8 required", who);
+    TPAMD_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "%s: leading dimension smaller than the row", who);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int esz = 2;
+    for (int64_t m0 = 0; m0 < M; m0 += SKINNY_W8_SLAB) {  // weights are re-streamed once per slab of 64 rows
+        const int64_t mm = M - m0 < SKINNY_W8_SLAB ? M - m0 : SKINNY_W8_SLAB;
+        int rc = skinny_dispatch(static_cast<const char *>(x_dev) + m0 * ldx * esz, wq_dev, nullptr, bias_dev, scale_dev,
+                                 outlier_idx_dev, w_out_dev, n_out, static_cast<char *>(y_dev) + m0 * ldy * esz, mm, N, K, ldx,
+                                 ldw, ldy, ld_wout, dtype, act, false, true, s);
+        if (rc != TPAMD_OK) return rc;
+    }
+    return TPAMD_OK;
+}

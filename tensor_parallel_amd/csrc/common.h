@@ -1,0 +1,84 @@
+// Shared host/device helpers for the gfx950 kernels behind include/tpamd.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/tpamd.h"
+
+namespace tpamd {
+
+// ---- error plumbing -----------------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+
+#define TPAMD_REQUIRE(cond, ...)                 \
+    do {                                         \
+        if (!(cond)) {                           \
+            ::tpamd::set_error(__VA_ARGS__);     \
+            return TPAMD_ERR_INVALID;            \
+        }                                        \
+    } while (0)
+
+#define TPAMD_HIP(call)                                                                          \
+    do {                                                                                         \
+        hipError_t e_ = (call);                                                                  \
+        if (e_ != hipSuccess) {                                                                  \
+            ::tpamd::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__,  \
+                               __LINE__);                                                        \
+            return TPAMD_ERR_HIP;                                                                \
+        }                                                                                        \
+    } while (0)
+
+static inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- streaming (non-temporal) 16-byte accesses: data that is touched once should not displace cache lines
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 nt_load_u4(const void *p) {
+    const v4u v = __builtin_nontemporal_load(static_cast<const v4u *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void nt_store_u4(void *p, uint4 u) {
+    const v4u v = {u.x, u.y, u.z, u.w};
+    __builtin_nontemporal_store(v, static_cast<v4u *>(p));
+}
+
+// ---- device-side scalar conversions ---------------------------------------------------------------
+// bf16 is handled as raw uint16_t bits so that rounding is spelled out (round to nearest even, NaN
+// kept quiet), identical to what torch does when it stores an fp32 result into a bf16 tensor.
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(static_cast<uint32_t>(h) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);  // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+__device__ __forceinline__ float f16_to_f32(uint16_t h) {
+    _Float16 v = __builtin_bit_cast(_Float16, h);
+    return static_cast<float>(v);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+    _Float16 v = static_cast<_Float16>(f);  // v_cvt_f16_f32: round to nearest even
+    return __builtin_bit_cast(uint16_t, v);
+}
+
+template <int DT>
+__device__ __forceinline__ float half_to_f32(uint16_t h) {
+    if constexpr (DT == TPAMD_BF16) return bf16_to_f32(h);
+    else return f16_to_f32(h);
+}
+template <int DT>
+__device__ __forceinline__ uint16_t f32_to_half(float f) {
+    if constexpr (DT == TPAMD_BF16) return f32_to_bf16(f);
+    else return f32_to_f16(f);
+}
+
+__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+
+}  // namespace tpamd

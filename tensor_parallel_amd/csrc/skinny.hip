@@ -1,0 +1,321 @@
+// Rank-shard Linear for decode-sized M (M <= 64): weight streaming, HBM-bound.
+//
+// A block owns 16 output columns (16 rows of w; for the SiLU-gated pair 16 gate rows + 16 up rows) and
+// splits K over its wavefronts in chunks of 64 bytes per lane. Each lane loads 64 contiguous bytes of
+// one w row (4 lanes cover 256 contiguous bytes of that row) straight from global memory into MFMA
+// operands: v_mfma_f32_16x16x32 does both the multiply and the reduction over K, so no cross-lane
+// shuffles are needed. The K positions an MFMA sees are a permutation of the real ones; x is loaded
+// with the same permutation. Partial sums of the wavefronts meet in LDS; the epilogue applies scale,
+// outliers, bias, activation and stores 16 consecutive columns per row.
+//
+// The weight is either the activation dtype (bf16/f16) or int8 (weight-only quantisation: converted to
+// the activation dtype in registers, exact for |q| <= 128).
+#include "common.h"
+
+#include <type_traits>
+
+namespace tpamd {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+enum { SK_LINEAR = 0, SK_SWIGLU = 1 };
+constexpr int SK_WAVES = 8;
+constexpr int SK_THREADS = SK_WAVES * 64;
+
+struct SkinnyParams {
+    const char *x;
+    const char *w;
+    const char *w2;
+    const char *bias;
+    const float *scale;        // int8 path: per output row
+    const int *outlier_idx;    // int8 path
+    const char *w_out;         // int8 path: [N, n_out] in activation dtype
+    char *y;
+    int M, N, K;
+    int n_out;
+    int64_t ldx, ldw, ldy, ld_wout;
+    int act;
+};
+
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
+    if constexpr (DT == TPAMD_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// Four int8 (one dword) -> four values of the activation dtype, packed as lo = elements 0,1 and
+// hi = elements 2,3. Exact: |q| <= 128 fits both f16 and bf16 significands.
+template <int DT>
+__device__ __forceinline__ void cvt_i8x4(uint32_t q, uint32_t &lo, uint32_t &hi) {
+    const uint32_t u = q ^ 0x80808080u;  // biased to 0..255
+    if constexpr (DT == TPAMD_F16) {
+        // f16 0x6400 | u == 1024 + u; subtracting 1152 gives q
+        const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+        const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+        const f16x2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+        lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, p0) - bias);
+        hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, p1) - bias);
+    } else {
+        // f32 0x4B000000 | u == 2^23 + u; subtracting 2^23 + 128 gives q; its high half is the bf16
+        const float f0 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050400u)) - 8388736.0f;
+        const float f1 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050401u)) - 8388736.0f;
+        const float f2 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050402u)) - 8388736.0f;
+        const float f3 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050403u)) - 8388736.0f;
+        lo = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+        hi = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+    }
+}
+
+// W8 = weight is int8. MT = number of 16-row tiles of x (M <= 16*MT). MODE = SK_LINEAR / SK_SWIGLU.
+template <int DT, bool W8, int MT, int MODE>
+__global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
+    constexpr int NMAT = MODE == SK_SWIGLU ? 2 : 1;
+    constexpr int LANE_K = W8 ? 64 : 32;      // K elements per lane per chunk (64 bytes of w)
+    constexpr int CHUNK_K = LANE_K * 4;       // K elements per chunk
+    constexpr int WV = 4;                     // 16-byte loads of w per lane per chunk
+    constexpr int XV = LANE_K / 8;            // 16-byte loads of x per lane per chunk per m-tile
+
+    __shared__ float red[SK_WAVES][NMAT][MT][4][64];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+
+    int wrow = n0 + lr;
+    wrow = wrow < p.N ? wrow : p.N - 1;
+    const int wbytes = W8 ? 1 : 2;
+    const char *wp[NMAT];
+    wp[0] = p.w + (static_cast<int64_t>(wrow) * p.ldw + lg * LANE_K) * wbytes;
+    if constexpr (NMAT == 2) wp[1] = p.w2 + (static_cast<int64_t>(wrow) * p.ldw + lg * LANE_K) * wbytes;
+    const char *xp[MT];
+    bool xok[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + lr;
+        xok[t] = m < p.M;
+        xp[t] = p.x + (static_cast<int64_t>(xok[t] ? m : 0) * p.ldx + lg * LANE_K) * 2;
+    }
+
+    f32x4 acc[NMAT][MT];
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[a][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nchunks = (p.K + CHUNK_K - 1) / CHUNK_K;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+    // Register double buffers for the weights (and for x when it is small enough). Buffer indices are
+    // compile-time constants so that the arrays stay in registers.
+    constexpr bool XPRE = MT * XV <= 8;
+    uint4 wv[2][NMAT][WV];
+    uint4 xv[XPRE ? 2 : 1][MT][XV];
+    auto load_w = [&](auto bufc, int c) {
+        constexpr int buf = decltype(bufc)::value;
+        const int kbase = c * CHUNK_K + lg * LANE_K;  // first K element of this lane
+        const int64_t off = static_cast<int64_t>(c) * CHUNK_K * wbytes;
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+            for (int v = 0; v < WV; ++v) {
+                const int k = kbase + v * (LANE_K / WV);
+                wv[buf][a][v] = k < p.K ? nt_load_u4(reinterpret_cast<const uint4 *>(wp[a] + off) + v) : zero4;
+            }
+    };
+    auto load_x = [&](auto bufc, int c) {
+        constexpr int buf = decltype(bufc)::value;
+        const int kbase = c * CHUNK_K + lg * LANE_K;
+        const int64_t xoff = static_cast<int64_t>(c) * CHUNK_K * 2;
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < XV; ++v)
+                xv[buf][t][v] = (xok[t] && kbase + v * 8 < p.K) ? *(reinterpret_cast<const uint4 *>(xp[t] + xoff) + v) : zero4;
+    };
+    auto compute = [&](auto bufc) {
+        constexpr int buf = decltype(bufc)::value;
+        constexpr int xb = XPRE ? buf : 0;
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a) {
+            if constexpr (W8) {
+#pragma unroll
+                for (int v = 0; v < WV; ++v) {  // 16 int8 -> two operands of 8
+                    const uint4 q = wv[buf][a][v];
+                    uint4 w0, w1;
+                    cvt_i8x4<DT>(q.x, w0.x, w0.y);
+                    cvt_i8x4<DT>(q.y, w0.z, w0.w);
+                    cvt_i8x4<DT>(q.z, w1.x, w1.y);
+                    cvt_i8x4<DT>(q.w, w1.z, w1.w);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        acc[a][t] = mfma16<DT>(w0, xv[xb][t][2 * v], acc[a][t]);
+                        acc[a][t] = mfma16<DT>(w1, xv[xb][t][2 * v + 1], acc[a][t]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < WV; ++v)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) acc[a][t] = mfma16<DT>(wv[buf][a][v], xv[xb][t][v], acc[a][t]);
+            }
+        }
+    };
+    static_assert(W8 ? (XV == 2 * WV) : (XV == WV), "operand chunking");
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+
+    // This wavefront's chunks are wave, wave + SK_WAVES, ... The next chunk's loads are issued before the
+    // current one is multiplied. Loads return in order, so whatever the multiply waits for is issued
+    // ahead of the prefetch.
+    int c = wave;
+    if (c < nchunks) {
+        load_w(B0{}, c);
+        if constexpr (XPRE) load_x(B0{}, c);
+    }
+    while (c < nchunks) {
+        int cn = c + SK_WAVES;
+        if constexpr (!XPRE) load_x(B0{}, c);
+        if (cn < nchunks) {
+            load_w(B1{}, cn);
+            if constexpr (XPRE) load_x(B1{}, cn);
+        }
+        compute(B0{});
+        c = cn;
+        if (c >= nchunks) break;
+        cn = c + SK_WAVES;
+        if constexpr (!XPRE) load_x(B0{}, c);
+        if (cn < nchunks) {
+            load_w(B0{}, cn);
+            if constexpr (XPRE) load_x(B0{}, cn);
+        }
+        compute(B1{});
+        c = cn;
+    }
+
+    // ---- int8 path: the outlier columns, spread over the wavefronts in groups of 32 ----------------
+    f32x4 acc_o[MT];
+    if constexpr (W8) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc_o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const uint16_t *xo = reinterpret_cast<const uint16_t *>(p.x);
+        const uint16_t *wo = reinterpret_cast<const uint16_t *>(p.w_out);
+        for (int s = wave; s * 32 < p.n_out; s += SK_WAVES) {
+            uint32_t wq[4] = {0, 0, 0, 0};
+            uint32_t xq[MT][4];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) xq[t][0] = xq[t][1] = xq[t][2] = xq[t][3] = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int o = s * 32 + lg * 8 + j;
+                if (o < p.n_out) {
+                    const int col = p.outlier_idx[o];
+                    const uint32_t wval = wo[static_cast<int64_t>(wrow) * p.ld_wout + o];
+                    wq[j >> 1] |= wval << ((j & 1) * 16);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                        if (xok[t]) {
+                            const uint32_t xval = xo[static_cast<int64_t>(t * 16 + lr) * p.ldx + col];
+                            xq[t][j >> 1] |= xval << ((j & 1) * 16);
+                        }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc_o[t] = mfma16<DT>(make_uint4(wq[0], wq[1], wq[2], wq[3]), make_uint4(xq[t][0], xq[t][1], xq[t][2], xq[t][3]), acc_o[t]);
+        }
+    }
+
+    // ---- cross-wave reduction. D[n_local][m_local]: lane -> m_local = lr, register i -> n_local = 4*lg + i
+    if constexpr (W8) {
+        // fold the per-row scale in before the partial sums meet, then add the outlier product
+        float sc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int n = n0 + lg * 4 + i;
+            n = n < p.N ? n : p.N - 1;
+            sc[i] = p.scale[n];
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[0][t][i] = acc[0][t][i] * sc[i] + acc_o[t][i];
+    }
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][a][t][i][lane] = acc[a][t][i];
+    __syncthreads();
+
+    // thread e -> output (m = e / 16, n_local = e % 16): 16 consecutive threads store one 32-byte row piece
+    for (int e = tid; e < MT * 256; e += SK_THREADS) {
+        const int m = e >> 4, nl = e & 15;
+        const int n = n0 + nl;
+        if (m >= p.M || n >= p.N) continue;
+        const int t = m >> 4, src_lane = (nl >> 2) * 16 + (m & 15), i = nl & 3;
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) {
+            s0 += red[w][0][t][i][src_lane];
+            if constexpr (NMAT == 2) s1 += red[w][1][t][i][src_lane];
+        }
+        uint16_t out;
+        if constexpr (MODE == SK_SWIGLU) {
+            const float g = half_to_f32<DT>(f32_to_half<DT>(s0));
+            const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
+            const float s = half_to_f32<DT>(f32_to_half<DT>(silu_f32(g)));
+            out = f32_to_half<DT>(s * u);
+        } else {
+            float v = s0;
+            if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
+            if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+            out = f32_to_half<DT>(v);
+        }
+        reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
+    }
+}
+
+template <int DT, bool W8, int MODE>
+int launch_skinny(const SkinnyParams &p, hipStream_t s) {
+    const unsigned grid = static_cast<unsigned>((p.N + 15) / 16);
+    if (p.M <= 16) hipLaunchKernelGGL((skinny_kernel<DT, W8, 1, MODE>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    else if (p.M <= 32) hipLaunchKernelGGL((skinny_kernel<DT, W8, 2, MODE>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((skinny_kernel<DT, W8, 4, MODE>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+}  // namespace
+
+// M <= 64. dtype is BF16 or F16. `w8` selects the int8 weight path (linear only).
+int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *scale,
+                    const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N, int64_t K,
+                    int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
+                    hipStream_t s) {
+    SkinnyParams p{};
+    p.x = static_cast<const char *>(x);
+    p.w = static_cast<const char *>(w);
+    p.w2 = static_cast<const char *>(w2);
+    p.bias = static_cast<const char *>(bias);
+    p.scale = static_cast<const float *>(scale);
+    p.outlier_idx = static_cast<const int *>(outlier_idx);
+    p.w_out = static_cast<const char *>(w_out);
+    p.y = static_cast<char *>(y);
+    p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
+    p.n_out = static_cast<int>(n_out);
+    p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ld_wout = ld_wout;
+    p.act = act;
+    const bool bf = dtype == TPAMD_BF16;
+    if (w8) return bf ? launch_skinny<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_skinny<TPAMD_F16, true, SK_LINEAR>(p, s);
+    if (swiglu) return bf ? launch_skinny<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_skinny<TPAMD_F16, false, SK_SWIGLU>(p, s);
+    return bf ? launch_skinny<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_skinny<TPAMD_F16, false, SK_LINEAR>(p, s);
+}
+
+}  // namespace tpamd

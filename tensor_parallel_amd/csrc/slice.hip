@@ -1,0 +1,270 @@
+// Slicing engine: a batched 2-D byte-region mover. One launch moves every (tensor, rank) shard of a
+// state dict. The host cuts each job into tiles of at most TILE_UNITS vector units; a persistent grid
+// walks the tile table. HBM-bound: every byte is read once and written once.
+#include "common.h"
+
+#include <new>
+#include <vector>
+
+namespace tpamd {
+
+namespace {
+
+constexpr uint32_t TILE_UNITS = 4096;  // vector units per tile (64 KiB when units are 16 bytes)
+constexpr int COPY_THREADS = 256;
+
+struct alignas(16) Tile {
+    const char *src;
+    char *dst;
+    uint64_t src_pitch;
+    uint64_t dst_pitch;
+    uint32_t rows;
+    uint32_t units_per_row;  // row length in units of `vec` bytes
+    uint32_t magic;          // ceil(2^32 / units_per_row), 0 when units_per_row == 1
+    uint32_t vec;            // 16, 8, 4, 2 or 1
+};
+static_assert(sizeof(Tile) == 48, "Tile layout");
+
+template <typename V>
+__device__ __forceinline__ V ld_stream(const V *p) { return __builtin_nontemporal_load(p); }
+template <typename V>
+__device__ __forceinline__ void st_stream(V *p, V v) { __builtin_nontemporal_store(v, p); }
+
+// Moves one tile with units of type V. idx -> (row, col) uses a multiply-high by a host-made
+// reciprocal: exact because idx < 2^12 and units_per_row <= 2^12.
+template <typename V>
+__device__ __forceinline__ void move_tile(const Tile &t, int tid) {
+    const uint32_t upr = t.units_per_row;
+    const uint32_t total = t.rows * upr;
+    if (t.rows == 1) {
+        const V *s = reinterpret_cast<const V *>(t.src);
+        V *d = reinterpret_cast<V *>(t.dst);
+        uint32_t i = tid;
+        for (; i + 3 * COPY_THREADS < total; i += 4 * COPY_THREADS) {
+            V a = ld_stream(s + i), b = ld_stream(s + i + COPY_THREADS), c = ld_stream(s + i + 2 * COPY_THREADS),
+              e = ld_stream(s + i + 3 * COPY_THREADS);
+            st_stream(d + i, a);
+            st_stream(d + i + COPY_THREADS, b);
+            st_stream(d + i + 2 * COPY_THREADS, c);
+            st_stream(d + i + 3 * COPY_THREADS, e);
+        }
+        for (; i < total; i += COPY_THREADS) st_stream(d + i, ld_stream(s + i));
+        return;
+    }
+    const uint32_t magic = t.magic;
+    auto src_of = [&](uint32_t idx) -> const V * {
+        uint32_t row = magic ? __umulhi(idx, magic) : idx;
+        uint32_t col = idx - row * upr;
+        return reinterpret_cast<const V *>(t.src + static_cast<uint64_t>(row) * t.src_pitch) + col;
+    };
+    auto dst_of = [&](uint32_t idx) -> V * {
+        uint32_t row = magic ? __umulhi(idx, magic) : idx;
+        uint32_t col = idx - row * upr;
+        return reinterpret_cast<V *>(t.dst + static_cast<uint64_t>(row) * t.dst_pitch) + col;
+    };
+    uint32_t i = tid;
+    for (; i + 3 * COPY_THREADS < total; i += 4 * COPY_THREADS) {
+        V a = ld_stream(src_of(i)), b = ld_stream(src_of(i + COPY_THREADS)), c = ld_stream(src_of(i + 2 * COPY_THREADS)),
+          e = ld_stream(src_of(i + 3 * COPY_THREADS));
+        st_stream(dst_of(i), a);
+        st_stream(dst_of(i + COPY_THREADS), b);
+        st_stream(dst_of(i + 2 * COPY_THREADS), c);
+        st_stream(dst_of(i + 3 * COPY_THREADS), e);
+    }
+    for (; i < total; i += COPY_THREADS) st_stream(dst_of(i), ld_stream(src_of(i)));
+}
+
+__global__ __launch_bounds__(COPY_THREADS) void copy_tiles_kernel(const Tile *__restrict__ tiles, uint32_t n_tiles) {
+    const int tid = threadIdx.x;
+    for (uint32_t ti = blockIdx.x; ti < n_tiles; ti += gridDim.x) {
+        const Tile t = tiles[ti];  // block-uniform: scalar loads
+        switch (t.vec) {
+            case 16: move_tile<v4u>(t, tid); break;
+            case 8: move_tile<v2u>(t, tid); break;
+            case 4: move_tile<uint32_t>(t, tid); break;
+            case 2: move_tile<uint16_t>(t, tid); break;
+            default: move_tile<uint8_t>(t, tid); break;
+        }
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void scale_kernel(const void *__restrict__ in, void *__restrict__ out, uint64_t n,
+                                                    float w, int mul) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+    for (; i < n; i += stride) {
+        if constexpr (DT == TPAMD_F32) {
+            float v = static_cast<const float *>(in)[i];
+            static_cast<float *>(out)[i] = mul ? v * w : v / w;
+        } else {
+            float v = half_to_f32<DT>(static_cast<const uint16_t *>(in)[i]);
+            static_cast<uint16_t *>(out)[i] = f32_to_half<DT>(mul ? v * w : v / w);
+        }
+    }
+}
+
+uint32_t pick_vec(const tpamd_copy_job &j) {
+    uint64_t bits = reinterpret_cast<uintptr_t>(j.src_dev) | reinterpret_cast<uintptr_t>(j.dst_dev) | j.row_bytes;
+    if (j.rows > 1) bits |= j.src_pitch | j.dst_pitch;
+    for (uint32_t v = 16; v > 1; v >>= 1)
+        if ((bits & (v - 1)) == 0) return v;
+    return 1;
+}
+
+}  // namespace
+
+}  // namespace tpamd
+
+struct tpamd_copy_plan {
+    tpamd::Tile *tiles_dev = nullptr;
+    uint32_t n_tiles = 0;
+    uint64_t bytes = 0;
+    int device = -1;
+    int grid = 0;
+};
+
+using namespace tpamd;
+
+extern "C" int tpamd_copy_plan_create(const tpamd_copy_job *jobs, size_t n_jobs, tpamd_copy_plan **plan_out) {
+    TPAMD_REQUIRE(plan_out != nullptr, "tpamd_copy_plan_create: plan_out is NULL");
+    TPAMD_REQUIRE(jobs != nullptr || n_jobs == 0, "tpamd_copy_plan_create: jobs is NULL with n_jobs=%zu", n_jobs);
+    *plan_out = nullptr;
+    std::vector<Tile> tiles;
+    uint64_t bytes = 0;
+    try {
+        for (size_t ji = 0; ji < n_jobs; ++ji) {
+            const tpamd_copy_job &j = jobs[ji];
+            if (j.rows == 0 || j.row_bytes == 0) continue;
+            TPAMD_REQUIRE(j.src_dev != nullptr && j.dst_dev != nullptr, "copy job %zu: null pointer", ji);
+            TPAMD_REQUIRE(j.rows == 1 || (j.src_pitch >= j.row_bytes && j.dst_pitch >= j.row_bytes),
+                          "copy job %zu: pitch (%llu src, %llu dst) smaller than row_bytes %llu", ji,
+                          (unsigned long long)j.src_pitch, (unsigned long long)j.dst_pitch,
+                          (unsigned long long)j.row_bytes);
+            bytes += j.rows * j.row_bytes;
+            const uint32_t vec = pick_vec(j);
+            const uint64_t upr_full = j.row_bytes / vec;
+            const char *src = static_cast<const char *>(j.src_dev);
+            char *dst = static_cast<char *>(j.dst_dev);
+            const bool contiguous = (j.rows == 1) || (j.src_pitch == j.row_bytes && j.dst_pitch == j.row_bytes);
+            if (contiguous) {
+                const uint64_t units = j.rows * upr_full;
+                for (uint64_t u = 0; u < units; u += TILE_UNITS) {
+                    Tile t{};
+                    t.src = src + u * vec;
+                    t.dst = dst + u * vec;
+                    t.rows = 1;
+                    t.units_per_row = static_cast<uint32_t>(units - u < TILE_UNITS ? units - u : TILE_UNITS);
+                    t.vec = vec;
+                    tiles.push_back(t);
+                }
+            } else if (upr_full >= TILE_UNITS) {  // long rows: cut every row into column tiles
+                for (uint64_t r = 0; r < j.rows; ++r)
+                    for (uint64_t u = 0; u < upr_full; u += TILE_UNITS) {
+                        Tile t{};
+                        t.src = src + r * j.src_pitch + u * vec;
+                        t.dst = dst + r * j.dst_pitch + u * vec;
+                        t.rows = 1;
+                        t.units_per_row = static_cast<uint32_t>(upr_full - u < TILE_UNITS ? upr_full - u : TILE_UNITS);
+                        t.vec = vec;
+                        tiles.push_back(t);
+                    }
+            } else {  // short rows: several whole rows per tile
+                const uint32_t upr = static_cast<uint32_t>(upr_full);
+                const uint64_t rpt = TILE_UNITS / upr;  // >= 1
+                for (uint64_t r = 0; r < j.rows; r += rpt) {
+                    Tile t{};
+                    t.src = src + r * j.src_pitch;
+                    t.dst = dst + r * j.dst_pitch;
+                    t.src_pitch = j.src_pitch;
+                    t.dst_pitch = j.dst_pitch;
+                    t.rows = static_cast<uint32_t>(j.rows - r < rpt ? j.rows - r : rpt);
+                    t.units_per_row = upr;
+                    t.magic = upr == 1 ? 0u : static_cast<uint32_t>(((1ull << 32) + upr - 1) / upr);
+                    t.vec = vec;
+                    tiles.push_back(t);
+                }
+            }
+            TPAMD_REQUIRE(tiles.size() < 0xffffff00ull, "copy plan too large (%zu tiles)", tiles.size());
+        }
+    } catch (const std::bad_alloc &) {
+        set_error("tpamd_copy_plan_create: out of host memory building the tile table");
+        return TPAMD_ERR_NOMEM;
+    }
+
+    tpamd_copy_plan *plan = new (std::nothrow) tpamd_copy_plan();
+    if (!plan) {
+        set_error("tpamd_copy_plan_create: out of host memory");
+        return TPAMD_ERR_NOMEM;
+    }
+    plan->n_tiles = static_cast<uint32_t>(tiles.size());
+    plan->bytes = bytes;
+    hipError_t e = hipGetDevice(&plan->device);
+    hipDeviceProp_t prop;
+    if (e == hipSuccess) e = hipGetDeviceProperties(&prop, plan->device);
+    if (e == hipSuccess && plan->n_tiles) {
+        int per_cu = 8;
+        if (const char *s = getenv("TPAMD_COPY_BLOCKS_PER_CU")) {
+            int v = atoi(s);
+            if (v >= 1 && v <= 64) per_cu = v;
+        }
+        const uint64_t cap = static_cast<uint64_t>(prop.multiProcessorCount) * per_cu;
+        plan->grid = static_cast<int>(plan->n_tiles < cap ? plan->n_tiles : cap);
+        e = hipMalloc(reinterpret_cast<void **>(&plan->tiles_dev), tiles.size() * sizeof(Tile));
+        if (e == hipSuccess)
+            e = hipMemcpy(plan->tiles_dev, tiles.data(), tiles.size() * sizeof(Tile), hipMemcpyHostToDevice);
+    }
+    if (e != hipSuccess) {
+        set_error("tpamd_copy_plan_create: %s", hipGetErrorString(e));
+        if (plan->tiles_dev) (void)hipFree(plan->tiles_dev);
+        delete plan;
+        return TPAMD_ERR_HIP;
+    }
+    *plan_out = plan;
+    return TPAMD_OK;
+}
+
+extern "C" int tpamd_copy_plan_run(const tpamd_copy_plan *plan, void *stream) {
+    TPAMD_REQUIRE(plan != nullptr, "tpamd_copy_plan_run: plan is NULL");
+    if (plan->n_tiles == 0) return TPAMD_OK;
+    int dev = -1;
+    TPAMD_HIP(hipGetDevice(&dev));
+    TPAMD_REQUIRE(dev == plan->device, "tpamd_copy_plan_run: plan was made on device %d, current is %d", plan->device,
+                  dev);
+    hipLaunchKernelGGL(copy_tiles_kernel, dim3(plan->grid), dim3(COPY_THREADS), 0, static_cast<hipStream_t>(stream),
+                       plan->tiles_dev, plan->n_tiles);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+extern "C" uint64_t tpamd_copy_plan_bytes(const tpamd_copy_plan *plan) { return plan ? plan->bytes : 0; }
+
+extern "C" int tpamd_copy_plan_destroy(tpamd_copy_plan *plan) {
+    if (!plan) return TPAMD_OK;
+    hipError_t e = plan->tiles_dev ? hipFree(plan->tiles_dev) : hipSuccess;
+    delete plan;
+    if (e != hipSuccess) {
+        set_error("tpamd_copy_plan_destroy: %s", hipGetErrorString(e));
+        return TPAMD_ERR_HIP;
+    }
+    return TPAMD_OK;
+}
+
+extern "C" int tpamd_scale(const void *in_dev, void *out_dev, uint64_t n_elems, int dtype, int world_size, int mul,
+                           void *stream) {
+    TPAMD_REQUIRE(world_size >= 1, "tpamd_scale: world_size %d", world_size);
+    if (n_elems == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(in_dev && out_dev, "tpamd_scale: null pointer");
+    const uint64_t want = (n_elems + 255) / 256;
+    const int grid = static_cast<int>(want < 4096 ? want : 4096);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const float w = static_cast<float>(world_size);
+    switch (dtype) {
+        case TPAMD_BF16: hipLaunchKernelGGL(scale_kernel<TPAMD_BF16>, dim3(grid), dim3(256), 0, s, in_dev, out_dev, n_elems, w, mul); break;
+        case TPAMD_F16: hipLaunchKernelGGL(scale_kernel<TPAMD_F16>, dim3(grid), dim3(256), 0, s, in_dev, out_dev, n_elems, w, mul); break;
+        case TPAMD_F32: hipLaunchKernelGGL(scale_kernel<TPAMD_F32>, dim3(grid), dim3(256), 0, s, in_dev, out_dev, n_elems, w, mul); break;
+        default: set_error("tpamd_scale: unknown dtype %d", dtype); return TPAMD_ERR_INVALID;
+    }
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}

@@ -1,0 +1,77 @@
+"""Shard-local compute modules: the Linear layers of a rank's shard run on the HIP kernels.
+
+In the reference a shard is a deep copy of the user's module whose `torch.nn.Linear`s hold sliced weights and
+run ATen GEMMs (src/tensor_parallel/shard.py:160,184-187; wrapper.py:69-72). Here every `nn.Linear` of a shard
+is re-classed to `ShardLinear` (same parameters, same attributes, still an `nn.Linear`), and SiLU-gated MLP
+blocks with `gate_proj` / `up_proj` / `down_proj` children get a fused gate/up forward.
+
+Inference only: the kernels have no backward; asking for one raises.
+"""
+from __future__ import annotations
+
+import types
+
+import torch
+from torch import nn
+
+from . import _native
+
+
+class _NoBackward(torch.autograd.Function):
+    """Marks a kernel result so that a backward pass through it fails loudly instead of silently stopping."""
+
+    @staticmethod
+    def forward(ctx, out, *inputs):
+        return out.view_as(out)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("tensor_parallel_amd kernels are inference-only: no backward is implemented")
+
+
+def _guard(out: torch.Tensor, *inputs: torch.Tensor) -> torch.Tensor:
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in inputs):
+        return _NoBackward.apply(out, *inputs)
+    return out
+
+
+class ShardLinear(nn.Linear):
+    """`nn.Linear` whose forward is `tpamd_linear` on the shard's (sliced) weight."""
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:  # noqa: A002
+        out = _native.linear(input.detach(), self.weight.detach(), None if self.bias is None else self.bias.detach())
+        return _guard(out, input, self.weight, self.bias)
+
+
+def _is_silu(fn) -> bool:
+    if isinstance(fn, nn.SiLU):
+        return True
+    name = type(fn).__name__.lower()
+    return name in ("silu", "siluactivation", "swish") or fn is torch.nn.functional.silu
+
+
+def _gated_mlp_forward(self, x: torch.Tensor) -> torch.Tensor:
+    gate, up, down = self.gate_proj, self.up_proj, self.down_proj
+    h = _native.swiglu_up(x.detach(), gate.weight.detach(), up.weight.detach())
+    h = _guard(h, x, gate.weight, up.weight)
+    return down(h)
+
+
+def is_gated_silu_mlp(module: nn.Module) -> bool:
+    parts = [getattr(module, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
+    if not all(isinstance(p, nn.Linear) for p in parts):
+        return False
+    gate, up, _ = parts
+    if gate.bias is not None or up.bias is not None or gate.weight.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    return _is_silu(getattr(module, "act_fn", None))
+
+
+def install_shard_kernels(shard: nn.Module) -> None:
+    """Route the shard's Linear layers (and gated MLP blocks) to the HIP kernels, in place."""
+    for module in shard.modules():
+        if type(module) is nn.Linear:
+            module.__class__ = ShardLinear
+    for module in shard.modules():
+        if is_gated_silu_mlp(module):
+            module.forward = types.MethodType(_gated_mlp_forward, module)

@@ -1,0 +1,232 @@
+"""`TensorParallel`: a module split into W rank shards that all live on one HIP device
+(reference: src/tensor_parallel/tensor_parallel.py:26-315).
+
+Construction slices the whole state for all ranks with one launch of the region mover. A forward runs the
+W shards on W host threads, as the reference does (tensor_parallel.py:237-287); the threads meet in the
+"sum" / "gather" ops, which are single-device kernels here. The ZeRO-3 side-car of the reference
+(`sharded=True`) is not part of this package: the argument is accepted, and `apply_sharding` raises.
+"""
+from __future__ import annotations
+
+import logging
+import threading
+from typing import Any, Collection, Optional, Sequence, Union
+
+import torch
+from torch import nn
+
+from .autoconfig import get_default_config
+from .config import Config
+from .shard import make_shard
+from .slicing import BatchSlicer, concat_specs
+from .state_actions import SegmentedAction
+from .utils import nested_flatten, nested_pack
+
+logger = logging.getLogger(__file__)
+
+
+def canonicalize_device(device: Union[torch.device, str, int]) -> torch.device:
+    device = torch.device(device)
+    if device.type == "cuda" and device.index is None:
+        device = torch.device("cuda", 0)
+    return device
+
+
+def check_device_ids(device_ids: Optional[Sequence[Union[torch.device, str]]]) -> Sequence[torch.device]:
+    if device_ids is None:
+        device_ids = list(range(torch.cuda.device_count())) if torch.cuda.is_available() else []
+        device_ids = [torch.device("cuda", i) for i in device_ids]
+    return tuple(canonicalize_device(d) for d in device_ids)
+
+
+class TensorParallel(nn.Module):
+    def __init__(
+        self,
+        module: nn.Module,
+        device_ids: Optional[Sequence[torch.device]] = None,
+        output_device: Optional[torch.device] = None,
+        output_device_index: Optional[int] = None,
+        tensor_parallel_config: Optional[Config] = None,
+        delay_init: bool = False,
+        distributed: bool = True,
+        sharded: bool = True,
+        sharded_param_names: Optional[Collection[str]] = None,
+    ):
+        super().__init__()
+        original_params = sum(p.numel() for p in module.parameters())
+        assert output_device is None or output_device_index is None, "please specify either device or index, not both"
+        device_ids = check_device_ids(device_ids)
+        if output_device is not None:
+            output_device = canonicalize_device(output_device)
+            assert output_device in device_ids, f"Output device {output_device} not in {device_ids}"
+            output_device_index = device_ids.index(output_device)
+        elif output_device_index is None:
+            output_device_index = 0
+
+        self.module_shards = nn.ModuleList()
+        self.devices = device_ids
+        self.output_device_index = output_device_index
+        self.all_cuda = all(d.type == "cuda" for d in self.devices)
+        self.device_ids = [d.index if d.type == "cuda" else None for d in self.devices]
+        self.need_delayed_init = delay_init
+        self.sharding_manager = None
+        world_size = len(self.devices)
+
+        if world_size <= 1:
+            self.module_shards.append(module)
+            if world_size == 1 and not delay_init:
+                self.module_shards[0].to(device_ids[0])
+            return
+        if delay_init:
+            raise NotImplementedError("delay_init builds shards on the host, which tensor_parallel_amd does not do")
+
+        if tensor_parallel_config is None:
+            tensor_parallel_config = get_default_config(module, self.devices)
+            logger.info("Using automatic config: sharding individual linear/emb layers")
+        self.tensor_parallel_config = tensor_parallel_config
+        config_with_ops = tensor_parallel_config.create_collective_ops(self.devices, distributed)
+
+        # all ranks' slicing is queued per device and launched once
+        batches = {}
+        self.modified_parameters_names = set()
+        for rank, device in enumerate(self.devices):
+            batch = batches.setdefault(device, BatchSlicer(device if device.type == "cuda" else None))
+            shard, modified = make_shard(module, device, config_with_ops, rank=rank, world_size=world_size, batch=batch)
+            self.module_shards.append(shard)
+            self.modified_parameters_names.update(modified)
+        self.sliced_bytes = 0
+        for batch in batches.values():
+            self.sliced_bytes += batch.run()
+        for device, batch in batches.items():
+            if device.type == "cuda" and batch.plan is not None:
+                torch.cuda.synchronize(device)  # sources uploaded for slicing are released below
+            batch.close()
+
+        params_per_shard = [sum(p.numel() for p in shard.parameters()) for shard in self.module_shards]
+        assert sum(params_per_shard) >= original_params, "Internal assert failed: lost some parameters during sharding"
+        self.param_fractions = tuple(n / original_params for n in params_per_shard) if original_params else ()
+        inefficiency_rate = (sum(self.param_fractions) - 1) / len(device_ids)
+        logger.log(
+            logging.DEBUG if inefficiency_rate < 0.1 else logging.WARNING,
+            f"Inefficiency warning: model has {original_params} params but shards have {params_per_shard} params. "
+            f"This means that each device uses {inefficiency_rate * 100:.3f}% extra memory for parameters",
+        )
+
+        # one empty parameter per rank, on the rank's device: shows whether someone moved the whole model
+        # (a model built on the meta device keeps them on meta until its weights are loaded)
+        all_meta = all(t.device.type == "meta" for t in module.state_dict().values())
+        self._sanity_check_params = nn.ParameterList(
+            [nn.Parameter(torch.empty(0, device="meta" if all_meta else d), requires_grad=False) for d in self.devices]
+        )
+        self.preserve_shards_when_saving: bool = True
+        if sharded:
+            logger.info("sharded=True (ZeRO-3 of the replicated parameters) is not available; parameters stay replicated")
+
+    def apply_sharding(self, replicated_param_names: Optional[Collection[str]] = None):
+        raise NotImplementedError("ZeRO-3 sharding of replicated parameters is not part of tensor_parallel_amd")
+
+    def prepare_args_kwargs_for_forward(self, *args, **kwargs):
+        """One copy of (args, kwargs) per rank; every tensor is moved to that rank's device (tensor_parallel.py:121-137)."""
+        structure = (args, kwargs)
+        per_rank = []
+        for device in self.devices:
+            leaves = [x.to(device, non_blocking=True) if isinstance(x, torch.Tensor) else x for x in nested_flatten(structure)]
+            per_rank.append(nested_pack(leaves, structure))
+        return zip(*per_rank)
+
+    def forward(self, *args, **kwargs):
+        if len(self.module_shards) <= 1:
+            return [self.module_shards[0](*args, **kwargs)][self.output_device_index]
+        if not all(p.device == d for p, d in zip(self._sanity_check_params, self.devices) if p.device.type != "meta"):
+            raise ValueError(
+                "Model parameters were moved to incorrect devices, did call on model.cuda() or "
+                "model.to(device)? If so, please avoid doing that"
+            )
+        inputs, kwargs_tup = self.prepare_args_kwargs_for_forward(*args, **kwargs)
+        return parallel_apply_simple(self.module_shards, inputs, kwargs_tup, self.devices)[self.output_device_index]
+
+    def set_preserve_shards_when_saving(self, value: bool):
+        self.preserve_shards_when_saving = value
+
+    def state_dict(self, *args, **kwargs):
+        """Sharded names by default; inside `save_tensor_parallel` the original model's names and full tensors,
+        rebuilt with each rule's `undo` (tensor_parallel.py:168-221)."""
+        state_dict = super().state_dict(*args, **kwargs)
+        if self.preserve_shards_when_saving or len(self.module_shards) <= 1:
+            return state_dict
+        world_size = len(self.module_shards)
+        for name in [n for n in state_dict if "_sanity_check_params." in n]:
+            del state_dict[name]
+        for name in [n for n in state_dict if "tp_wrapped_module." in n]:
+            state_dict[name.replace("tp_wrapped_module.", "")] = state_dict.pop(name)
+        marker = "module_shards."
+        first = next((n for n in state_dict if marker in n), None)
+        if first is None:
+            return state_dict
+        shards_prefix = first[: first.find(marker) + len(marker)]
+        module_prefix = shards_prefix[: -len(marker)]
+        rank0 = shards_prefix + "0."
+        for key in [n for n in state_dict if n.startswith(rank0)]:
+            unsharded = key[len(rank0):]
+            pieces = [state_dict.pop(f"{shards_prefix}{r}.{unsharded}") for r in range(world_size)]
+            for pattern, action in self.tensor_parallel_config.state_rules.items():
+                if pattern.search(unsharded) is not None:
+                    state_dict[module_prefix + unsharded] = action.undo(pieces)
+                    break
+            else:
+                state_dict[module_prefix + unsharded] = pieces[0]
+        return state_dict
+
+
+def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devices: Sequence[torch.device]):
+    """Run shard i on (inputs[i], kwargs_tup[i]) in its own thread; re-raise the first failure
+    (tensor_parallel.py:237-287)."""
+    assert len(modules) == len(inputs)
+    kwargs_tup = kwargs_tup if kwargs_tup is not None else ({},) * len(modules)
+    assert len(modules) == len(kwargs_tup)
+    results: dict = {}
+    lock = threading.Lock()
+    grad_enabled = torch.is_grad_enabled()
+
+    def worker(i, module, args, kwargs, device):
+        torch.set_grad_enabled(grad_enabled)
+        try:
+            if device.type == "cuda":
+                torch.cuda.set_device(device)
+            if not isinstance(args, (list, tuple)):
+                args = (args,)
+            out = module(*args, **kwargs)
+            with lock:
+                results[i] = (True, out)
+        except BaseException as e:
+            with lock:
+                results[i] = (False, e)
+            # a rank that fails must not leave its peers waiting in a collective
+            for m in module.modules():
+                for rules in (getattr(m, "input_actions", {}), getattr(m, "output_actions", {})):
+                    for op in rules.values():
+                        barrier = getattr(op, "_barrier", None)
+                        if barrier is not None:
+                            barrier.abort()
+
+    threads = [
+        threading.Thread(target=worker, args=(i, m, a, k, d))
+        for i, (m, a, k, d) in enumerate(zip(modules, inputs, kwargs_tup, devices))
+    ]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    # barriers aborted by a failing rank are usable again for the next forward
+    failures = [r for r in results.values() if not r[0]]
+    if failures:
+        for module in modules:
+            for m in module.modules():
+                for rules in (getattr(m, "input_actions", {}), getattr(m, "output_actions", {})):
+                    for op in rules.values():
+                        barrier = getattr(op, "_barrier", None)
+                        if barrier is not None:
+                            barrier.reset()
+        real = [e for ok, e in failures if not isinstance(e, threading.BrokenBarrierError)]
+        raise (real[0] if real else failures[0][1])
+    return [results[i][1] for i in range(len(modules))]

@@ -1,0 +1,317 @@
+"""Host-side logic of the product, checked without a GPU: slice specs and copy-job tables against the oracle,
+renaming against the golden vectors, rule matching, meta-device model building, and the C ABI's exports."""
+import ctypes
+import json
+import re
+import threading
+from pathlib import Path
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+import tensor_parallel_amd as tp
+from conftest import run_jobs_on_host
+from oracle import slicing as osl
+from tensor_parallel_amd import _native
+from tensor_parallel_amd.aux_actions import split_inner_dim, split_num_heads
+from tensor_parallel_amd.collectives import CollectiveOperation
+from tensor_parallel_amd.config import get_parameter_name_mapping
+from tensor_parallel_amd.shard import find_matching_actions
+from tensor_parallel_amd.slicing import SliceSpec, copy_jobs, tensor_split_range
+from tensor_parallel_amd.slicing_configs import get_gpt2_config, get_llama_config, get_refined_web_config
+
+ROOT = Path(__file__).resolve().parent.parent
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "naming.json").read_text())
+
+
+# ---------------------------------------------------------------------------------------- C ABI
+def test_library_loads_and_exports_every_declared_symbol():
+    assert _native.available(), _native.load_error()
+    header = (ROOT / "include" / "tpamd.h").read_text()
+    declared = set(re.findall(r"\b(tpamd_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_native.EXPORTS)
+    lib = ctypes.CDLL(str(_native.LIB_PATH))
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.tpamd_abi_version() == _native.ABI_VERSION
+
+
+def test_compute_refuses_host_tensors():
+    with pytest.raises(_native.NativeLibraryError):
+        _native.linear(torch.zeros(2, 8), torch.zeros(4, 8))
+    with pytest.raises(_native.NativeLibraryError):
+        _native.reduce_partials([torch.zeros(4), torch.zeros(4)])
+    if not torch.cuda.is_available():
+        with pytest.raises(_native.NativeLibraryError):
+            tp.Split(2, 0)(torch.zeros(4, 4), rank=0)
+        with pytest.raises(_native.NativeLibraryError):
+            tp.TensorParallel(nn.Sequential(nn.Linear(4, 4)), ["cpu", "cpu"])
+
+
+# ---------------------------------------------------------------------------------------- specs and job tables
+def _run_spec_on_host(a: np.ndarray, spec: SliceSpec) -> np.ndarray:
+    src = np.ascontiguousarray(a).view(np.uint8).reshape(-1).copy()
+    out = np.zeros(int(np.prod(spec.out_shape)) * a.itemsize, dtype=np.uint8)
+    SRC, DST = 1 << 20, 1 << 30
+    run_jobs_on_host(copy_jobs(spec, a.itemsize, SRC, DST), {SRC: src, DST: out})
+    return out.view(a.dtype).reshape(spec.out_shape)
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 10, 71])
+@pytest.mark.parametrize("world", [1, 2, 3, 8])
+def test_tensor_split_range_closed_form(n, world):
+    parts = torch.tensor_split(torch.arange(n), world)
+    for r in range(world):
+        start, length = tensor_split_range(n, world, r)
+        assert length == parts[r].numel()
+        if length:
+            assert start == parts[r][0].item()
+
+
+@pytest.mark.parametrize("shape,dim", [((10, 6), 0), ((10, 6), 1), ((4, 9, 5), 1), ((4, 9, 5), -1), ((7,), 0), ((3, 1, 8), 2)])
+@pytest.mark.parametrize("world", [1, 2, 3, 4])
+@pytest.mark.parametrize("dtype", [np.uint8, np.uint16, np.float32])
+def test_split_jobs_match_oracle(shape, dim, world, dtype):
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 200, size=shape).astype(dtype)
+    action = tp.Split(world, dim)
+    for r in range(world):
+        got = _run_spec_on_host(a, action.spec(shape, r))
+        assert np.array_equal(got, osl.split(a, world, dim, r))
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 5])
+def test_chunk_and_grouped_jobs_match_oracle(world):
+    rng = np.random.default_rng(1)
+    a = rng.integers(0, 60000, size=(12, 30)).astype(np.uint16)
+    for r in range(world):
+        for dim, chunk in ((0, 3), (1, 5), (-1, 2), (-2, 4)):
+            spec = tp.SplitInChunks(world, dim, chunk).spec(a.shape, r)
+            assert np.array_equal(_run_spec_on_host(a, spec), osl.split_in_chunks(a, world, dim, chunk, r))
+        for dim, groups, chunk in ((1, 3, 2), (1, 2, 5), (0, 3, 1), (0, 2, 3)):
+            spec = tp.SplitInGroupedChunks(world, dim, groups, chunk).spec(a.shape, r)
+            assert np.array_equal(_run_spec_on_host(a, spec), osl.split_in_grouped_chunks(a, world, dim, groups, chunk, r))
+
+
+def test_undo_jobs_restore_the_tensor():
+    rng = np.random.default_rng(2)
+    a = rng.integers(0, 255, size=(6, 18)).astype(np.uint8)
+    for action in (tp.Split(4, 1), tp.SplitInChunks(3, 0, 2), tp.SplitInGroupedChunks(2, 1, 3, 3)):
+        world = action.world_size
+        parts = [_run_spec_on_host(a, action.spec(a.shape, r)) for r in range(world)]
+        full = np.zeros(a.size, dtype=np.uint8)
+        FULL = 1 << 30
+        bufs = {FULL: full}
+        jobs = []
+        for r, p in enumerate(parts):
+            base = (r + 1) << 20
+            bufs[base] = p.reshape(-1).copy()
+            jobs += copy_jobs(action.spec(a.shape, r), 1, FULL, base, scatter=True)
+        run_jobs_on_host(jobs, bufs)
+        assert np.array_equal(full.reshape(a.shape), a)
+
+
+def test_action_errors():
+    with pytest.raises(AssertionError):
+        tp.SplitInChunks(2, 0, 4).spec((10, 3), 0)  # 10 % 4 != 0, state_actions.py:80
+    with pytest.raises(ValueError):
+        tp.SplitInGroupedChunks(2, -1, 3, 2)
+    assert tp.SplitInChunks(2, 0, 4, optional=True)(None, rank=0) is None
+    with pytest.raises(IndexError):
+        tp.Split(2, 3).spec((4, 4), 0)
+
+
+def test_meta_tensors_pass_through_as_shapes():
+    t = torch.empty(11008, 4096, device="meta", dtype=torch.bfloat16)
+    assert tp.Split(2, 0)(t, rank=1).shape == (5504, 4096)
+    assert tp.Split(8, 1)(t, rank=7).shape == (11008, 512)
+    qkv = torch.empty(9216, 8192, device="meta")
+    assert tp.SplitInChunks(2, 0, 1152)(qkv, rank=0).shape == (4608, 8192)
+    parts = [tp.SplitInGroupedChunks(3, 1, 3, 64)(torch.empty(768, 2304, device="meta"), rank=r) for r in range(3)]
+    assert [p.shape for p in parts] == [(768, 768)] * 3
+    assert tp.SplitInGroupedChunks(3, 1, 3, 64).undo(parts).shape == (768, 2304)
+    assert tp.Scale(4)(t, rank=0).shape == t.shape
+
+
+def test_attr_math_matches_oracle():
+    for heads, world in ((8, 3), (2, 4), (128, 2), (32, 8)):
+        for r in range(world):
+            assert split_num_heads(heads, rank=r, world_size=world) == osl.split_num_heads(heads, r, world)
+            assert split_inner_dim(heads * 64, rank=r, num_heads=heads, world_size=world) == osl.split_inner_dim(heads * 64, r, heads, world)
+
+
+# ---------------------------------------------------------------------------------------- names and rules
+@pytest.mark.parametrize("case", GOLDEN["name_mapping"], ids=lambda c: c["label"])
+def test_name_mapping_golden(case):
+    half = len(case["module_patterns"])  # inputs first, then outputs; the split point does not matter
+    cfg = tp.Config({}, {}, {}, {})
+    cfg.input_rules = {re.compile(p): {} for p in case["module_patterns"][:half]}
+    assert dict(get_parameter_name_mapping(case["names"], cfg)) == case["mapping"]
+
+
+@pytest.mark.parametrize("case", GOLDEN["convert_state_dict"], ids=lambda c: f"W{c['world_size']}-pre{int(c['for_pretrained'])}")
+def test_convert_state_dict_names_and_shapes_golden(case):
+    world = case["world_size"]
+    cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=64, num_attention_heads=8, num_key_value_heads=4),
+                           [torch.device("cuda", 0)] * world)
+    state = {k: torch.empty(shape, device="meta") for k, shape in case["input"].items()}
+    out = tp.convert_state_dict(state, cfg, world, for_pretrained=case["for_pretrained"])
+    assert set(out.keys()) == set(case["output"].keys())
+    for k, shape in case["output"].items():
+        assert list(out[k].shape) == shape, k
+    # unmatched tensors are the same object for every rank (dispatch.py:110)
+    pre = "wrapped_model." if case["for_pretrained"] else ""
+    assert out[pre + "module_shards.0.model.norm.weight"] is state["model.norm.weight"]
+
+
+def test_llama_7b_and_falcon_40b_tables_give_the_baseline_shapes():
+    llama = SimpleNamespace(model_type="llama", hidden_size=4096, num_attention_heads=32, num_key_value_heads=32)
+    state = {
+        "model.layers.0.self_attn.q_proj.weight": (4096, 4096), "model.layers.0.self_attn.k_proj.weight": (4096, 4096),
+        "model.layers.0.self_attn.v_proj.weight": (4096, 4096), "model.layers.0.self_attn.o_proj.weight": (4096, 4096),
+        "model.layers.0.mlp.gate_proj.weight": (11008, 4096), "model.layers.0.mlp.up_proj.weight": (11008, 4096),
+        "model.layers.0.mlp.down_proj.weight": (4096, 11008), "model.embed_tokens.weight": (32000, 4096),
+        "lm_head.weight": (32000, 4096), "model.norm.weight": (4096,),
+    }
+    want = {2: [(2048, 4096)] * 3 + [(4096, 2048), (5504, 4096), (5504, 4096), (4096, 5504), (32000, 2048), (16000, 4096), (4096,)],
+            8: [(512, 4096)] * 3 + [(4096, 512), (1376, 4096), (1376, 4096), (4096, 1376), (32000, 512), (4000, 4096), (4096,)]}
+    for world, shapes in want.items():
+        cfg = get_llama_config(llama, [torch.device("cuda", 0)] * world)
+        meta = {k: torch.empty(s, device="meta", dtype=torch.bfloat16) for k, s in state.items()}
+        out = tp.convert_state_dict(meta, cfg, world)
+        names = get_parameter_name_mapping(state.keys(), cfg)
+        assert [tuple(out[f"module_shards.0.{names[k]}"].shape) for k in state] == shapes
+    falcon = SimpleNamespace(model_type="RefinedWeb", hidden_size=8192, n_head=128, n_head_kv=8, num_attention_heads=128, bias=False, alibi=False)
+    cfg = get_refined_web_config(falcon, [torch.device("cuda", 0)] * 2)
+    meta = {"transformer.h.0.self_attention.query_key_value.weight": torch.empty(9216, 8192, device="meta"),
+            "transformer.h.0.self_attention.dense.weight": torch.empty(8192, 8192, device="meta")}
+    out = tp.convert_state_dict(meta, cfg, 2)
+    assert out["module_shards.0.transformer.h.0.self_attention.tp_wrapped_module.query_key_value.weight"].shape == (4608, 8192)
+    assert out["module_shards.1.transformer.h.0.self_attention.tp_wrapped_module.dense.weight"].shape == (8192, 4096)
+    attn = cfg.attr_rules[next(iter(cfg.attr_rules))]
+    assert attn["num_kv"](8, rank=0) == 4 and attn["num_heads"](128, rank=0) == 64
+
+
+def test_state_rules_first_match_wins_and_module_rules_merge():
+    cfg = tp.Config(
+        state_rules={r"w$": tp.Split(2, 0), r"\.w$": tp.Split(2, 1)},
+        input_rules={r"^a$": {0: "split -1"}, r"a": {"0": "split -1", "x": "scale"}},
+        output_rules={r"^a$": {0: "sum"}, r"^a": {0: "gather -1"}},
+        attr_rules={},
+    )
+    out = tp.convert_state_dict({"m.w": torch.empty(4, 6, device="meta")}, cfg, 2)
+    assert out["module_shards.0.m.w"].shape == (2, 6)
+    assert find_matching_actions("input", "a", cfg.input_rules) == {0: "split -1", "x": "scale"}  # "0" canonicalised to 0
+    with pytest.raises(ValueError):
+        find_matching_actions("output", "a", cfg.output_rules)
+
+
+def test_legacy_state_rules_are_accepted():
+    fn = lambda t, rank: torch.tensor_split(t, 2, dim=0)[rank]  # noqa: E731
+    undo = lambda ts: torch.cat(list(ts), dim=0)  # noqa: E731
+    cfg = tp.Config({r"w$": fn, r"v$": (fn, undo)}, {}, {}, {})
+    acts = list(cfg.state_rules.values())
+    assert all(isinstance(a, tp.StateAction) for a in acts)
+    t = torch.arange(8.0).reshape(4, 2)
+    assert torch.equal(acts[0](t, rank=1), t[2:])
+    assert torch.equal(acts[1].undo([t[:2], t[2:]]), t)
+    with pytest.raises(Exception):
+        acts[0].undo([t])
+    with pytest.raises(Exception):
+        tp.Config({r"w$": 3}, {}, {}, {})
+
+
+def test_gpt2_table_uses_grouped_split():
+    cfg = get_gpt2_config(SimpleNamespace(num_attention_heads=12, hidden_size=768), [torch.device("cuda", 0)] * 2)
+    out = tp.convert_state_dict({"h.0.attn.c_attn.weight": torch.empty(768, 2304, device="meta"),
+                                 "h.0.attn.c_attn.bias": torch.empty(2304, device="meta")}, cfg, 2)
+    assert out["module_shards.1.h.0.attn.tp_wrapped_module.c_attn.weight"].shape == (768, 1152)
+    assert out["module_shards.1.h.0.attn.tp_wrapped_module.c_attn.bias"].shape == (1152,)
+
+
+# ---------------------------------------------------------------------------------------- model building on meta
+def _toy(device="meta"):
+    return nn.Sequential(nn.Embedding(1337, 64, device=device), nn.LayerNorm(64, device=device), nn.Linear(64, 128, device=device),
+                         nn.ReLU(), nn.Linear(128, 10, device=device))
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_meta_model_linear_attributes_follow_weights(world):
+    # tests/test_basic.py:12-29 of the reference, on meta tensors
+    model_tp = tp.TensorParallel(_toy(), ["cuda:0"] * world, sharded=False)
+    assert len(model_tp.module_shards) == world
+    seen = 0
+    for name, module in model_tp.named_modules():
+        if isinstance(module, nn.Linear):
+            assert module.weight.shape == (module.out_features, module.in_features), name
+            seen += 1
+    assert seen == 2 * world
+    shard0 = model_tp.module_shards[0]
+    assert shard0[0].tp_wrapped_module.weight.shape == (1337, 64 // world + (64 % world > 0))
+    total = sum(p.numel() for p in _toy().parameters())
+    assert sum(p.numel() for p in model_tp.parameters()) >= total
+    # names of the sharded model are what convert_state_dict produces (tests/test_saving.py:139-169 of the reference)
+    conv = tp.convert_state_dict(_toy().state_dict(), model_tp.tensor_parallel_config, world)
+    assert set(conv.keys()) == set(model_tp.state_dict().keys())
+    for k, v in model_tp.state_dict().items():
+        assert conv[k].shape == v.shape, k
+
+
+def test_factory_and_single_device_passthrough():
+    m = _toy()
+    one = tp.tensor_parallel(m, ["meta"]) if False else tp.TensorParallel(m, [], sharded=False)
+    assert len(one.module_shards) == 1 and one.module_shards[0] is m
+    two = tp.tensor_parallel(_toy(), ["cuda:0", "cuda:0"])
+    assert isinstance(two, tp.TensorParallel) and two.sharding_manager is None
+    with pytest.raises(NotImplementedError):
+        tp.tensor_parallel(_toy(), ["cuda:0"], distributed=True)
+    with pytest.raises(AssertionError):
+        tp.TensorParallel(nn.Linear(4, 4, device="meta"), ["cuda:0", "cuda:0"])  # not a container, shard.py:31-33
+
+
+def test_unshard_state_dict_names_on_meta():
+    model_tp = tp.TensorParallel(_toy(), ["cuda:0"] * 2, sharded=False)
+    with tp.save_tensor_parallel(model_tp):
+        sd = model_tp.state_dict()
+    ref = _toy().state_dict()
+    assert set(sd.keys()) == set(ref.keys())
+    for k in ref:
+        assert sd[k].shape == ref[k].shape, k
+    assert any(k.startswith("module_shards.1.") for k in model_tp.state_dict())
+
+
+# ---------------------------------------------------------------------------------------- failure handling
+def test_collective_operation_fans_errors_out_and_recovers():
+    world = 3
+
+    def func(*xs):
+        if any(x == "boom" for x in xs):
+            raise RuntimeError("rank 0 failed")
+        return [sum(xs)] * world
+
+    op = CollectiveOperation(world, func, timeout=30)
+    results = [None] * world
+
+    def run(rank, value):
+        try:
+            results[rank] = op(value, rank)
+        except Exception as e:  # noqa: BLE001
+            results[rank] = e
+
+    for values in (["boom", 1, 2], [1, 2, 3]):
+        ts = [threading.Thread(target=run, args=(r, values[r])) for r in range(world)]
+        [t.start() for t in ts]
+        [t.join(60) for t in ts]
+        if values[0] == "boom":
+            assert all(isinstance(r, RuntimeError) for r in results)
+        else:
+            assert results == [6, 6, 6]
+
+
+def test_rendezvous_timeout_does_not_hang():
+    op = CollectiveOperation(2, lambda *xs: list(xs), timeout=0.2)
+    with pytest.raises(threading.BrokenBarrierError):
+        op(1, 0)  # the peer never arrives
