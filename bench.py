@@ -1,0 +1,218 @@
+"""Benchmark of the per-rank hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): the rank-0 shard at W = 2 of a Llama-7B MLP, d = 4096, shard width 5504,
+bf16, M = 4096 tokens. One step = fused gate/up GEMM + SiLU gate, down-projection GEMM (the row-parallel
+partial), and the on-device sum with the other rank's partial. Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+D_MODEL, FFN_SHARD = 4096, 5504
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+
+
+def cpu_baseline(seconds_budget: float = 20.0) -> dict:
+    """The reference path on the host, restated by the oracle: both rank shards of the MLP on two threads,
+    torch CPU ops in bf16, then the sum (device_ids=['cpu','cpu'] in the reference). Bounded sample."""
+    import torch
+
+    from oracle import shard_forward as ofw
+
+    m = 256
+    g = torch.Generator().manual_seed(0)
+    shards = []
+    for _ in range(2):
+        wg, wu = ((torch.randn(FFN_SHARD, D_MODEL, generator=g) * 0.02).bfloat16() for _ in range(2))
+        wd = (torch.randn(D_MODEL, FFN_SHARD, generator=g) * 0.02).bfloat16()
+        shards.append((wg, wu, wd))
+    x = torch.randn(m, D_MODEL, generator=torch.Generator().manual_seed(1)).bfloat16()
+    ofw.run_mlp_shards(x, shards, threads=True)  # warm
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ofw.run_mlp_shards(x, shards, threads=True)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds_budget or reps >= 50:
+            break
+    return {
+        "value": m * reps / dt,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{reps} forwards of {m} tokens through both W=2 shards (2 threads) + sum, bf16 on host, {dt:.1f} s",
+        "host_cpus": os.cpu_count(),
+        "torch": torch.__version__,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--tokens", type=int, default=4096)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the tensor-parallel layer; --gpus above 1 is not supported "
+              "(this package has no inter-GPU collective).", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from tensor_parallel_amd import _native
+
+    if not _native.available():
+        print(f"HIP library missing: {_native.load_error()}", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    M = args.tokens
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def w(shape):
+        return (torch.randn(shape, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+
+    n_sets = 3  # weight sets rotated so that HBM-bound shapes are not served from the 256 MB Infinity Cache
+    sets = [(w((FFN_SHARD, D_MODEL)), w((FFN_SHARD, D_MODEL)), w((D_MODEL, FFN_SHARD))) for _ in range(n_sets)]
+    x = torch.randn(M, D_MODEL, generator=torch.Generator(device=dev).manual_seed(1), device=dev).to(torch.bfloat16)
+    other = torch.randn(M, D_MODEL, generator=g, device=dev).to(torch.bfloat16)  # the other rank's partial
+
+    def step(i, ev=None):
+        wg, wu, wd = sets[i % n_sets]
+        if ev is not None:
+            ev[0].record()
+        h = _native.swiglu_up(x, wg, wu)
+        if ev is not None:
+            ev[1].record()
+        p = _native.linear(h, wd)
+        return _native.reduce_partials([p, other], out=p)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, events[i])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tokens_per_s = M * args.steps / dt
+
+    # dominant kernel: the fused gate/up GEMM (two thirds of the FLOPs). Events sit on the stream the kernels
+    # are launched on (torch's current stream is handed to the library).
+    up_ms = sum(a.elapsed_time(b) for a, b in events) / len(events)
+    up_flops = 4.0 * M * D_MODEL * FFN_SHARD
+    mfma_bound = M >= 256
+    if mfma_bound:
+        achieved = up_flops / (up_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                    "kernel": "gemm_kernel<bf16, swiglu> (tpamd_swiglu_up)", "avg_launch_ms": up_ms,
+                    "algorithmic_flops_per_launch": up_flops}
+    else:
+        up_bytes = 2.0 * FFN_SHARD * D_MODEL * 2 + M * D_MODEL * 2 + M * FFN_SHARD * 2
+        achieved = up_bytes / (up_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                    "kernel": "skinny_kernel<bf16, swiglu> (tpamd_swiglu_up)", "avg_launch_ms": up_ms,
+                    "algorithmic_bytes_per_launch": up_bytes}
+
+    out = {
+        "metric": "rank-0 shard tokens/s + % MFMA/HBM roofline, Llama-7B-shape layer W=2",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"llama7b_mlp_rank0_shard_w2_m{M}_bf16", "d_model": D_MODEL, "ffn_shard": FFN_SHARD,
+                   "tokens": M, "step": "swiglu_up + down + 2-partial reduce", "weights": "N(0,0.02) seed 0", "weight_sets_rotated": n_sets},
+        "roofline": roofline,
+    }
+    if not args.no_extra:
+        out["extra"] = extra_measurements(torch, _native, dev, sets, other)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def _time_us(torch, fn, warm, iters):
+    for i in range(warm):
+        fn(i)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(iters):
+        fn(i)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters * 1e3
+
+
+def extra_measurements(torch, _native, dev, sets, other) -> dict:
+    """The other two targets of the same path, reported beside the headline: decode (M = 1, HBM-bound) and
+    state-dict slicing (8 Llama-2-7B decoder layers' split tensors, W = 2, HBM-bound)."""
+    extra = {}
+    n_sets = len(sets)
+    for m in (1, 16):
+        x = torch.randn(m, D_MODEL, device=dev).to(torch.bfloat16)
+
+        def fn(i):
+            wg, wu, wd = sets[i % n_sets]
+            return _native.linear(_native.swiglu_up(x, wg, wu), wd)
+
+        us = _time_us(torch, fn, 10, 100)
+        by = 3.0 * FFN_SHARD * D_MODEL * 2 + 38400.0 * m
+        extra[f"decode_m{m}"] = {"us_per_step": us, "tokens_per_s": m / us * 1e6, "GBps": by / us / 1e3,
+                                 "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS, "algorithmic_bytes": by}
+    from types import SimpleNamespace
+
+    from tensor_parallel_amd.slicing import BatchSlicer
+    from tensor_parallel_amd.slicing_configs import get_llama_config
+
+    layers, world = 8, 2
+    cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=4096, num_attention_heads=32, num_key_value_heads=32), [dev] * world)
+    state = {}
+    for layer in range(layers):
+        p = f"model.layers.{layer}."
+        for name, shape in (("self_attn.q_proj", (4096, 4096)), ("self_attn.k_proj", (4096, 4096)), ("self_attn.v_proj", (4096, 4096)),
+                            ("self_attn.o_proj", (4096, 4096)), ("mlp.gate_proj", (11008, 4096)), ("mlp.up_proj", (11008, 4096)),
+                            ("mlp.down_proj", (4096, 11008))):
+            state[p + name + ".weight"] = torch.empty(shape, device=dev, dtype=torch.bfloat16).normal_(0, 0.02)
+    batch = BatchSlicer(dev)
+    keep = []
+    for r in range(world):
+        for name, t in state.items():
+            action = next(a for p, a in cfg.state_rules.items() if p.search(name))
+            keep.append(batch.add(t, action.spec(tuple(t.shape), r)))
+    plan = batch.build()
+    us = _time_us(torch, lambda i: plan.run(), 2, 10)
+    moved = 2.0 * plan.nbytes
+    extra["slicing_w2"] = {"tensors": len(state), "bytes_read_plus_written": moved, "us_per_launch": us,
+                           "GBps": moved / us / 1e3, "hbm_frac": moved / us / 1e3 / PEAK_HBM_GBS}
+    batch.close()
+    return extra
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -17,6 +17,7 @@ from typing import Any, Callable, List, Optional
 import torch
 
 from . import _native
+from .shard_modules import _guard
 from .slicing import concat_dim
 
 RENDEZVOUS_TIMEOUT_S = 600.0
@@ -76,9 +77,9 @@ class DeviceAllReduce(CollectiveOperation):
         self.accum = accum
 
     def _reduce(self, *parts: torch.Tensor):
-        out = _native.reduce_partials(list(parts), accum=self.accum)
+        out = _native.reduce_partials([p.detach() for p in parts], accum=self.accum)
         # each rank continues with a tensor of its own: later in-place ops on one rank must not leak
-        return [out] + [out.clone() for _ in range(self.world_size - 1)]
+        return [_guard(o, *parts) for o in [out] + [out.clone() for _ in range(self.world_size - 1)]]
 
 
 class DeviceAllGather(CollectiveOperation):
@@ -91,5 +92,5 @@ class DeviceAllGather(CollectiveOperation):
     def _gather(self, *parts: torch.Tensor):
         for p in parts:
             _native.require_device(p, "gather")
-        out = concat_dim(list(parts), self.dim)
-        return [out] + [out.clone() for _ in range(self.world_size - 1)]
+        out = concat_dim([p.detach() for p in parts], self.dim)
+        return [_guard(o, *parts) for o in [out] + [out.clone() for _ in range(self.world_size - 1)]]

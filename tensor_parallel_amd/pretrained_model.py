@@ -27,6 +27,8 @@ def find_predefined_tensor_parallel_config(model_config: PretrainedConfig, devic
 
 class TensorParallelPreTrainedModel(PreTrainedModel):
     is_parallelizable = model_parallel = True
+    # the wrapper only delegates to the wrapped model, whatever attention implementation that one runs
+    _supports_sdpa = _supports_flash_attn = _supports_flex_attn = _supports_attention_backend = True
 
     def __init__(
         self,

@@ -1,0 +1,141 @@
+"""Rank-shard Linears on the GPU against the oracle (torch on CPU).
+
+Tolerances: bf16/fp16 results are compared with the fp32 CPU product of the same bf16/fp16 inputs at
+rtol 2e-2 (atol scaled to the typical output magnitude), fp32 results at rtol 1e-5."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import shard_forward as ofw
+from tensor_parallel_amd import _native
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+RTOL_HALF = 2e-2
+RTOL_F32 = 1e-5
+
+
+def rnd(shape, seed, std=1.0, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std).to(dtype)
+
+
+def check_half(got, want_f32, K, x_std=1.0, w_std=0.02):
+    """rtol 2e-2 plus an absolute floor of 2e-2 output standard deviations (entries near zero)."""
+    sigma = x_std * w_std * math.sqrt(K)
+    torch.testing.assert_close(got.float().cpu(), want_f32, rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 32, 33, 64, 130, 256, 300])
+@pytest.mark.parametrize("N,K", [(64, 64), (132, 200), (260, 72), (512, 1024)])
+def test_linear_half(dtype, M, N, K):
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
+    want = F.linear(x.float(), w.float(), b.float())
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert got.shape == (M, N) and got.dtype == dtype
+    check_half(got, want, K)
+    got_nb = _native.linear(x.to(DEV), w.to(DEV))
+    check_half(got_nb, F.linear(x.float(), w.float()), K)
+    # leading dimensions are kept
+    if M % 2 == 0:
+        got3 = _native.linear(x.view(2, M // 2, K).to(DEV), w.to(DEV))
+        assert got3.shape == (2, M // 2, N) and torch.equal(got3.view(M, N), got_nb)
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 31, 40, 128, 257])
+@pytest.mark.parametrize("N,K", [(64, 64), (100, 136), (344, 128), (256, 512)])
+def test_swiglu_matches_oracle(M, N, K):
+    x, wg, wu = rnd((M, K), 1), rnd((N, K), 0, 0.05), rnd((N, K), 3, 0.05)
+    got = _native.swiglu_up(x.to(DEV), wg.to(DEV), wu.to(DEV))
+    want32 = ofw.gated_mlp_hidden(x.float(), wg.float(), wu.float())
+    sigma = (0.05 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(got.float().cpu(), want32, rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    # against the reference's own bf16 op chain on the host: same roundings, so differences are a few ulp
+    want_bf16 = ofw.gated_mlp_hidden(x, wg, wu).float()
+    torch.testing.assert_close(got.float().cpu(), want_bf16, rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 10, 16), (7, 33, 50), (64, 64, 64), (130, 70, 129), (128, 768, 3072)])
+def test_linear_fp32(M, N, K):
+    x, w, b = rnd((M, K), 1, 1.0, torch.float32), rnd((N, K), 0, 0.02, torch.float32), rnd((N,), 2, 0.1, torch.float32)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV)).cpu()
+    want = F.linear(x.double(), w.double(), b.double()).float()
+    torch.testing.assert_close(got, want, rtol=RTOL_F32, atol=RTOL_F32 * 0.02 * math.sqrt(K))
+
+
+def test_gelu_epilogue_and_argument_errors():
+    x, w = rnd((40, 64), 1, 1.0, torch.float16), rnd((64, 64), 0, 0.1, torch.float16)
+    for M in (8, 40):
+        got = _native.linear(x[:M].to(DEV), w.to(DEV), act=_native.ACT_GELU)
+        want = F.gelu(F.linear(x[:M].float(), w.float()))
+        torch.testing.assert_close(got.float().cpu(), want, rtol=RTOL_HALF, atol=2e-2)
+    with pytest.raises(ValueError):
+        _native.linear(x.to(DEV), rnd((64, 60), 0, 0.1, torch.float16).to(DEV))  # K mismatch
+    with pytest.raises(ValueError):
+        _native.linear(rnd((4, 12), 0, 1, torch.float16).to(DEV), rnd((8, 12), 0, 1, torch.float16).to(DEV))  # K % 8
+    with pytest.raises(TypeError):
+        _native.linear(x.to(DEV), w.to(DEV).bfloat16())
+    assert _native.linear(torch.empty(0, 64, dtype=torch.float16, device=DEV), w.to(DEV)).shape == (0, 64)
+
+
+@pytest.mark.parametrize("world", [2, 4])
+def test_shards_recombine(world):
+    """Column-parallel shard outputs are the columns of the unsplit product bit for bit (same kernel, same K
+    order); row-parallel partials reduced on the device agree with the unsplit product within tolerance."""
+    M, N, K = 96, 256, 512
+    x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
+    full = _native.linear(x, w)
+    cols = [_native.linear(x, torch.tensor_split(w, world, 0)[r].contiguous()) for r in range(world)]
+    assert torch.equal(torch.cat(cols, dim=-1), full)
+    parts = [_native.linear(torch.tensor_split(x, world, 1)[r].contiguous(), torch.tensor_split(w, world, 1)[r].contiguous()) for r in range(world)]
+    summed = _native.reduce_partials(parts)
+    check_half(summed, F.linear(x.float().cpu(), w.float().cpu()), K)
+    # strided (non-copied) column slices of x and w are accepted as they are: leading dimension > K
+    xs, ws = torch.tensor_split(x, world, 1)[1], torch.tensor_split(w, world, 1)[1]
+    assert not xs.is_contiguous()
+    assert torch.equal(_native.linear(xs, ws), parts[1])
+
+
+@pytest.mark.parametrize("M", [1, 16, 512])
+def test_llama_mlp_shard_full_shape(M):
+    """BASELINE config 2: rank-0 shard at W=2 of a Llama-7B MLP, d=4096, ffn shard 5504, bf16."""
+    d, f = 4096, 5504
+    x, wg, wu, wd = rnd((M, d), 1), rnd((f, d), 0, 0.02), rnd((f, d), 3, 0.02), rnd((d, f), 4, 0.02)
+    xd, gd, ud, dd = (t.to(DEV) for t in (x, wg, wu, wd))
+    h = _native.swiglu_up(xd, gd, ud)
+    y = _native.linear(h, dd)
+    h_want = ofw.gated_mlp_hidden(x.float(), wg.float(), wu.float())
+    sig_h = (0.02 * math.sqrt(d)) ** 2
+    torch.testing.assert_close(h.float().cpu(), h_want, rtol=RTOL_HALF, atol=RTOL_HALF * sig_h)
+    y_want = F.linear(h.float().cpu(), wd.float())  # the down projection of the hidden the device produced
+    sig_y = 0.5 * sig_h * 0.02 * math.sqrt(f)
+    torch.testing.assert_close(y.float().cpu(), y_want, rtol=RTOL_HALF, atol=RTOL_HALF * sig_y)
+    if M <= 16:  # the reference's op chain in bf16 on the host, end to end
+        y_ref = ofw.gated_mlp_shard(x, wg, wu, wd).float()
+        torch.testing.assert_close(y.float().cpu(), y_ref, rtol=RTOL_HALF, atol=2 * RTOL_HALF * sig_y)
+
+
+def test_llama_mlp_shard_prefill_4096_sampled_rows():
+    """M = 4096 at the full shape: 96 sampled rows against the host, all rows for finiteness, and row
+    independence (a row's result does not depend on which other rows share the launch)."""
+    d, f, M = 4096, 5504, 4096
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(M, d, generator=g, device=DEV).to(torch.bfloat16)
+    wg, wu = ((torch.randn(f, d, generator=g, device=DEV) * 0.02).to(torch.bfloat16) for _ in range(2))
+    wd = (torch.randn(d, f, generator=g, device=DEV) * 0.02).to(torch.bfloat16)
+    h = _native.swiglu_up(x, wg, wu)
+    y = _native.linear(h, wd)
+    assert torch.isfinite(y.float()).all()
+    rows = torch.cat([torch.arange(0, 32), torch.arange(2030, 2062), torch.arange(4064, 4096)])
+    xs = x[rows.to(DEV)].cpu()
+    h_want = ofw.gated_mlp_hidden(xs.float(), wg.float().cpu(), wu.float().cpu())
+    sig_h = (0.02 * math.sqrt(d)) ** 2
+    torch.testing.assert_close(h[rows.to(DEV)].float().cpu(), h_want, rtol=RTOL_HALF, atol=RTOL_HALF * sig_h)
+    y_want = F.linear(h[rows.to(DEV)].float().cpu(), wd.float().cpu())
+    sig_y = 0.5 * sig_h * 0.02 * math.sqrt(f)
+    torch.testing.assert_close(y[rows.to(DEV)].float().cpu(), y_want, rtol=RTOL_HALF, atol=RTOL_HALF * sig_y)
+    sub = _native.linear(_native.swiglu_up(x[1024:1536].contiguous(), wg, wu), wd)
+    assert torch.equal(sub, y[1024:1536])

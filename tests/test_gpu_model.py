@@ -1,0 +1,132 @@
+"""Whole-module parity through the drop-in API: rank shards on one GPU recombine to the unsplit module."""
+from copy import deepcopy
+from types import SimpleNamespace
+
+import pytest
+import torch
+from torch import nn
+
+import tensor_parallel_amd as tp
+from tensor_parallel_amd.shard_modules import ShardLinear
+from tensor_parallel_amd.slicing_configs import get_llama_config
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def toy():
+    return nn.Sequential(nn.Embedding(1337, 64), nn.LayerNorm(64), nn.Linear(64, 128), nn.ReLU(), nn.Linear(128, 12))
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 4])
+def test_embeds_and_linear_forward_parity(world):
+    # forward half of tests/test_basic.py:32-56 of the reference, fp32, atol 1e-6 / rtol 1e-5
+    torch.manual_seed(0)
+    model = toy()
+    inputs = torch.randint(1, 1000, size=(1, 10))
+    with torch.no_grad():
+        ref = model(inputs)
+    model_tp = tp.TensorParallel(deepcopy(model), [DEV] * world, sharded=False)
+    with torch.no_grad():
+        out = model_tp(inputs.to(DEV))
+    torch.testing.assert_close(out.cpu(), ref, atol=1e-6, rtol=1e-5)
+    if world > 1:
+        assert all(isinstance(m, ShardLinear) for m in model_tp.modules() if isinstance(m, nn.Linear))
+        for m in model_tp.modules():
+            if isinstance(m, nn.Linear):
+                assert m.weight.shape == (m.out_features, m.in_features)
+        # un-shard: original names and bit-identical tensors (tests/test_saving.py:43-62 of the reference)
+        with tp.save_tensor_parallel(model_tp):
+            sd = model_tp.state_dict()
+        assert set(sd) == set(model.state_dict())
+        for k, v in model.state_dict().items():
+            assert torch.equal(sd[k].cpu(), v), k
+
+
+def test_backward_is_refused():
+    model_tp = tp.TensorParallel(toy(), [DEV] * 2, sharded=False)
+    out = model_tp(torch.randint(1, 1000, size=(1, 10), device=DEV))
+    with pytest.raises(NotImplementedError):
+        out.norm().backward()
+
+
+def test_worker_failure_is_raised_not_hung():
+    class Boom(nn.Module):
+        def forward(self, x):
+            raise RuntimeError("shard failed")
+
+    model = nn.Sequential(nn.Linear(8, 8), Boom())
+    model_tp = tp.TensorParallel(model, [DEV] * 2, sharded=False)
+    with pytest.raises(RuntimeError, match="shard failed"):
+        model_tp(torch.randn(2, 8, device=DEV))
+    with pytest.raises(ValueError):
+        model_tp.to("cpu")(torch.randn(2, 8))
+
+
+class LlamaMLP(nn.Module):
+    def __init__(self, d, f):
+        super().__init__()
+        self.gate_proj, self.up_proj, self.down_proj = nn.Linear(d, f, bias=False), nn.Linear(d, f, bias=False), nn.Linear(f, d, bias=False)
+        self.act_fn = nn.SiLU()
+
+    def forward(self, x):
+        return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+
+class Block(nn.Module):
+    def __init__(self, d, f):
+        super().__init__()
+        self.mlp = LlamaMLP(d, f)
+
+    def forward(self, x):
+        return self.mlp(x)
+
+
+@pytest.mark.parametrize("world", [2, 4])
+@pytest.mark.parametrize("tokens", [3, 200])
+def test_llama_mlp_block_with_llama_rules(world, tokens):
+    torch.manual_seed(0)
+    d, f = 256, 688
+    block = Block(d, f)
+    for p in block.parameters():
+        nn.init.normal_(p, std=0.05)
+    block = block.to(torch.bfloat16)
+    x = torch.randn(2, tokens, d).to(torch.bfloat16)
+    with torch.no_grad():
+        ref = block.float()(x.float())
+    block = block.to(torch.bfloat16)
+    cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=d, num_attention_heads=4, num_key_value_heads=4), [DEV] * world)
+    model_tp = tp.TensorParallel(block, [DEV] * world, tensor_parallel_config=cfg, sharded=False)
+    shard_mlp = model_tp.module_shards[0].mlp.tp_wrapped_module
+    assert shard_mlp.gate_proj.weight.shape == (f // world, d) and shard_mlp.down_proj.weight.shape == (d, f // world)
+    with torch.no_grad():
+        out = model_tp(x.to(DEV))
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=2e-2, atol=2e-2 * ref.std().item())
+
+
+def test_opt_125m_tensor_parallel_logits():
+    """BASELINE config 1: OPT-125m architecture, fp32, N(0, 0.02) weights from seed 0, W = 2 through
+    tp.tensor_parallel, batch 2 x seq 64; final logits against the unsplit model."""
+    from transformers import OPTConfig, OPTForCausalLM
+
+    torch.manual_seed(0)
+    model = OPTForCausalLM(OPTConfig()).eval()
+    with torch.no_grad():
+        for p in model.parameters():
+            p.normal_(0.0, 0.02)
+    ids = torch.randint(0, 50272, (2, 64), generator=torch.Generator().manual_seed(1))
+    with torch.no_grad():
+        ref = model(input_ids=ids, use_cache=False).logits
+    model_tp = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    assert isinstance(model_tp, tp.TensorParallelPreTrainedModel)
+    shard0 = model_tp.wrapped_model.module_shards[0]
+    assert shard0.model.decoder.layers[0].fc1.tp_wrapped_module.weight.shape == (1536, 768)
+    assert shard0.model.decoder.embed_tokens.tp_wrapped_module.weight.shape == (50272, 384)
+    for r, shard in enumerate(model_tp.wrapped_model.module_shards):  # rank shards are the oracle's slices
+        w = shard.model.decoder.layers[3].fc2.tp_wrapped_module.weight
+        assert torch.equal(w.cpu(), torch.tensor_split(model.model.decoder.layers[3].fc2.weight, 2, dim=0)[r])
+    with torch.no_grad():
+        out = model_tp(input_ids=ids.to(DEV), use_cache=False).logits
+    assert out.shape == (2, 64, 50272)
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=3e-3)
+    assert (out.cpu() - ref).abs().max().item() < 1e-3

@@ -1,0 +1,72 @@
+"""int8 weight-only shard Linear with 16-bit outlier columns against its closed-form definition (oracle/quant.py,
+evaluated in float64). The reference has no such path: parity is against the definition, not the reference."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+from tensor_parallel_amd import _native
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def make_case(M, N, K, n_out, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(dtype).float().numpy()
+    x = torch.randn(M, K, generator=g)
+    cols = np.sort(torch.randperm(K, generator=torch.Generator().manual_seed(2))[:n_out].numpy())
+    x[:, cols] *= 20
+    x = x.to(dtype)
+    wq, scale, w_out = oq.quantize_rows(w, cols)
+    return x, wq, scale, cols, w_out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 2, 5, 16, 17, 33, 64, 70])
+@pytest.mark.parametrize("N,K,n_out", [(64, 256, 0), (48, 512, 3), (128, 1024, 41), (36, 272, 33)])
+def test_linear_w8_matches_definition(dtype, M, N, K, n_out):
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, dtype)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
+    got = _native.linear_w8(
+        x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+        torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None,
+        torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None,
+    )
+    sigma = 0.02 * math.sqrt(K + 400 * n_out)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
+
+
+def test_int8_conversion_is_exact_for_every_code():
+    """Every int8 code -127..127 (and -128) through the in-register conversion: x = one-hot rows pick out
+    single weights, scale 1, so the output must equal the integer exactly."""
+    K = 256
+    codes = torch.arange(-128, 128, dtype=torch.int16).to(torch.int8)  # one row holding every code once
+    wq = torch.stack([codes, codes.flip(0)] * 8)  # N = 16
+    x = torch.eye(K)[:64]
+    for dtype in (torch.float16, torch.bfloat16):
+        for m0 in range(0, K, 64):
+            xs = torch.eye(K)[m0 : m0 + 64].to(dtype)
+            got = _native.linear_w8(xs.to(DEV), wq.to(DEV), torch.ones(16, device=DEV), None, None)
+            want = wq[:, m0 : m0 + 64].t().float()
+            assert torch.equal(got.float().cpu(), want)
+
+
+def test_falcon_mlp_shard_full_shape():
+    """BASELINE config 5 at its real shape: up [16384 x 8192] + GELU, down [8192 x 16384], fp16, batch 4."""
+    M, d, f = 4, 8192, 16384
+    x, wq1, s1, c1, o1 = make_case(M, f, d, 41, torch.float16, 0)
+    up = _native.linear_w8(x.to(DEV), torch.from_numpy(wq1).to(DEV), torch.from_numpy(s1).to(DEV),
+                           torch.from_numpy(c1.astype(np.int32)).to(DEV), torch.from_numpy(o1).half().to(DEV), act=_native.ACT_GELU)
+    want_up = oq.linear_w8_f64(x.float().numpy(), wq1, s1, c1, o1)
+    want_up = torch.nn.functional.gelu(torch.from_numpy(want_up))
+    torch.testing.assert_close(up.double().cpu(), want_up, rtol=2e-2, atol=2e-2 * 0.02 * math.sqrt(d + 400 * 41))
+    h, wq2, s2, c2, o2 = make_case(M, d, f, 82, torch.float16, 1)
+    h = up.cpu()  # feed the device's own hidden forward
+    down = _native.linear_w8(up, torch.from_numpy(wq2).to(DEV), torch.from_numpy(s2).to(DEV),
+                             torch.from_numpy(c2.astype(np.int32)).to(DEV), torch.from_numpy(o2).half().to(DEV))
+    want_down = oq.linear_w8_f64(h.float().numpy(), wq2, s2, c2, o2)
+    scale_y = float(np.abs(want_down).std())
+    torch.testing.assert_close(down.double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * scale_y)
