@@ -125,9 +125,10 @@ int tpamd_reduce_partials(const void *const *parts_dev, int world_size, void *ou
  *   column-parallel shard: w = rows ts(N,W,r) of the full weight, bias sliced alike;
  *   row-parallel shard:    w = columns ts(K,W,r), x = the matching columns, bias NULL or pre-scaled;
  *                          the result is a partial sum for tpamd_reduce_partials.
- * bias_dev may be NULL. x, w, y must be 16-byte aligned; for bf16/f16 K, ldx and ldw must be
- * multiples of 8 and N, ldy multiples of 4 (every shape the slicing rules above produce from
- * head-aligned models satisfies this).
+ * bias_dev may be NULL. Any shape and alignment is accepted. bf16/f16 operands run on the MFMA kernels
+ * when x, w are 16-byte aligned, y and bias 8-byte aligned, K, ldx, ldw are multiples of 8 and N, ldy
+ * multiples of 4 (every shape the slicing rules above produce from head-aligned models); other
+ * bf16/f16 operands and all fp32 operands run on a scalar-load FMA kernel.
  * ---------------------------------------------------------------------------------------------- */
 int tpamd_linear(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, void *stream);

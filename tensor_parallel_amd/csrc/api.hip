@@ -15,7 +15,7 @@ void set_error(const char *fmt, ...) {
 }
 
 int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias, void *y, int64_t M, int64_t N,
-                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu, hipStream_t s);
+                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu, bool generic, hipStream_t s);
 int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *scale,
                     const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N, int64_t K,
                     int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
@@ -27,6 +27,14 @@ namespace {
 constexpr int64_t SKINNY_MAX_M = 32;
 constexpr int64_t SKINNY_W8_SLAB = 64;
 
+// What the MFMA kernels need from 16-bit operands: 16-byte aligned rows of x and w, 8-byte aligned groups of 4
+// outputs. Anything else goes to the scalar-load kernel.
+bool mfma_ok(const void *x, const void *w, const void *w2, const void *bias, const void *y, int64_t N, int64_t K,
+             int64_t ldx, int64_t ldw, int64_t ldy) {
+    return aligned(x, 16) && aligned(w, 16) && (!w2 || aligned(w2, 16)) && aligned(y, 8) && (!bias || aligned(bias, 8)) &&
+           K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && N % 4 == 0 && ldy % 4 == 0;
+}
+
 int check_common(const char *who, const void *x, const void *w, const void *y, int64_t M, int64_t N, int64_t K,
                  int64_t ldx, int64_t ldw, int64_t ldy, int dtype) {
     TPAMD_REQUIRE(M >= 0 && N >= 0 && K >= 0, "%s: negative dimension (M=%lld N=%lld K=%lld)", who, (long long)M,
@@ -37,13 +45,6 @@ int check_common(const char *who, const void *x, const void *w, const void *y, i
     TPAMD_REQUIRE(x && w && y, "%s: null pointer", who);
     TPAMD_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "%s: leading dimension smaller than the row (ldx=%lld ldw=%lld ldy=%lld)",
                   who, (long long)ldx, (long long)ldw, (long long)ldy);
-    if (dtype != TPAMD_F32) {
-        TPAMD_REQUIRE(aligned(x, 16) && aligned(w, 16) && aligned(y, 8), "%s: x/w must be 16-byte and y 8-byte aligned", who);
-        TPAMD_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "%s: K, ldx, ldw must be multiples of 8 (K=%lld ldx=%lld ldw=%lld)",
-                      who, (long long)K, (long long)ldx, (long long)ldw);
-        TPAMD_REQUIRE(N % 4 == 0 && ldy % 4 == 0, "%s: N and ldy must be multiples of 4 (N=%lld ldy=%lld)", who,
-                      (long long)N, (long long)ldy);
-    }
     return TPAMD_OK;
 }
 
@@ -61,26 +62,26 @@ extern "C" int tpamd_linear(const void *x_dev, const void *w_dev, const void *bi
     if (rc != TPAMD_OK) return rc;
     TPAMD_REQUIRE(act == TPAMD_ACT_NONE || act == TPAMD_ACT_GELU, "tpamd_linear: unknown activation %d", act);
     if (M == 0 || N == 0) return TPAMD_OK;
-    if (bias_dev && dtype != TPAMD_F32) TPAMD_REQUIRE(aligned(bias_dev, 8), "tpamd_linear: bias must be 8-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype != TPAMD_F32 && M <= SKINNY_MAX_M)
+    const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, w_dev, nullptr, bias_dev, y_dev, N, K, ldx, ldw, ldy);
+    if (fast && M <= SKINNY_MAX_M)
         return skinny_dispatch(x_dev, w_dev, nullptr, bias_dev, nullptr, nullptr, nullptr, 0, y_dev, M, N, K, ldx, ldw, ldy, 0,
                                dtype, act, false, false, s);
-    return gemm_dispatch(x_dev, w_dev, nullptr, bias_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, false, s);
+    return gemm_dispatch(x_dev, w_dev, nullptr, bias_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, false, !fast, s);
 }
 
 extern "C" int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void *wu_dev, void *h_dev, int64_t M, int64_t N,
                                int64_t K, int64_t ldx, int64_t ldw, int64_t ldh, int dtype, void *stream) {
     int rc = check_common("tpamd_swiglu_up", x_dev, wg_dev, h_dev, M, N, K, ldx, ldw, ldh, dtype);
     if (rc != TPAMD_OK) return rc;
-    TPAMD_REQUIRE(dtype != TPAMD_F32, "tpamd_swiglu_up: fp32 is not supported, use tpamd_linear twice");
     if (M == 0 || N == 0) return TPAMD_OK;
-    TPAMD_REQUIRE(wu_dev && aligned(wu_dev, 16), "tpamd_swiglu_up: wu must be non-null and 16-byte aligned");
+    TPAMD_REQUIRE(wu_dev != nullptr, "tpamd_swiglu_up: wu is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (M <= SKINNY_MAX_M)
+    const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, wg_dev, wu_dev, nullptr, h_dev, N, K, ldx, ldw, ldh);
+    if (fast && M <= SKINNY_MAX_M)
         return skinny_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw, ldh, 0,
                                dtype, TPAMD_ACT_NONE, true, false, s);
-    return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true, s);
+    return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true, !fast, s);
 }
 
 extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,

@@ -1,12 +1,12 @@
 // Rank-shard Linear for decode-sized M (M <= 64): weight streaming, HBM-bound.
 //
 // A block owns 16 output columns (16 rows of w; for the SiLU-gated pair 16 gate rows + 16 up rows) and
-// splits K over its wavefronts in chunks of 64 bytes per lane. Each lane loads 64 contiguous bytes of
-// one w row (4 lanes cover 256 contiguous bytes of that row) straight from global memory into MFMA
-// operands: v_mfma_f32_16x16x32 does both the multiply and the reduction over K, so no cross-lane
-// shuffles are needed. The K positions an MFMA sees are a permutation of the real ones; x is loaded
-// with the same permutation. Partial sums of the wavefronts meet in LDS; the epilogue applies scale,
-// outliers, bias, activation and stores 16 consecutive columns per row.
+// splits K over its wavefronts in chunks of 256 bytes of every w row. A chunk is fetched by 4 wavefront-wide
+// 16-byte loads; in each of them the 4 lanes that share a row read 64 contiguous bytes, so every load
+// instruction touches 16 whole 64-byte sectors. The loaded registers are MFMA operands as they are:
+// v_mfma_f32_16x16x32 does both the multiply and the reduction over K, so no cross-lane shuffles are
+// needed. Partial sums of the wavefronts meet in LDS; the epilogue applies scale, outliers, bias,
+// activation and stores 16 consecutive columns per row.
 //
 // The weight is either the activation dtype (bf16/f16) or int8 (weight-only quantisation: converted to
 // the activation dtype in registers, exact for |q| <= 128).
@@ -80,6 +80,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     constexpr int CHUNK_K = LANE_K * 4;       // K elements per chunk
     constexpr int WV = 4;                     // 16-byte loads of w per lane per chunk
     constexpr int XV = LANE_K / 8;            // 16-byte loads of x per lane per chunk per m-tile
+    constexpr int WK = W8 ? 16 : 8;           // K elements in one 16-byte load of w
 
     __shared__ float red[SK_WAVES][NMAT][MT][4][64];
 
@@ -91,15 +92,16 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     wrow = wrow < p.N ? wrow : p.N - 1;
     const int wbytes = W8 ? 1 : 2;
     const char *wp[NMAT];
-    wp[0] = p.w + (static_cast<int64_t>(wrow) * p.ldw + lg * LANE_K) * wbytes;
-    if constexpr (NMAT == 2) wp[1] = p.w2 + (static_cast<int64_t>(wrow) * p.ldw + lg * LANE_K) * wbytes;
+    // load v of a chunk: this lane's 16 bytes sit at byte lg*16 + v*64 of the chunk's 256 bytes of row wrow
+    wp[0] = p.w + static_cast<int64_t>(wrow) * p.ldw * wbytes + lg * 16;
+    if constexpr (NMAT == 2) wp[1] = p.w2 + static_cast<int64_t>(wrow) * p.ldw * wbytes + lg * 16;
     const char *xp[MT];
     bool xok[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + lr;
         xok[t] = m < p.M;
-        xp[t] = p.x + (static_cast<int64_t>(xok[t] ? m : 0) * p.ldx + lg * LANE_K) * 2;
+        xp[t] = p.x + (static_cast<int64_t>(xok[t] ? m : 0) * p.ldx + lg * WK) * 2;
     }
 
     f32x4 acc[NMAT][MT];
@@ -118,25 +120,28 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     uint4 xv[XPRE ? 2 : 1][MT][XV];
     auto load_w = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
-        const int kbase = c * CHUNK_K + lg * LANE_K;  // first K element of this lane
+        const int kbase = c * CHUNK_K + lg * WK;  // first K element of this lane's load 0
         const int64_t off = static_cast<int64_t>(c) * CHUNK_K * wbytes;
 #pragma unroll
         for (int a = 0; a < NMAT; ++a)
 #pragma unroll
             for (int v = 0; v < WV; ++v) {
-                const int k = kbase + v * (LANE_K / WV);
-                wv[buf][a][v] = k < p.K ? nt_load_u4(reinterpret_cast<const uint4 *>(wp[a] + off) + v) : zero4;
+                const int k = kbase + v * 4 * WK;
+                wv[buf][a][v] = k < p.K ? nt_load_u4(wp[a] + off + v * 64) : zero4;
             }
     };
     auto load_x = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
-        const int kbase = c * CHUNK_K + lg * LANE_K;
+        const int kbase = c * CHUNK_K + lg * WK;
         const int64_t xoff = static_cast<int64_t>(c) * CHUNK_K * 2;
 #pragma unroll
         for (int t = 0; t < MT; ++t)
 #pragma unroll
-            for (int v = 0; v < XV; ++v)
-                xv[buf][t][v] = (xok[t] && kbase + v * 8 < p.K) ? *(reinterpret_cast<const uint4 *>(xp[t] + xoff) + v) : zero4;
+            for (int v = 0; v < XV; ++v) {
+                // the x elements that meet w load v (bf16/f16 w) or half (v & 1) of w load v / 2 (int8 w)
+                const int krel = W8 ? (v / 2) * 64 + (v & 1) * 8 : v * 32;
+                xv[buf][t][v] = (xok[t] && kbase + krel < p.K) ? *reinterpret_cast<const uint4 *>(xp[t] + xoff + krel * 2) : zero4;
+            }
     };
     auto compute = [&](auto bufc) {
         constexpr int buf = decltype(bufc)::value;

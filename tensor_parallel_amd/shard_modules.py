@@ -58,13 +58,15 @@ def _gated_mlp_forward(self, x: torch.Tensor) -> torch.Tensor:
 
 
 def is_gated_silu_mlp(module: nn.Module) -> bool:
-    parts = [getattr(module, n, None) for n in ("gate_proj", "up_proj", "down_proj")]
+    # only the module's own children count: a wrapper forwards attribute lookups to the module it wraps
+    parts = [module._modules.get(n) for n in ("gate_proj", "up_proj", "down_proj")]
     if not all(isinstance(p, nn.Linear) for p in parts):
         return False
     gate, up, _ = parts
     if gate.bias is not None or up.bias is not None or gate.weight.dtype not in (torch.bfloat16, torch.float16):
         return False
-    return _is_silu(getattr(module, "act_fn", None))
+    act = module._modules.get("act_fn", module.__dict__.get("act_fn"))
+    return _is_silu(act)
 
 
 def install_shard_kernels(shard: nn.Module) -> None:

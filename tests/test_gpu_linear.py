@@ -74,11 +74,27 @@ def test_gelu_epilogue_and_argument_errors():
         torch.testing.assert_close(got.float().cpu(), want, rtol=RTOL_HALF, atol=2e-2)
     with pytest.raises(ValueError):
         _native.linear(x.to(DEV), rnd((64, 60), 0, 0.1, torch.float16).to(DEV))  # K mismatch
-    with pytest.raises(ValueError):
-        _native.linear(rnd((4, 12), 0, 1, torch.float16).to(DEV), rnd((8, 12), 0, 1, torch.float16).to(DEV))  # K % 8
     with pytest.raises(TypeError):
         _native.linear(x.to(DEV), w.to(DEV).bfloat16())
     assert _native.linear(torch.empty(0, 64, dtype=torch.float16, device=DEV), w.to(DEV)).shape == (0, 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(4, 8, 12), (6, 256, 172), (70, 10, 36), (33, 130, 8), (5, 7, 3)])
+def test_unaligned_shapes_take_the_scalar_kernel(dtype, M, N, K):
+    """K not a multiple of 8 or N not a multiple of 4 (what an uneven split of a small model produces)."""
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.1, dtype), rnd((N,), 2, 0.1, dtype)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV))
+    torch.testing.assert_close(got.float().cpu(), F.linear(x.float(), w.float(), b.float()), rtol=RTOL_HALF, atol=2e-2)
+    w2 = rnd((N, K), 5, 0.1, dtype)
+    h = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=2e-2)
+
+
+def test_swiglu_fp32():
+    x, wg, wu = rnd((9, 40), 1, 1.0, torch.float32), rnd((24, 40), 0, 0.1, torch.float32), rnd((24, 40), 3, 0.1, torch.float32)
+    got = _native.swiglu_up(x.to(DEV), wg.to(DEV), wu.to(DEV)).cpu()
+    torch.testing.assert_close(got, ofw.gated_mlp_hidden(x, wg, wu), rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.parametrize("world", [2, 4])
