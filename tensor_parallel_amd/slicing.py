@@ -115,6 +115,7 @@ def apply_spec(t: torch.Tensor, spec: SliceSpec, device: Optional[torch.device] 
     if jobs:
         plan = _native.CopyPlan(jobs, src.device)
         plan.run()
+        torch.cuda.current_stream(src.device).synchronize()  # the plan's tile table must outlive the launch
         plan.close()
     return out
 
@@ -140,6 +141,7 @@ def concat_specs(parts: Sequence[torch.Tensor], specs: Sequence[SliceSpec]) -> t
     if jobs:
         plan = _native.CopyPlan(jobs, device)
         plan.run()
+        torch.cuda.current_stream(device).synchronize()  # the plan's tile table must outlive the launch
         plan.close()
     return out
 
