@@ -248,6 +248,18 @@ typedef __attribute__((address_space(3))) void lds_void;
 __device__ __forceinline__ void load16_to_lds(const void *g, void *lds_base) {
     __builtin_amdgcn_global_load_lds(g, (lds_void *)lds_base, 16, 0, 0);
 }
+// Fragment read that the compiler does not see as an LDS access. With ordinary loads it waits for every
+// in-flight global->LDS load before each LDS read (it cannot tell that they go to the other stage), which
+// serialises the pipeline; this way the waits are the counted ones written out in the main loop.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 lds_read16(uint32_t lds_addr) {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_addr));
+    return v;
+}
+__device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char *)p));
+}
 // All of this wavefront's loads and LDS accesses done, then the workgroup barrier. The memory clobber keeps
 // the compiler from moving LDS accesses across it.
 __device__ __forceinline__ void drain_and_barrier() {
@@ -345,24 +357,34 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
 
-    uint4 xf[2][TM], wf[2][TN];
-    auto read_frags = [&](auto bufc, const char *stage, int ks) {
+    static_assert(TM == 4 && TN == 2, "the counted waits below assume 6 fragment reads per K step");
+    u32x4 xf[2][TM], wf[2][TN];
+    const uint32_t smem_base = lds_addr_of(smem);
+    auto read_frags = [&](auto bufc, int stage_off, int ks) {
         constexpr int buf = decltype(bufc)::value;
 #pragma unroll
-        for (int t = 0; t < TM; ++t) xf[buf][t] = *reinterpret_cast<const uint4 *>(stage + x_rd[t] + ks_off[ks]);
+        for (int t = 0; t < TM; ++t) xf[buf][t] = lds_read16(smem_base + stage_off + x_rd[t] + ks_off[ks]);
 #pragma unroll
-        for (int t = 0; t < TN; ++t) wf[buf][t] = *reinterpret_cast<const uint4 *>(stage + w_rd[t] + ks_off[ks]);
+        for (int t = 0; t < TN; ++t) wf[buf][t] = lds_read16(smem_base + stage_off + w_rd[t] + ks_off[ks]);
     };
+    // LDS reads return in order: "at most N outstanding" means every read issued before the last N has landed.
+    // Naming the fragments as operands keeps the MFMAs that consume them behind the wait.
+#define TPAMD_WAIT_FRAGS(N, buf)                                                                                    \
+    asm volatile("s_waitcnt lgkmcnt(" #N ")"                                                                        \
+                 : "+v"(xf[buf][0]), "+v"(xf[buf][1]), "+v"(xf[buf][2]), "+v"(xf[buf][3]), "+v"(wf[buf][0]), "+v"(wf[buf][1]))
+#define TPAMD_DRAIN_BARRIER(buf)                                                                                    \
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"                                                       \
+                 : "+v"(xf[buf][0]), "+v"(xf[buf][1]), "+v"(xf[buf][2]), "+v"(xf[buf][3]), "+v"(wf[buf][0]), "+v"(wf[buf][1]) \
+                 :: "memory")
     auto mfmas = [&](auto bufc) {
         constexpr int buf = decltype(bufc)::value;
-        __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(1);  // the matrix pipe is the scarce unit: do not let the peer's loads cut in
 #pragma unroll
         for (int a = 0; a < TM; ++a)
 #pragma unroll
-            for (int b = 0; b < TN; ++b) acc[a][b] = mfma32<DT>(wf[buf][b], xf[buf][a], acc[a][b]);
+            for (int b = 0; b < TN; ++b)
+                acc[a][b] = mfma32<DT>(__builtin_bit_cast(uint4, wf[buf][b]), __builtin_bit_cast(uint4, xf[buf][a]), acc[a][b]);
         __builtin_amdgcn_s_setprio(0);
-        __builtin_amdgcn_sched_barrier(0);
     };
     using B0 = std::integral_constant<int, 0>;
     using B1 = std::integral_constant<int, 1>;
@@ -371,25 +393,30 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
     load_x(0, 0);
     load_w(0, 0);
     drain_and_barrier();
-    read_frags(B0{}, smem, 0);
+    read_frags(B0{}, 0, 0);
     for (int kt = 0; kt < KT; ++kt) {
         const bool more = kt + 1 < KT;
-        const char *stage = smem + (kt & 1) * STAGE;
-        const char *next = smem + ((kt + 1) & 1) * STAGE;
+        const int cur = (kt & 1) * STAGE, nxt = ((kt + 1) & 1) * STAGE;
         // K step 0: fragments of step 1 and half of the next tile's loads are issued, then step 0 multiplies
-        read_frags(B1{}, stage, 1);
+        read_frags(B1{}, cur, 1);
         if (more) load_x(kt + 1, (kt + 1) & 1);
+        TPAMD_WAIT_FRAGS(6, 0);
         mfmas(B0{});
-        read_frags(B0{}, stage, 2);
+        read_frags(B0{}, cur, 2);
         if (more) load_w(kt + 1, (kt + 1) & 1);
+        TPAMD_WAIT_FRAGS(6, 1);
         mfmas(B1{});
-        read_frags(B1{}, stage, 3);
+        read_frags(B1{}, cur, 3);
+        TPAMD_WAIT_FRAGS(6, 0);
         mfmas(B0{});
-        // every wavefront is done reading this tile and the next one has landed
-        drain_and_barrier();
-        if (more) read_frags(B0{}, next, 0);
+        // every wavefront is done reading this tile and the next one has landed; the MFMAs of step 3 then run
+        // under the first fragment reads of the next tile
+        TPAMD_DRAIN_BARRIER(1);
+        if (more) read_frags(B0{}, nxt, 0);
         mfmas(B1{});
     }
+#undef TPAMD_WAIT_FRAGS
+#undef TPAMD_DRAIN_BARRIER
 
     epilogue<DT, MODE, BM, BN, WAVES_M, WAVES_N>(p, acc, m0, n0, wm, wn, l32, lhi);
 }
@@ -525,7 +552,7 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     // 256x256 tiles once they fill the chip at least about once, else 128x128 tiles.
     const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
     if (big_tiles >= 200) {
-        if (p.K % 64 == 0) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
+        if (p.K % 64 == 0 && p.K >= 64) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
         return swiglu ? launch_gemm<DT, MODE_SWIGLU, 256, 256, 2, 4>(p, s) : launch_gemm<DT, MODE_LINEAR, 256, 256, 2, 4>(p, s);
     }
     return swiglu ? launch_gemm<DT, MODE_SWIGLU, 128, 128, 2, 2>(p, s) : launch_gemm<DT, MODE_LINEAR, 128, 128, 2, 2>(p, s);

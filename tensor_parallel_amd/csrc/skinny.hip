@@ -287,6 +287,177 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     }
 }
 
+// ---- M <= 4: row-streaming kernel --------------------------------------------------------------------
+// One wavefront owns one output column (linear: one row of w; gated pair: the gate row and the up row of that
+// column) over the whole of K. A load instruction covers 1 KiB of consecutive bytes of a row, K_BATCH of them
+// per row are in flight before anything is multiplied, x (at most 4 rows) sits in LDS, products go through
+// v_dot2 with fp32 accumulation, and 64 lane sums meet in a butterfly at the end.
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+template <int DT>
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    if constexpr (DT == TPAMD_BF16)
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+    else
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+template <int DT>
+__device__ __forceinline__ float dot8(uint4 w, uint4 x, float c) {
+    c = dot2<DT>(w.x, x.x, c);
+    c = dot2<DT>(w.y, x.y, c);
+    c = dot2<DT>(w.z, x.z, c);
+    return dot2<DT>(w.w, x.w, c);
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// GV_WAVES wavefronts per block; K_BATCH = loads per row in flight before anything is multiplied.
+template <int DT, bool W8, int MODE, int MR, int GV_WAVES, int K_BATCH>
+__global__ __launch_bounds__(GV_WAVES * 64) void gemv_kernel(SkinnyParams p) {
+    constexpr int GV_THREADS = GV_WAVES * 64;
+    constexpr int NMAT = MODE == SK_SWIGLU ? 2 : 1;
+    constexpr int STEP_K = W8 ? 1024 : 512;          // K elements per wavefront-wide 16-byte load of w
+    constexpr int XPL = W8 ? 2 : 1;                  // 16-byte pieces of x per lane per step
+
+    extern __shared__ __align__(16) char xs[];       // x[MR][K]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = blockIdx.x * GV_WAVES + wave;
+    const bool live = n < p.N;
+    const int row = live ? n : p.N - 1;
+    const int wbytes = W8 ? 1 : 2;
+    const int row_bytes = p.K * 2;
+    const int nsteps = (p.K + STEP_K - 1) / STEP_K;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+    const char *wp[NMAT];
+    wp[0] = p.w + static_cast<int64_t>(row) * p.ldw * wbytes + lane * 16;
+    if constexpr (NMAT == 2) wp[1] = p.w2 + static_cast<int64_t>(row) * p.ldw * wbytes + lane * 16;
+    const int lane_k = lane * (W8 ? 16 : 8);          // first K element of this lane inside a step
+
+    float acc[NMAT][MR];
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[a][m] = 0.f;
+
+    uint4 wv[K_BATCH][NMAT];
+    auto issue = [&](int s0) {
+#pragma unroll
+        for (int j = 0; j < K_BATCH; ++j) {
+            const int s = s0 + j;
+            const bool ok = s < nsteps && s * STEP_K + lane_k < p.K;
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a) {
+                // out-of-range pieces are fetched from the row's start (always valid) and zeroed: unconditional
+                // loads keep the whole batch in flight together
+                const uint4 raw = nt_load_u4(ok ? wp[a] + static_cast<int64_t>(s) * STEP_K * wbytes : wp[a] - lane * 16);
+                wv[j][a] = ok ? raw : zero4;
+            }
+        }
+    };
+
+    issue(0);
+    // stage x while the first batch is in flight
+    for (int m = 0; m < MR; ++m)
+        for (int i = tid; i * 8 < p.K; i += GV_THREADS)
+            *reinterpret_cast<uint4 *>(xs + m * row_bytes + i * 16) =
+                *reinterpret_cast<const uint4 *>(p.x + (static_cast<int64_t>(m) * p.ldx + i * 8) * 2);
+    __syncthreads();
+
+    for (int s0 = 0; s0 < nsteps; s0 += K_BATCH) {
+        if (s0 > 0) issue(s0);
+#pragma unroll
+        for (int j = 0; j < K_BATCH; ++j) {
+            const int k = (s0 + j) * STEP_K + lane_k;
+            if (s0 + j < nsteps && k < p.K) {
+#pragma unroll
+                for (int m = 0; m < MR; ++m) {
+                    uint4 xv[XPL];
+#pragma unroll
+                    for (int h = 0; h < XPL; ++h) xv[h] = *reinterpret_cast<const uint4 *>(xs + m * row_bytes + (k + h * 8) * 2);
+#pragma unroll
+                    for (int a = 0; a < NMAT; ++a) {
+                        if constexpr (W8) {
+                            uint4 w0, w1;
+                            cvt_i8x4<DT>(wv[j][a].x, w0.x, w0.y);
+                            cvt_i8x4<DT>(wv[j][a].y, w0.z, w0.w);
+                            cvt_i8x4<DT>(wv[j][a].z, w1.x, w1.y);
+                            cvt_i8x4<DT>(wv[j][a].w, w1.z, w1.w);
+                            acc[a][m] = dot8<DT>(w0, xv[0], acc[a][m]);
+                            acc[a][m] = dot8<DT>(w1, xv[XPL - 1], acc[a][m]);
+                        } else {
+                            acc[a][m] = dot8<DT>(wv[j][a], xv[0], acc[a][m]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    float acc_o[MR];
+    if constexpr (W8) {
+        // outlier columns: lanes stride over them
+        const uint16_t *xo = reinterpret_cast<const uint16_t *>(xs);
+        const uint16_t *wo = reinterpret_cast<const uint16_t *>(p.w_out);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc_o[m] = 0.f;
+        for (int o = lane; o < p.n_out; o += 64) {
+            const float wval = half_to_f32<DT>(wo[static_cast<int64_t>(row) * p.ld_wout + o]);
+            const int col = p.outlier_idx[o];
+#pragma unroll
+            for (int m = 0; m < MR; ++m) acc_o[m] = fmaf(half_to_f32<DT>(xo[m * p.K + col]), wval, acc_o[m]);
+        }
+    }
+
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        float s0 = wave_sum(acc[0][m]);
+        float s1 = 0.f;
+        if constexpr (NMAT == 2) s1 = wave_sum(acc[NMAT - 1][m]);
+        if constexpr (W8) s0 = s0 * p.scale[row] + wave_sum(acc_o[m]);
+        if (lane == 0 && live) {
+            uint16_t out;
+            if constexpr (MODE == SK_SWIGLU) {
+                const float g = half_to_f32<DT>(f32_to_half<DT>(s0));
+                const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
+                const float sg = half_to_f32<DT>(f32_to_half<DT>(silu_f32(g)));
+                out = f32_to_half<DT>(sg * u);
+            } else {
+                float v = s0;
+                if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
+                if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+                out = f32_to_half<DT>(v);
+            }
+            reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
+        }
+    }
+}
+
+constexpr int GEMV_MAX_M = 4;
+constexpr int64_t GEMV_MAX_X_BYTES = 64 * 1024;  // x[M][K] lives in LDS
+
+template <int DT, bool W8, int MODE>
+int launch_gemv(const SkinnyParams &p, hipStream_t s) {
+    // measured on the Llama-7B shard shapes: small blocks and short batches for the gated pair (two rows per
+    // wavefront), whole rows in flight for a single matrix
+    constexpr int GV_WAVES = MODE == SK_SWIGLU ? 4 : 8;
+    constexpr int GV_THREADS = GV_WAVES * 64;
+    constexpr int KB = MODE == SK_SWIGLU ? 4 : 12;
+    const unsigned grid = static_cast<unsigned>((p.N + GV_WAVES - 1) / GV_WAVES);
+    const size_t lds = static_cast<size_t>(p.M) * p.K * 2;
+    switch (p.M) {
+        case 1: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 1, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
+        case 2: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 2, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
+        case 3: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 3, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
+        default: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 4, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
+    }
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 template <int DT, bool W8, int MODE>
 int launch_skinny(const SkinnyParams &p, hipStream_t s) {
     const unsigned grid = static_cast<unsigned>((p.N + 15) / 16);
@@ -318,6 +489,12 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ld_wout = ld_wout;
     p.act = act;
     const bool bf = dtype == TPAMD_BF16;
+    static const int gemv_max_m = getenv("TPAMD_GEMV_MAX_M") ? atoi(getenv("TPAMD_GEMV_MAX_M")) : GEMV_MAX_M;
+    if (M <= gemv_max_m && M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
+        if (w8) return bf ? launch_gemv<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, true, SK_LINEAR>(p, s);
+        if (swiglu) return bf ? launch_gemv<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_gemv<TPAMD_F16, false, SK_SWIGLU>(p, s);
+        return bf ? launch_gemv<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, false, SK_LINEAR>(p, s);
+    }
     if (w8) return bf ? launch_skinny<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_skinny<TPAMD_F16, true, SK_LINEAR>(p, s);
     if (swiglu) return bf ? launch_skinny<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_skinny<TPAMD_F16, false, SK_SWIGLU>(p, s);
     return bf ? launch_skinny<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_skinny<TPAMD_F16, false, SK_LINEAR>(p, s);

@@ -10,7 +10,7 @@ namespace tpamd {
 
 namespace {
 
-constexpr uint32_t TILE_UNITS = 4096;  // vector units per tile (64 KiB when units are 16 bytes)
+constexpr uint32_t MAX_TILE_UNITS = 4096;  // vector units per tile (64 KiB when units are 16 bytes)
 constexpr int COPY_THREADS = 256;
 
 struct alignas(16) Tile {
@@ -132,6 +132,11 @@ extern "C" int tpamd_copy_plan_create(const tpamd_copy_job *jobs, size_t n_jobs,
     *plan_out = nullptr;
     std::vector<Tile> tiles;
     uint64_t bytes = 0;
+    uint32_t TILE_UNITS = MAX_TILE_UNITS;
+    if (const char *e = getenv("TPAMD_COPY_TILE_UNITS")) {  // tuning knob
+        const int v = atoi(e);
+        if (v >= 256 && v <= static_cast<int>(MAX_TILE_UNITS)) TILE_UNITS = static_cast<uint32_t>(v);
+    }
     try {
         for (size_t ji = 0; ji < n_jobs; ++ji) {
             const tpamd_copy_job &j = jobs[ji];
