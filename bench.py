@@ -20,6 +20,10 @@ if str(ROOT) not in sys.path:
 D_MODEL, FFN_SHARD = 4096, 5504
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
+# Fabric bytes per launch of the fused gate/up GEMM at M = 4096, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
+# each scaled by what the same counter reads for the slicing kernel's known 13.476 GB (factors 1.994 and 1.000):
+# profiles/pmc_fetch_write_bench_kernels.txt. A counter reading cannot be taken inside this script.
+MEASURED_TRAFFIC_BYTES_M4096 = 639.6e6
 
 
 def cpu_baseline(seconds_budget: float = 15.0) -> dict:
@@ -120,7 +124,8 @@ def main() -> int:
     if mfma_bound:
         achieved = up_flops / (up_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_M4096 if M == 4096 else None,
+                    "traffic_unit": "bytes per launch (L2<->fabric, rocprofv3 --pmc; algorithmic 168.8e6)",
                     "kernel": "gemm_direct_kernel<bf16, swiglu> (tpamd_swiglu_up)", "avg_launch_ms": up_ms,
                     "algorithmic_flops_per_launch": up_flops}
     else:
