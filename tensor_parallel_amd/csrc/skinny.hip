@@ -1,12 +1,12 @@
 // Rank-shard Linear for decode-sized M (M <= 64): weight streaming, HBM-bound.
 //
-// A block owns 16 output columns (16 rows of w; for the SiLU-gated pair 16 gate rows + 16 up rows) and
-// splits K over its wavefronts in chunks of 256 bytes of every w row. A chunk is fetched by 4 wavefront-wide
-// 16-byte loads; in each of them the 4 lanes that share a row read 64 contiguous bytes, so every load
-// instruction touches 16 whole 64-byte sectors. The loaded registers are MFMA operands as they are:
-// v_mfma_f32_16x16x32 does both the multiply and the reduction over K, so no cross-lane shuffles are
-// needed. Partial sums of the wavefronts meet in LDS; the epilogue applies scale, outliers, bias,
-// activation and stores 16 consecutive columns per row.
+// Two kernels:
+//   skinny_kernel (4 <= M <= 32, int8 weights up to 64): a block owns 16 output columns (16 rows of w; for the
+//     SiLU-gated pair 16 gate rows + 16 up rows) and splits K over its wavefronts in chunks of 256 bytes of every
+//     w row. v_mfma_f32_16x16x32 does both the multiply and the reduction over K, so no cross-lane shuffles are
+//     needed. Partial sums of the wavefronts meet in LDS; the epilogue applies scale, outliers, bias, activation
+//     and stores 16 consecutive columns per row.
+//   gemv_kernel (M <= 3): one wavefront per output column, v_dot2 products, x in LDS.
 //
 // The weight is either the activation dtype (bf16/f16) or int8 (weight-only quantisation: converted to
 // the activation dtype in registers, exact for |q| <= 128).
@@ -73,6 +73,12 @@ __device__ __forceinline__ void cvt_i8x4(uint32_t q, uint32_t &lo, uint32_t &hi)
 }
 
 // W8 = weight is int8. MT = number of 16-row tiles of x (M <= 16*MT). MODE = SK_LINEAR / SK_SWIGLU.
+//
+// Fetching. The MFMA row operand wants lane l to hold 16 bytes of row l%16 at K slot l/16; loading it that way
+// makes every load instruction touch 16 rows x 64 bytes, and the pace of such a kernel is set by the number of
+// half-line requests, not by bytes (measured: 1.5-2x slower). So a load instruction here fetches 8 rows x 128
+// contiguous bytes (whole cache lines), and the loaded registers go through a wavefront-private LDS tile:
+// written in fetch order, read back in MFMA operand order. x takes the same route when the weights are 16-bit.
 template <int DT, bool W8, int MT, int MODE>
 __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     constexpr int NMAT = MODE == SK_SWIGLU ? 2 : 1;
@@ -82,7 +88,10 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     constexpr int XV = LANE_K / 8;            // 16-byte loads of x per lane per chunk per m-tile
     constexpr int WK = W8 ? 16 : 8;           // K elements in one 16-byte load of w
 
+    constexpr int TROW = 272;                 // staged row pitch: 256 bytes + 16 pad
+    constexpr bool XT = !W8;                  // x goes through the LDS tile too
     __shared__ float red[SK_WAVES][NMAT][MT][4][64];
+    __shared__ __align__(16) char stage_all[SK_WAVES][16 * TROW];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
@@ -91,10 +100,21 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     int wrow = n0 + lr;
     wrow = wrow < p.N ? wrow : p.N - 1;
     const int wbytes = W8 ? 1 : 2;
-    const char *wp[NMAT];
-    // load v of a chunk: this lane's 16 bytes sit at byte lg*16 + v*64 of the chunk's 256 bytes of row wrow
-    wp[0] = p.w + static_cast<int64_t>(wrow) * p.ldw * wbytes + lg * 16;
-    if constexpr (NMAT == 2) wp[1] = p.w2 + static_cast<int64_t>(wrow) * p.ldw * wbytes + lg * 16;
+    const char *wp[2];
+    const char *wp2[2];
+    (void)wp2;
+    // fetch order: load i of a chunk covers rows (lane/8) + 8*(i&1), bytes (i/2)*128 + (lane%8)*16 of the chunk's 256
+    const int crow = lane >> 3, cpiece = lane & 7;
+    char *stage = stage_all[wave];
+    const int st_wr = crow * TROW + cpiece * 16;   // + (i&1)*8*TROW + (i/2)*128
+    const int st_rd = lr * TROW + lg * 16;         // + v*64
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        int r = n0 + crow + 8 * h;
+        r = r < p.N ? r : p.N - 1;
+        wp[h] = p.w + static_cast<int64_t>(r) * p.ldw * wbytes + cpiece * 16;
+        if constexpr (NMAT == 2) wp2[h] = p.w2 + static_cast<int64_t>(r) * p.ldw * wbytes + cpiece * 16;
+    }
     const char *xp[MT];
     bool xok[MT];
 #pragma unroll
@@ -103,6 +123,16 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
         xok[t] = m < p.M;
         xp[t] = p.x + (static_cast<int64_t>(xok[t] ? m : 0) * p.ldx + lg * WK) * 2;
     }
+    const char *xpc[MT][2];
+    bool xokc[MT][2];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int m = t * 16 + crow + 8 * h;
+            xokc[t][h] = m < p.M;
+            xpc[t][h] = p.x + static_cast<int64_t>(xokc[t][h] ? m : 0) * p.ldx * 2 + cpiece * 16;
+        }
 
     f32x4 acc[NMAT][MT];
 #pragma unroll
@@ -120,20 +150,44 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     uint4 xv[XPRE ? 2 : 1][MT][XV];
     auto load_w = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
-        const int kbase = c * CHUNK_K + lg * WK;  // first K element of this lane's load 0
         const int64_t off = static_cast<int64_t>(c) * CHUNK_K * wbytes;
 #pragma unroll
         for (int a = 0; a < NMAT; ++a)
 #pragma unroll
-            for (int v = 0; v < WV; ++v) {
-                const int k = kbase + v * 4 * WK;
-                wv[buf][a][v] = k < p.K ? nt_load_u4(wp[a] + off + v * 64) : zero4;
+            for (int i = 0; i < WV; ++i) {
+                const int byte = (i >> 1) * 128 + cpiece * 16;            // inside the chunk's 256 bytes of the row
+                const bool ok = c * CHUNK_K + byte / wbytes < p.K;
+                const char *base = a == 0 ? wp[i & 1] : wp2[i & 1];
+                const uint4 raw = nt_load_u4(ok ? base + off + (i >> 1) * 128 : base - cpiece * 16);  // unconditional
+                wv[buf][a][i] = ok ? raw : zero4;
             }
+    };
+    // registers in fetch order -> registers in MFMA operand order, through this wavefront's LDS tile
+    auto transpose = [&](uint4 (&r)[WV]) {
+#pragma unroll
+        for (int i = 0; i < WV; ++i) *reinterpret_cast<uint4 *>(stage + st_wr + (i & 1) * 8 * TROW + (i >> 1) * 128) = r[i];
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int v = 0; v < WV; ++v) r[v] = *reinterpret_cast<const uint4 *>(stage + st_rd + v * 64);
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
     };
     auto load_x = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
         const int kbase = c * CHUNK_K + lg * WK;
         const int64_t xoff = static_cast<int64_t>(c) * CHUNK_K * 2;
+        if constexpr (XT) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int i = 0; i < XV; ++i) {
+                    const int byte = (i >> 1) * 128 + cpiece * 16;
+                    const bool ok = xokc[t][i & 1] && c * CHUNK_K + byte / 2 < p.K;
+                    xv[buf][t][i] = ok ? *reinterpret_cast<const uint4 *>(xpc[t][i & 1] + xoff + (i >> 1) * 128) : zero4;
+                }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -146,6 +200,12 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     auto compute = [&](auto bufc) {
         constexpr int buf = decltype(bufc)::value;
         constexpr int xb = XPRE ? buf : 0;
+#pragma unroll
+        for (int a = 0; a < NMAT; ++a) transpose(wv[buf][a]);
+        if constexpr (XT) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) transpose(xv[xb][t]);
+        }
 #pragma unroll
         for (int a = 0; a < NMAT; ++a) {
             if constexpr (W8) {
@@ -436,7 +496,7 @@ __global__ __launch_bounds__(GV_WAVES * 64) void gemv_kernel(SkinnyParams p) {
     }
 }
 
-constexpr int GEMV_MAX_M = 4;
+constexpr int GEMV_MAX_M = 3;  // from 4 rows on the MFMA kernel is faster
 constexpr int64_t GEMV_MAX_X_BYTES = 64 * 1024;  // x[M][K] lives in LDS
 
 template <int DT, bool W8, int MODE>
@@ -451,8 +511,7 @@ int launch_gemv(const SkinnyParams &p, hipStream_t s) {
     switch (p.M) {
         case 1: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 1, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
         case 2: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 2, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
-        case 3: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 3, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
-        default: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 4, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
+        default: hipLaunchKernelGGL((gemv_kernel<DT, W8, MODE, 3, GV_WAVES, KB>), dim3(grid), dim3(GV_THREADS), lds, s, p); break;
     }
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
@@ -489,8 +548,7 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ld_wout = ld_wout;
     p.act = act;
     const bool bf = dtype == TPAMD_BF16;
-    static const int gemv_max_m = getenv("TPAMD_GEMV_MAX_M") ? atoi(getenv("TPAMD_GEMV_MAX_M")) : GEMV_MAX_M;
-    if (M <= gemv_max_m && M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
+    if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
         if (w8) return bf ? launch_gemv<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, true, SK_LINEAR>(p, s);
         if (swiglu) return bf ? launch_gemv<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_gemv<TPAMD_F16, false, SK_SWIGLU>(p, s);
         return bf ? launch_gemv<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, false, SK_LINEAR>(p, s);
