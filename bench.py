@@ -211,6 +211,8 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
         except Exception as e:  # noqa: BLE001 - the eager figure stands on its own
             entry["graph"] = {"error": str(e)[:200]}
         extra[f"decode_m{m}"] = entry
+    extra["w8_decode_m1"] = w8_decode(torch, _native, dev)
+
     from types import SimpleNamespace
 
     from tensor_parallel_amd.slicing import BatchSlicer
@@ -240,6 +242,34 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
                            "GBps": moved / us / 1e3, "hbm_frac": moved / us / 1e3 / PEAK_HBM_GBS}
     batch.close()
     return extra
+
+
+def w8_decode(torch, _native, dev) -> dict:
+    """BASELINE config 5 at batch 1: int8 weight-only rank-0 shard of a Falcon-40B-shape MLP (up [16384 x 8192] + GELU,
+    down [8192 x 16384], per-row scales, 41 / 82 outlier columns in fp16), fp16 activations. HBM-bound."""
+    d, f, n_sets = 8192, 16384, 3
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def make(n, k, n_out):
+        wq = torch.randint(-127, 128, (n, k), device=dev, dtype=torch.int8, generator=g)
+        scale = torch.rand(n, device=dev, generator=g) * 1e-3
+        idx = torch.randperm(k, device=dev, generator=g)[:n_out].sort().values.int()
+        w_out = (torch.randn(n, n_out, device=dev, generator=g) * 0.02).half()
+        return wq, scale, idx, w_out
+
+    ups = [make(f, d, 41) for _ in range(n_sets)]
+    downs = [make(d, f, 82) for _ in range(n_sets)]
+    x = torch.randn(1, d, device=dev, generator=g).half()
+
+    def fn(i):
+        u, dn = ups[i % n_sets], downs[i % n_sets]
+        h = _native.linear_w8(x, u[0], u[1], u[2], u[3], act=_native.ACT_GELU)
+        return _native.linear_w8(h, dn[0], dn[1], dn[2], dn[3])
+
+    us = _time_us(torch, fn, 10, 100)
+    by = 2.0 * f * d + (f * 41 + d * 82) * 2.0 + (f + d) * 4.0
+    return {"us_per_step": us, "tokens_per_s": 1e6 / us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
+            "algorithmic_bytes": by, "launch": "eager"}
 
 
 if __name__ == "__main__":

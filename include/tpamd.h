@@ -99,6 +99,11 @@ int tpamd_copy_plan_run(const tpamd_copy_plan *plan, void *stream);
 uint64_t tpamd_copy_plan_bytes(const tpamd_copy_plan *plan);
 int tpamd_copy_plan_destroy(tpamd_copy_plan *plan);
 
+/* The same copies without a plan: up to 16 jobs are passed to the kernel by value, nothing is allocated and
+ * nothing has to be kept alive afterwards. For single tensors: one state action on one tensor, the undo of
+ * one rule, one "gather d" of W column-parallel outputs. */
+int tpamd_copy_jobs_run(const tpamd_copy_job *jobs, size_t n_jobs, void *stream);
+
 /* Scale state action: out[i] = in[i] / world_size in the tensor's dtype
  * (Scale.__call__, src/tensor_parallel/state_actions.py:59-60). For bf16/f16 the quotient of the
  * fp32-widened value is rounded to nearest even, as torch does. `mul != 0` multiplies instead

@@ -22,6 +22,7 @@ EXPORTS = (
     "tpamd_copy_plan_run",
     "tpamd_copy_plan_bytes",
     "tpamd_copy_plan_destroy",
+    "tpamd_copy_jobs_run",
     "tpamd_scale",
     "tpamd_reduce_partials",
     "tpamd_linear",
@@ -72,6 +73,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_copy_plan_bytes.argtypes = [vp]
     lib.tpamd_copy_plan_destroy.restype = ci
     lib.tpamd_copy_plan_destroy.argtypes = [vp]
+    lib.tpamd_copy_jobs_run.restype = ci
+    lib.tpamd_copy_jobs_run.argtypes = [c.POINTER(CopyJob), c.c_size_t, vp]
     lib.tpamd_scale.restype = ci
     lib.tpamd_scale.argtypes = [vp, vp, u64, ci, ci, ci, vp]
     lib.tpamd_reduce_partials.restype = ci
@@ -181,6 +184,25 @@ class CopyPlan:
             self.close()
         except Exception:
             pass
+
+
+SMALL_COPY_MAX_JOBS = 16
+
+
+def run_copy_jobs(jobs: Sequence[tuple], device: torch.device) -> None:
+    """Launch up to 16 copy jobs without building a plan (nothing allocated, nothing to keep alive); more jobs go
+    through a plan, which is destroyed once its launch has finished."""
+    if not jobs:
+        return
+    with torch.cuda.device(device):
+        if len(jobs) <= SMALL_COPY_MAX_JOBS:
+            arr = (CopyJob * len(jobs))(*[CopyJob(*j) for j in jobs])
+            _check(lib().tpamd_copy_jobs_run(arr, len(jobs), ctypes.c_void_p(current_stream_ptr(device))), "tpamd_copy_jobs_run")
+            return
+    plan = CopyPlan(jobs, device)
+    plan.run()
+    torch.cuda.current_stream(device).synchronize()  # the plan's tile table must outlive the launch
+    plan.close()
 
 
 def scale(inp: torch.Tensor, world_size: int, multiply: bool = False) -> torch.Tensor:

@@ -252,9 +252,11 @@ __device__ __forceinline__ void load16_to_lds(const void *g, void *lds_base) {
 // in-flight global->LDS load before each LDS read (it cannot tell that they go to the other stage), which
 // serialises the pipeline; this way the waits are the counted ones written out in the main loop.
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <int OFFSET>
 __device__ __forceinline__ u32x4 lds_read16(uint32_t lds_addr) {
+    static_assert(OFFSET >= 0 && OFFSET < 65536, "ds offset field is 16 bits");
     u32x4 v;
-    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_addr));
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFFSET));
     return v;
 }
 __device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
@@ -290,60 +292,57 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    // ---- global -> LDS: lane (rb, slot) of a load fetches chunk slot ^ rb of row rb of its block
+    // ---- global -> LDS: lane (rb, slot) of a load fetches chunk slot ^ rb of row rb of its block.
+    // Addresses are a wavefront-uniform base (tile origin + K offset, advanced on the scalar unit) plus a 32-bit
+    // per-lane offset computed once, so the loop spends no vector instructions on address arithmetic; the LDS
+    // destination of each load is uniform too.
     const int rb = lane >> 3, slot = lane & 7;
     const int lchunk = slot ^ rb;
-    const char *xg[XB];
-    const char *wg[WB];
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
+    const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
+    const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : nullptr;
+    uint32_t x_off[XB], w_off[WB];
 #pragma unroll
     for (int i = 0; i < XB; ++i) {
-        int r = m0 + (wave + i * NW) * 8 + rb;
-        r = r < p.M ? r : p.M - 1;
-        xg[i] = p.x + (static_cast<int64_t>(r) * p.ldx + lchunk * 8) * 2;
+        int r = (wave_s + i * NW) * 8 + rb;
+        r = m0 + r < p.M ? r : p.M - 1 - m0;  // clamp to the last valid row of x
+        x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16;
     }
 #pragma unroll
     for (int i = 0; i < WB; ++i) {
-        const int tr = (wave + i * NW) * 8 + rb;
-        const char *base = p.w;
-        int r;
-        if constexpr (MODE == MODE_SWIGLU) {
-            base = tr < BN / 2 ? p.w : p.w2;
-            r = n0 + (tr < BN / 2 ? tr : tr - BN / 2);
-        } else {
-            r = n0 + tr;
-        }
-        r = r < p.N ? r : p.N - 1;
-        wg[i] = base + (static_cast<int64_t>(r) * p.ldw + lchunk * 8) * 2;
+        int tr = (wave_s + i * NW) * 8 + rb;
+        if constexpr (MODE == MODE_SWIGLU) tr = tr < BN / 2 ? tr : tr - BN / 2;  // gate rows, then up rows
+        tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
+        w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
     }
     auto load_x = [&](int kt, int stage) {
-        const int64_t off = static_cast<int64_t>(kt) * BK * 2;
+        const char *base = x_base + static_cast<int64_t>(kt) * BK * 2;
         char *xs = smem + stage * STAGE;
 #pragma unroll
-        for (int i = 0; i < XB; ++i) load16_to_lds(xg[i] + off, xs + (wave + i * NW) * BLK);
+        for (int i = 0; i < XB; ++i) load16_to_lds(base + x_off[i], xs + (wave_s + i * NW) * BLK);
     };
     auto load_w = [&](int kt, int stage) {
-        const int64_t off = static_cast<int64_t>(kt) * BK * 2;
         char *ws = smem + stage * STAGE + XREG;
 #pragma unroll
-        for (int i = 0; i < WB; ++i) load16_to_lds(wg[i] + off, ws + (wave + i * NW) * BLK);
+        for (int i = 0; i < WB; ++i) {
+            const char *base = w_base;
+            if constexpr (MODE == MODE_SWIGLU) base = (wave_s + i * NW) * 8 < BN / 2 ? w_base : w2_base;  // uniform per load
+            load16_to_lds(base + static_cast<int64_t>(kt) * BK * 2 + w_off[i], ws + (wave_s + i * NW) * BLK);
+        }
     };
 
-    // ---- LDS -> MFMA operand addresses
-    int x_rd[TM], w_rd[TN];
-#pragma unroll
-    for (int t = 0; t < TM; ++t) {
-        const int r = wm * (BM / WAVES_M) + t * 32 + l32;
-        x_rd[t] = (r >> 3) * BLK + (r & 7) * 128;
-    }
-#pragma unroll
-    for (int t = 0; t < TN; ++t) {
-        int row;
-        if constexpr (MODE == MODE_SWIGLU)
-            row = (t / (TN / 2)) * (BN / 2) + wn * (BN / 2 / WAVES_N) + (t % (TN / 2)) * 32;
-        else
-            row = wn * (BN / WAVES_N) + t * 32;
-        const int r = row + l32;
-        w_rd[t] = XREG + (r >> 3) * BLK + (r & 7) * 128;
+    // ---- LDS -> MFMA operand addresses: one per-lane base for x and one for w; the MFMA tiles of a wavefront are a
+    // compile-time number of 1152-byte blocks apart, which goes into the instruction's offset field
+    constexpr int X_TILE_STEP = 4 * BLK;                                         // 32 rows
+    constexpr int W_TILE_STEP = (MODE == MODE_SWIGLU ? (BN / 2) / 8 : 4) * BLK;  // swiglu: gate tile -> up tile
+    static_assert(MODE == MODE_LINEAR || TN == 2, "swiglu operand addressing assumes one gate and one up tile per wavefront");
+    int x_rd0, w_rd0;
+    {
+        const int r = wm * (BM / WAVES_M) + l32;
+        x_rd0 = (r >> 3) * BLK + (r & 7) * 128;
+        const int row = (MODE == MODE_SWIGLU ? wn * (BN / 2 / WAVES_N) : wn * (BN / WAVES_N)) + l32;
+        w_rd0 = XREG + (row >> 3) * BLK + (row & 7) * 128;
     }
     int ks_off[BK / 16];
 #pragma unroll
@@ -362,10 +361,14 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
     const uint32_t smem_base = lds_addr_of(smem);
     auto read_frags = [&](auto bufc, int stage_off, int ks) {
         constexpr int buf = decltype(bufc)::value;
-#pragma unroll
-        for (int t = 0; t < TM; ++t) xf[buf][t] = lds_read16(smem_base + stage_off + x_rd[t] + ks_off[ks]);
-#pragma unroll
-        for (int t = 0; t < TN; ++t) wf[buf][t] = lds_read16(smem_base + stage_off + w_rd[t] + ks_off[ks]);
+        const uint32_t xa = smem_base + stage_off + x_rd0 + ks_off[ks];
+        const uint32_t wa = smem_base + stage_off + w_rd0 + ks_off[ks];
+        xf[buf][0] = lds_read16<0>(xa);
+        xf[buf][1] = lds_read16<X_TILE_STEP>(xa);
+        xf[buf][2] = lds_read16<2 * X_TILE_STEP>(xa);
+        xf[buf][3] = lds_read16<3 * X_TILE_STEP>(xa);
+        wf[buf][0] = lds_read16<0>(wa);
+        wf[buf][1] = lds_read16<W_TILE_STEP>(wa);
     };
     // LDS reads return in order: "at most N outstanding" means every read issued before the last N has landed.
     // Naming the fragments as operands keeps the MFMAs that consume them behind the wait.

@@ -88,6 +88,65 @@ __global__ __launch_bounds__(COPY_THREADS) void copy_tiles_kernel(const Tile *__
     }
 }
 
+// ---- small batches: up to SMALL_MAX_JOBS jobs travel in the kernel arguments, tiles are derived on the device ----
+constexpr int SMALL_MAX_JOBS = 16;
+struct SmallJob {
+    const char *src;
+    char *dst;
+    uint64_t rows, src_pitch, dst_pitch;
+    uint64_t upr_full;    // row length in units of `vec` bytes
+    uint32_t vec;
+    uint32_t kind;        // 0 contiguous, 1 long rows, 2 short rows
+    uint32_t tiles_per_row_or_rows_per_tile;
+    uint32_t tile_begin;  // first global tile index of this job
+};
+struct SmallBatch {
+    SmallJob job[SMALL_MAX_JOBS];
+    uint32_t n_jobs, n_tiles;
+};
+
+__global__ __launch_bounds__(COPY_THREADS) void copy_small_kernel(SmallBatch b) {
+    const int tid = threadIdx.x;
+    for (uint32_t ti = blockIdx.x; ti < b.n_tiles; ti += gridDim.x) {
+        uint32_t ji = 0;
+        while (ji + 1 < b.n_jobs && b.job[ji + 1].tile_begin <= ti) ++ji;  // block-uniform
+        const SmallJob &j = b.job[ji];
+        const uint64_t local = ti - j.tile_begin;
+        Tile t{};
+        t.vec = j.vec;
+        if (j.kind == 0) {
+            const uint64_t units = j.rows * j.upr_full, u = local * MAX_TILE_UNITS;
+            t.src = j.src + u * j.vec;
+            t.dst = j.dst + u * j.vec;
+            t.rows = 1;
+            t.units_per_row = static_cast<uint32_t>(units - u < MAX_TILE_UNITS ? units - u : MAX_TILE_UNITS);
+        } else if (j.kind == 1) {
+            const uint64_t r = local / j.tiles_per_row_or_rows_per_tile, u = (local % j.tiles_per_row_or_rows_per_tile) * MAX_TILE_UNITS;
+            t.src = j.src + r * j.src_pitch + u * j.vec;
+            t.dst = j.dst + r * j.dst_pitch + u * j.vec;
+            t.rows = 1;
+            t.units_per_row = static_cast<uint32_t>(j.upr_full - u < MAX_TILE_UNITS ? j.upr_full - u : MAX_TILE_UNITS);
+        } else {
+            const uint64_t rpt = j.tiles_per_row_or_rows_per_tile, r = local * rpt;
+            const uint32_t upr = static_cast<uint32_t>(j.upr_full);
+            t.src = j.src + r * j.src_pitch;
+            t.dst = j.dst + r * j.dst_pitch;
+            t.src_pitch = j.src_pitch;
+            t.dst_pitch = j.dst_pitch;
+            t.rows = static_cast<uint32_t>(j.rows - r < rpt ? j.rows - r : rpt);
+            t.units_per_row = upr;
+            t.magic = upr == 1 ? 0u : static_cast<uint32_t>(((1ull << 32) + upr - 1) / upr);
+        }
+        switch (t.vec) {
+            case 16: move_tile<v4u>(t, tid); break;
+            case 8: move_tile<v2u>(t, tid); break;
+            case 4: move_tile<uint32_t>(t, tid); break;
+            case 2: move_tile<uint16_t>(t, tid); break;
+            default: move_tile<uint8_t>(t, tid); break;
+        }
+    }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void scale_kernel(const void *__restrict__ in, void *__restrict__ out, uint64_t n,
                                                     float w, int mul) {
@@ -238,6 +297,56 @@ extern "C" int tpamd_copy_plan_run(const tpamd_copy_plan *plan, void *stream) {
                   dev);
     hipLaunchKernelGGL(copy_tiles_kernel, dim3(plan->grid), dim3(COPY_THREADS), 0, static_cast<hipStream_t>(stream),
                        plan->tiles_dev, plan->n_tiles);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+extern "C" int tpamd_copy_jobs_run(const tpamd_copy_job *jobs, size_t n_jobs, void *stream) {
+    TPAMD_REQUIRE(n_jobs <= static_cast<size_t>(SMALL_MAX_JOBS), "tpamd_copy_jobs_run: at most %d jobs (got %zu); use a copy plan",
+                  SMALL_MAX_JOBS, n_jobs);
+    TPAMD_REQUIRE(jobs != nullptr || n_jobs == 0, "tpamd_copy_jobs_run: jobs is NULL");
+    SmallBatch b{};
+    uint64_t tiles = 0;
+    for (size_t ji = 0; ji < n_jobs; ++ji) {
+        const tpamd_copy_job &j = jobs[ji];
+        if (j.rows == 0 || j.row_bytes == 0) continue;
+        TPAMD_REQUIRE(j.src_dev != nullptr && j.dst_dev != nullptr, "copy job %zu: null pointer", ji);
+        TPAMD_REQUIRE(j.rows == 1 || (j.src_pitch >= j.row_bytes && j.dst_pitch >= j.row_bytes),
+                      "copy job %zu: pitch smaller than row_bytes", ji);
+        SmallJob &d = b.job[b.n_jobs++];
+        d.src = static_cast<const char *>(j.src_dev);
+        d.dst = static_cast<char *>(j.dst_dev);
+        d.rows = j.rows;
+        d.src_pitch = j.src_pitch;
+        d.dst_pitch = j.dst_pitch;
+        d.vec = pick_vec(j);
+        d.upr_full = j.row_bytes / d.vec;
+        d.tile_begin = static_cast<uint32_t>(tiles);
+        const bool contiguous = (j.rows == 1) || (j.src_pitch == j.row_bytes && j.dst_pitch == j.row_bytes);
+        uint64_t nt;
+        if (contiguous) {
+            d.kind = 0;
+            nt = (j.rows * d.upr_full + MAX_TILE_UNITS - 1) / MAX_TILE_UNITS;
+        } else if (d.upr_full >= MAX_TILE_UNITS) {
+            d.kind = 1;
+            d.tiles_per_row_or_rows_per_tile = static_cast<uint32_t>((d.upr_full + MAX_TILE_UNITS - 1) / MAX_TILE_UNITS);
+            nt = j.rows * d.tiles_per_row_or_rows_per_tile;
+        } else {
+            d.kind = 2;
+            d.tiles_per_row_or_rows_per_tile = static_cast<uint32_t>(MAX_TILE_UNITS / d.upr_full);
+            nt = (j.rows + d.tiles_per_row_or_rows_per_tile - 1) / d.tiles_per_row_or_rows_per_tile;
+        }
+        tiles += nt;
+        TPAMD_REQUIRE(tiles < 0xffffff00ull, "tpamd_copy_jobs_run: too many tiles");
+    }
+    if (tiles == 0) return TPAMD_OK;
+    b.n_tiles = static_cast<uint32_t>(tiles);
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const uint64_t cap = static_cast<uint64_t>(cus) * 8;
+    hipLaunchKernelGGL(copy_small_kernel, dim3(static_cast<unsigned>(tiles < cap ? tiles : cap)), dim3(COPY_THREADS), 0,
+                       static_cast<hipStream_t>(stream), b);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }

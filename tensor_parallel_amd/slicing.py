@@ -112,11 +112,7 @@ def apply_spec(t: torch.Tensor, spec: SliceSpec, device: Optional[torch.device] 
     src = _device_source(t, device)
     out = torch.empty(spec.out_shape, dtype=t.dtype, device=src.device)
     jobs = copy_jobs(spec, t.element_size(), src.data_ptr(), out.data_ptr())
-    if jobs:
-        plan = _native.CopyPlan(jobs, src.device)
-        plan.run()
-        torch.cuda.current_stream(src.device).synchronize()  # the plan's tile table must outlive the launch
-        plan.close()
+    _native.run_copy_jobs(jobs, src.device)
     return out
 
 
@@ -138,11 +134,7 @@ def concat_specs(parts: Sequence[torch.Tensor], specs: Sequence[SliceSpec]) -> t
         if p.device != device or p.dtype != first.dtype:
             raise ValueError("concat_specs: parts must share device and dtype")
         jobs += copy_jobs(spec, p.element_size(), out.data_ptr(), p.data_ptr(), scatter=True)
-    if jobs:
-        plan = _native.CopyPlan(jobs, device)
-        plan.run()
-        torch.cuda.current_stream(device).synchronize()  # the plan's tile table must outlive the launch
-        plan.close()
+    _native.run_copy_jobs(jobs, device)
     return out
 
 

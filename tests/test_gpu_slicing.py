@@ -215,3 +215,51 @@ def test_llama_7b_layer_full_size_round_trip():
             total = sum(int(s.view(torch.int16).to(torch.int64).sum()) for s in shards)
             assert total == int(full.view(torch.int16).to(torch.int64).sum())
         assert out[f"module_shards.{world - 1}.{names['model.layers.0.mlp.down_proj.weight']}"].shape == (4096, 11008 // world)
+
+
+@pytest.mark.parametrize("rows,row_bytes,src_pitch,dst_pitch", [
+    (1, 1 << 20, 0, 0),            # contiguous, many tiles
+    (3, 70001, 70001, 70001),      # contiguous by pitch, odd byte count (1-byte units)
+    (5, 200000, 262144, 200000),   # long rows: several tiles per row
+    (1000, 48, 96, 48),            # short rows: many rows per tile
+    (7, 6, 10, 8),                 # 2-byte units
+    (0, 16, 16, 16),               # empty
+])
+def test_planless_jobs_match_plan(rows, row_bytes, src_pitch, dst_pitch):
+    """tpamd_copy_jobs_run derives its tiles on the device; the plan derives them on the host. Same bytes."""
+    span_s = max(rows * max(src_pitch, row_bytes), 16)
+    span_d = max(rows * max(dst_pitch, row_bytes), 16)
+    g = torch.Generator().manual_seed(rows + row_bytes)
+    src = torch.randint(0, 256, (span_s,), generator=g, dtype=torch.uint8).to(DEV)
+    a = torch.full((span_d,), 0xEE, dtype=torch.uint8, device=DEV)
+    b = a.clone()
+    job = lambda dst: (src.data_ptr(), dst.data_ptr(), rows, row_bytes, src_pitch, dst_pitch)
+    plan = _native.CopyPlan([job(a)], DEV)
+    plan.run()
+    torch.cuda.synchronize()
+    plan.close()
+    _native.run_copy_jobs([job(b)], DEV)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    want = np.full(span_d, 0xEE, dtype=np.uint8)
+    s = src.cpu().numpy()
+    for r in range(rows):
+        want[r * dst_pitch: r * dst_pitch + row_bytes] = s[r * src_pitch: r * src_pitch + row_bytes]
+    assert np.array_equal(b.cpu().numpy(), want)
+
+
+def test_planless_many_jobs_and_limit():
+    src = torch.arange(16 * 64, dtype=torch.int32, device=DEV)
+    dst = torch.zeros_like(src)
+    jobs = [(src.data_ptr() + 256 * i, dst.data_ptr() + 256 * (15 - i), 1, 256, 0, 0) for i in range(16)]
+    _native.run_copy_jobs(jobs, DEV)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(16, 64), src.view(16, 64).flip(0))
+    arr = (_native.CopyJob * 17)(*[_native.CopyJob(*jobs[0]) for _ in range(17)])
+    assert _native.lib().tpamd_copy_jobs_run(arr, 17, None) == -1
+    assert b"at most" in _native.lib().tpamd_last_error()
+    # the Python helper falls back to a plan beyond the limit
+    dst.zero_()
+    _native.run_copy_jobs(jobs + [(src.data_ptr(), dst.data_ptr(), 0, 0, 0, 0)], DEV)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(16, 64), src.view(16, 64).flip(0))
