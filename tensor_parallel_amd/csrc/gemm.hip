@@ -1,15 +1,15 @@
 // Rank-shard Linear for prefill-sized M: y[M,N] = act(x[M,K] . w[N,K]^T + bias) on MFMA (bf16/f16),
 // and the fused SiLU-gated gate/up pair. Both operands are K-contiguous, so x rows and w rows are
-// staged into LDS the same way and fed to v_mfma_f32_32x32x16 with w as the row operand: a lane then
-// holds 4 consecutive output columns of one output row, which packs into one 8-byte store.
+// staged into LDS the same way and fed to the MFMA with w as the row operand: a lane then holds
+// 4 consecutive output columns of one output row, which packs into one 8-byte store.
 //
 // Two kernels share the tiling (block tile BM x BN x 64, WAVES_M x WAVES_N wavefronts of 64 lanes, two LDS
 // stages, one barrier per K tile):
-//   gemm_direct_kernel  256x256 tiles, K % 64 == 0. Global loads go straight into LDS (no register staging),
-//                       operand fragments are read one K step ahead of the MFMAs that use them, and the MFMAs of
-//                       the last K step of a tile overlap the barrier and the first fragment reads of the next.
-//   gemm_kernel         any K (multiple of 8) and the 128x128 tiling for small problems; next K tile prefetched
-//                       into registers while the current one is multiplied.
+//   gemm_direct_kernel  256x256 tiles, K % 64 == 0, v_mfma_f32_16x16x32. Global loads go straight into LDS (no
+//                       register staging), operand fragments are read one sub-step ahead of the MFMAs that use
+//                       them, and the loop body is scheduled by hand (see the comment on the kernel).
+//   gemm_kernel         any K (multiple of 8) and the 128x128 tiling for small problems, v_mfma_f32_32x32x16; next
+//                       K tile prefetched into registers while the current one is multiplied.
 #include "common.h"
 
 #include <type_traits>
@@ -244,9 +244,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 }
 
 typedef __attribute__((address_space(3))) void lds_void;
-// Each lane's 16 bytes land at lds_base + lane * 16; lds_base must be the same for the whole wavefront.
-__device__ __forceinline__ void load16_to_lds(const void *g, void *lds_base) {
-    __builtin_amdgcn_global_load_lds(g, (lds_void *)lds_base, 16, 0, 0);
+// Global->LDS load through a buffer descriptor: each lane's 16 bytes land at lds_base + lane * 16 (lds_base must be
+// the same for the whole wavefront); address = descriptor base + per-lane 32-bit offset + wavefront-uniform
+// offset, range-checked by the hardware against the descriptor's extent (a load beyond it returns zeros).
+// No per-lane 64-bit address arithmetic is needed to step through K.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t extent_bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(extent_bytes), 0x00020000);
+}
+__device__ __forceinline__ void buffer_load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t uniform_off, void *lds_base) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void *)lds_base, 16, static_cast<int>(lane_off), static_cast<int>(uniform_off), 0, 0);
 }
 // Fragment read that the compiler does not see as an LDS access. With ordinary loads it waits for every
 // in-flight global->LDS load before each LDS read (it cannot tell that they go to the other stage), which
@@ -268,17 +274,88 @@ __device__ __forceinline__ void drain_and_barrier() {
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// LDS layout of the direct kernel: staged rows are grouped in blocks of 8 (1 KiB, what one wavefront-wide
-// 16-byte-per-lane load fills), blocks are 1152 bytes apart, and inside a block the 16-byte chunk c of row r
-// sits in slot c ^ (r % 8). Reads of one chunk index over 32 consecutive rows are then bank-conflict free,
-// and every group of 8 lanes of a load still fetches one whole 128-byte row segment.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    if constexpr (DT == TPAMD_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// Epilogue of the direct kernel. With w as the first MFMA operand a lane holds D[n = 4*(lane/16) + i][m = lane%16],
+// i = 0..3: four consecutive output columns of one output row, one 8-byte store.
+// acc[a][b]: a = 16-row tile of x (8 per wavefront), b = 16-row tile of w (4 per wavefront; swiglu: 2 gate + 2 up).
+template <int DT, int MODE>
+__device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[8][4], int m_wave, int n_wave, int l16, int lq) {
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+        const int m = m_wave + a * 16 + l16;
+        if (m >= p.M) continue;
+        char *yrow = p.y + static_cast<int64_t>(m) * p.ldy * 2;
+#pragma unroll
+        for (int b = 0; b < (MODE == MODE_SWIGLU ? 2 : 4); ++b) {
+            const int n = n_wave + b * 16 + lq * 4;
+            if (n >= p.N) continue;  // N is a multiple of 4: the group of 4 is all in or all out
+            uint16_t h[4];
+            if constexpr (MODE == MODE_SWIGLU) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float g = half_to_f32<DT>(f32_to_half<DT>(acc[a][b][j]));
+                    const float u = half_to_f32<DT>(f32_to_half<DT>(acc[a][b + 2][j]));
+                    const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(g)));
+                    h[j] = f32_to_half<DT>(sl * u);
+                }
+            } else {
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (p.bias) {
+                    const uint2 braw = *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2);
+                    bv[0] = half_to_f32<DT>(braw.x & 0xffffu); bv[1] = half_to_f32<DT>(braw.x >> 16);
+                    bv[2] = half_to_f32<DT>(braw.y & 0xffffu); bv[3] = half_to_f32<DT>(braw.y >> 16);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float v = acc[a][b][j] + bv[j];
+                    if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+                    h[j] = f32_to_half<DT>(v);
+                }
+            }
+            uint2 o;
+            o.x = h[0] | (static_cast<uint32_t>(h[1]) << 16);
+            o.y = h[2] | (static_cast<uint32_t>(h[3]) << 16);
+            *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = o;
+        }
+    }
+}
+
+// gemm_direct_kernel: 256 x 256 x 64 tiles, 8 wavefronts (2 x 4, 128 x-rows by 64 w-rows each), 2 LDS stages.
+//
+// MFMA shape: v_mfma_f32_16x16x32. Under the chip's power limit it sustains about 14% more flops than the
+// 32x32x16 shape on random operands (it reads and writes a quarter of the accumulator bytes per instruction for
+// half the flops), and the main loop is power-bound.
+//
+// LDS layout: staged rows are grouped in blocks of 8 (1 KiB, what one wavefront-wide 16-byte-per-lane load fills),
+// blocks are 1152 bytes apart, and inside a block the 16-byte chunk c of row r sits in slot c ^ (r % 8). Reads of
+// one chunk index over 16 consecutive rows are then bank-conflict free, and every group of 8 lanes of a load still
+// fetches one whole 128-byte row segment.
+//
+// Global->LDS loads go through buffer descriptors (wavefront-uniform base and K offset, 32-bit per-lane offset
+// computed once), fragment reads are inline ds_read_b128 with counted waits, and the loop body is written out
+// instruction by instruction: one fragment read or one load between MFMAs, so LDS, the load path and the matrix
+// pipe see a steady trickle. A K tile is four sub-steps of 16 MFMAs:
+//   S1 (k 0..31, x tiles 0-3)   reads x tiles 4-7 of k 0..31
+//   S2 (k 0..31, x tiles 4-7)   reads x tiles 0-3 and the 4 w tiles of k 32..63
+//   S3 (k 32..63, x tiles 0-3)  reads x tiles 4-7 of k 32..63; then the one barrier of the tile
+//   S4 (k 32..63, x tiles 4-7)  reads x tiles 0-3 and w of k 0..31 of the NEXT tile
+// The loads of the tile after next are issued in S4, S1 and S2 (2 + 3 + 3 per wavefront) into the stage the
+// barrier has just freed.
 template <int DT, int MODE>
 __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
-    constexpr int BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 4, NW = 8;
-    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    constexpr int BM = 256, BN = 256, WAVES_N = 4, NW = 8;
     constexpr int BLK = 1152;
     constexpr int XREG = (BM / 8) * BLK, WREG = (BN / 8) * BLK, STAGE = XREG + WREG;
     constexpr int XB = BM / 8 / NW, WB = BN / 8 / NW;  // 1 KiB blocks per wavefront per operand
+    static_assert(XB == 4 && WB == 4, "8 loads per wavefront per tile");
 
     extern __shared__ __align__(16) char smem[];
 
@@ -290,18 +367,15 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    const int l32 = lane & 31, lhi = lane >> 5;
+    const int l16 = lane & 15, lq = lane >> 4;
 
-    // ---- global -> LDS: lane (rb, slot) of a load fetches chunk slot ^ rb of row rb of its block.
-    // Addresses are a wavefront-uniform base (tile origin + K offset, advanced on the scalar unit) plus a 32-bit
-    // per-lane offset computed once, so the loop spends no vector instructions on address arithmetic; the LDS
-    // destination of each load is uniform too.
+    // ---- global -> LDS: lane (rb, slot) of a load fetches chunk slot ^ rb of row rb of its block
     const int rb = lane >> 3, slot = lane & 7;
     const int lchunk = slot ^ rb;
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
     const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
-    const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : nullptr;
+    const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : w_base;
     uint32_t x_off[XB], w_off[WB];
 #pragma unroll
     for (int i = 0; i < XB; ++i) {
@@ -316,112 +390,158 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
         tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
         w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
     }
-    auto load_x = [&](int kt, int stage) {
-        const char *base = x_base + static_cast<int64_t>(kt) * BK * 2;
-        char *xs = smem + stage * STAGE;
-#pragma unroll
-        for (int i = 0; i < XB; ++i) load16_to_lds(base + x_off[i], xs + (wave_s + i * NW) * BLK);
+    // descriptor extents: up to the end of the last valid row below the tile origin
+    const int x_rows = p.M - m0 < BM ? p.M - m0 : BM;
+    const int w_rows = p.N - n0 < BN ? p.N - n0 : BN;
+    const uint32_t x_extent = static_cast<uint32_t>(x_rows - 1) * static_cast<uint32_t>(p.ldx * 2) + static_cast<uint32_t>(p.K) * 2;
+    const uint32_t w_extent = static_cast<uint32_t>(w_rows - 1) * static_cast<uint32_t>(p.ldw * 2) + static_cast<uint32_t>(p.K) * 2;
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x_base, x_extent);
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(w_base, w_extent);
+    const __amdgpu_buffer_rsrc_t w2_rsrc = make_rsrc(w2_base, w_extent);
+    auto gx = [&](int i, int kt, int stage) {
+        buffer_load16_to_lds(x_rsrc, x_off[i], static_cast<uint32_t>(kt) * (BK * 2), smem + stage * STAGE + (wave_s + i * NW) * BLK);
     };
-    auto load_w = [&](int kt, int stage) {
-        char *ws = smem + stage * STAGE + XREG;
-#pragma unroll
-        for (int i = 0; i < WB; ++i) {
-            const char *base = w_base;
-            if constexpr (MODE == MODE_SWIGLU) base = (wave_s + i * NW) * 8 < BN / 2 ? w_base : w2_base;  // uniform per load
-            load16_to_lds(base + static_cast<int64_t>(kt) * BK * 2 + w_off[i], ws + (wave_s + i * NW) * BLK);
-        }
+    auto gw = [&](int i, int kt, int stage) {
+        const bool up = MODE == MODE_SWIGLU && (wave_s + i * NW) * 8 >= BN / 2;  // i >= 2: known at compile time
+        buffer_load16_to_lds(up ? w2_rsrc : w_rsrc, w_off[i], static_cast<uint32_t>(kt) * (BK * 2),
+                             smem + stage * STAGE + XREG + (wave_s + i * NW) * BLK);
     };
 
-    // ---- LDS -> MFMA operand addresses: one per-lane base for x and one for w; the MFMA tiles of a wavefront are a
-    // compile-time number of 1152-byte blocks apart, which goes into the instruction's offset field
-    constexpr int X_TILE_STEP = 4 * BLK;                                         // 32 rows
-    constexpr int W_TILE_STEP = (MODE == MODE_SWIGLU ? (BN / 2) / 8 : 4) * BLK;  // swiglu: gate tile -> up tile
-    static_assert(MODE == MODE_LINEAR || TN == 2, "swiglu operand addressing assumes one gate and one up tile per wavefront");
+    // ---- LDS -> MFMA operands: one per-lane base for x and one for w; the 16-row tiles of a wavefront are a
+    // compile-time number of blocks apart, which goes into the instruction's offset field
+    constexpr int T16 = 2 * BLK;  // 16 rows
+    constexpr int WT1 = T16;
+    constexpr int WT2 = MODE == MODE_SWIGLU ? (BN / 2 / 8) * BLK : 2 * T16;  // swiglu: first up tile, 128 staged rows on
+    constexpr int WT3 = WT2 + T16;
     int x_rd0, w_rd0;
     {
-        const int r = wm * (BM / WAVES_M) + l32;
+        const int r = wm * 128 + l16;
         x_rd0 = (r >> 3) * BLK + (r & 7) * 128;
-        const int row = (MODE == MODE_SWIGLU ? wn * (BN / 2 / WAVES_N) : wn * (BN / WAVES_N)) + l32;
+        const int row = (MODE == MODE_SWIGLU ? wn * 32 : wn * 64) + l16;
         w_rd0 = XREG + (row >> 3) * BLK + (row & 7) * 128;
     }
-    int ks_off[BK / 16];
+    int kk_off[2];
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) ks_off[ks] = ((ks * 2 + lhi) ^ (l32 & 7)) * 16;
+    for (int kk = 0; kk < 2; ++kk) kk_off[kk] = ((kk * 4 + lq) ^ (l16 & 7)) * 16;
 
-    f32x16 acc[TM][TN];
+    f32x4 acc[8][4];
 #pragma unroll
-    for (int a = 0; a < TM; ++a)
+    for (int a = 0; a < 8; ++a)
 #pragma unroll
-        for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
+        for (int b = 0; b < 4; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    static_assert(TM == 4 && TN == 2, "the counted waits below assume 6 fragment reads per K step");
-    u32x4 xf[2][TM], wf[2][TN];
+    u32x4 xf[2][4], wf[2][4];
     const uint32_t smem_base = lds_addr_of(smem);
-    auto read_frags = [&](auto bufc, int stage_off, int ks) {
-        constexpr int buf = decltype(bufc)::value;
-        const uint32_t xa = smem_base + stage_off + x_rd0 + ks_off[ks];
-        const uint32_t wa = smem_base + stage_off + w_rd0 + ks_off[ks];
-        xf[buf][0] = lds_read16<0>(xa);
-        xf[buf][1] = lds_read16<X_TILE_STEP>(xa);
-        xf[buf][2] = lds_read16<2 * X_TILE_STEP>(xa);
-        xf[buf][3] = lds_read16<3 * X_TILE_STEP>(xa);
-        wf[buf][0] = lds_read16<0>(wa);
-        wf[buf][1] = lds_read16<W_TILE_STEP>(wa);
-    };
-    // LDS reads return in order: "at most N outstanding" means every read issued before the last N has landed.
-    // Naming the fragments as operands keeps the MFMAs that consume them behind the wait.
-#define TPAMD_WAIT_FRAGS(N, buf)                                                                                    \
-    asm volatile("s_waitcnt lgkmcnt(" #N ")"                                                                        \
-                 : "+v"(xf[buf][0]), "+v"(xf[buf][1]), "+v"(xf[buf][2]), "+v"(xf[buf][3]), "+v"(wf[buf][0]), "+v"(wf[buf][1]))
-#define TPAMD_DRAIN_BARRIER(buf)                                                                                    \
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"                                                       \
-                 : "+v"(xf[buf][0]), "+v"(xf[buf][1]), "+v"(xf[buf][2]), "+v"(xf[buf][3]), "+v"(wf[buf][0]), "+v"(wf[buf][1]) \
-                 :: "memory")
-    auto mfmas = [&](auto bufc) {
-        constexpr int buf = decltype(bufc)::value;
-        __builtin_amdgcn_s_setprio(1);  // the matrix pipe is the scarce unit: do not let the peer's loads cut in
-#pragma unroll
-        for (int a = 0; a < TM; ++a)
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-                acc[a][b] = mfma32<DT>(__builtin_bit_cast(uint4, wf[buf][b]), __builtin_bit_cast(uint4, xf[buf][a]), acc[a][b]);
-        __builtin_amdgcn_s_setprio(0);
-    };
-    using B0 = std::integral_constant<int, 0>;
-    using B1 = std::integral_constant<int, 1>;
+    // LDS reads return in order: "lgkmcnt(N)" = everything but the N youngest reads has landed. The counts below
+    // include the reads of the following sub-step issued in between. Naming a fragment as an operand of the wait
+    // keeps the MFMAs that consume it behind the wait. Everything is pinned in source order by the scheduling
+    // barriers: the compiler must not move a fragment register before its wait.
+#define TPAMD_SB __builtin_amdgcn_sched_barrier(0)
+#define TPAMD_WAIT(N, reg) asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(reg))
+#define TPAMD_MFMA(XS, WS, A0, a, b) acc[(A0) + (a)][b] = mfma16<DT>(wf[WS][b], xf[XS][a], acc[(A0) + (a)][b])
+#define TPAMD_DRAIN_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#define TPAMD_ROW(XS, WS, A0, a) TPAMD_MFMA(XS, WS, A0, a, 0); TPAMD_MFMA(XS, WS, A0, a, 1); TPAMD_MFMA(XS, WS, A0, a, 2); TPAMD_MFMA(XS, WS, A0, a, 3)
+    // Sub-step on x tiles 0-3 (fragments xf[0], read in the order x0 w0 w1 w2 w3 x1 x2 x3 by the sub-step before);
+    // reads x tiles 4-7 of the same k range into xf[1]; L0..L2: loads or nothing.
+#define TPAMD_SUB_A(WS, stage_off, kk, L0, L1, L2)                                                                  \
+    {                                                                                                               \
+        const uint32_t xa = smem_base + (stage_off) + x_rd0 + kk_off[kk];                                           \
+        TPAMD_SB;                                                                                                   \
+        TPAMD_WAIT(6, xf[0][0]); TPAMD_WAIT(6, wf[WS][0]); TPAMD_SB;                                                \
+        TPAMD_MFMA(0, WS, 0, 0, 0); TPAMD_SB; xf[1][0] = lds_read16<4 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_WAIT(6, wf[WS][1]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(0, WS, 0, 0, 1); TPAMD_SB; xf[1][1] = lds_read16<5 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_WAIT(6, wf[WS][2]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(0, WS, 0, 0, 2); TPAMD_SB; xf[1][2] = lds_read16<6 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_WAIT(6, wf[WS][3]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(0, WS, 0, 0, 3); TPAMD_SB; xf[1][3] = lds_read16<7 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_WAIT(6, xf[0][1]); TPAMD_SB;                                                                          \
+        TPAMD_ROW(0, WS, 0, 1); TPAMD_SB; L0; TPAMD_SB;                                                             \
+        TPAMD_WAIT(5, xf[0][2]); TPAMD_SB;                                                                          \
+        TPAMD_ROW(0, WS, 0, 2); TPAMD_SB; L1; TPAMD_SB;                                                             \
+        TPAMD_WAIT(4, xf[0][3]); TPAMD_SB;                                                                          \
+        TPAMD_ROW(0, WS, 0, 3); TPAMD_SB; L2; TPAMD_SB;                                                             \
+    }
+    // Sub-step on x tiles 4-7 (fragments xf[1]) with the same w fragments; reads x tiles 0-3 and the w tiles of
+    // (stage_off, kk) into xf[0] and wf[WR].
+#define TPAMD_SUB_B(WS, WR, stage_off, kk, L0, L1, L2)                                                              \
+    {                                                                                                               \
+        const uint32_t xa = smem_base + (stage_off) + x_rd0 + kk_off[kk];                                           \
+        const uint32_t wa = smem_base + (stage_off) + w_rd0 + kk_off[kk];                                           \
+        TPAMD_SB;                                                                                                   \
+        TPAMD_WAIT(3, xf[1][0]); TPAMD_SB;                                                                          \
+        TPAMD_MFMA(1, WS, 4, 0, 0); TPAMD_SB; xf[0][0] = lds_read16<0>(xa); TPAMD_SB;                               \
+        TPAMD_MFMA(1, WS, 4, 0, 1); TPAMD_SB; wf[WR][0] = lds_read16<0>(wa); TPAMD_SB;                              \
+        TPAMD_MFMA(1, WS, 4, 0, 2); TPAMD_SB; wf[WR][1] = lds_read16<WT1>(wa); TPAMD_SB;                            \
+        TPAMD_MFMA(1, WS, 4, 0, 3); TPAMD_SB; wf[WR][2] = lds_read16<WT2>(wa); TPAMD_SB;                            \
+        TPAMD_WAIT(6, xf[1][1]); TPAMD_SB;                                                                          \
+        TPAMD_MFMA(1, WS, 4, 1, 0); TPAMD_SB; wf[WR][3] = lds_read16<WT3>(wa); TPAMD_SB;                            \
+        TPAMD_MFMA(1, WS, 4, 1, 1); TPAMD_SB; xf[0][1] = lds_read16<1 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_MFMA(1, WS, 4, 1, 2); TPAMD_SB; xf[0][2] = lds_read16<2 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_MFMA(1, WS, 4, 1, 3); TPAMD_SB; xf[0][3] = lds_read16<3 * T16>(xa); TPAMD_SB;                         \
+        TPAMD_WAIT(9, xf[1][2]); TPAMD_SB;                                                                          \
+        TPAMD_ROW(1, WS, 4, 2); TPAMD_SB; L0; TPAMD_SB;                                                             \
+        TPAMD_WAIT(8, xf[1][3]); TPAMD_SB;                                                                          \
+        TPAMD_MFMA(1, WS, 4, 3, 0); TPAMD_MFMA(1, WS, 4, 3, 1); TPAMD_SB; L1; TPAMD_SB;                             \
+        TPAMD_MFMA(1, WS, 4, 3, 2); TPAMD_MFMA(1, WS, 4, 3, 3); TPAMD_SB; L2; TPAMD_SB;                             \
+    }
+#define NOP_ (void)0
 
     const int KT = p.K / BK;  // K is a multiple of 64 here
-    load_x(0, 0);
-    load_w(0, 0);
+    const int last = KT - 1;
+#pragma unroll
+    for (int i = 0; i < XB; ++i) gx(i, 0, 0);
+#pragma unroll
+    for (int i = 0; i < WB; ++i) gw(i, 0, 0);
     drain_and_barrier();
-    read_frags(B0{}, 0, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-        const bool more = kt + 1 < KT;
-        const int cur = (kt & 1) * STAGE, nxt = ((kt + 1) & 1) * STAGE;
-        // K step 0: fragments of step 1 and half of the next tile's loads are issued, then step 0 multiplies
-        read_frags(B1{}, cur, 1);
-        if (more) load_x(kt + 1, (kt + 1) & 1);
-        TPAMD_WAIT_FRAGS(6, 0);
-        mfmas(B0{});
-        read_frags(B0{}, cur, 2);
-        if (more) load_w(kt + 1, (kt + 1) & 1);
-        TPAMD_WAIT_FRAGS(6, 1);
-        mfmas(B1{});
-        read_frags(B1{}, cur, 3);
-        TPAMD_WAIT_FRAGS(6, 0);
-        mfmas(B0{});
-        // every wavefront is done reading this tile and the next one has landed; the MFMAs of step 3 then run
-        // under the first fragment reads of the next tile
-        TPAMD_DRAIN_BARRIER(1);
-        if (more) read_frags(B0{}, nxt, 0);
-        mfmas(B1{});
+    {
+        const uint32_t xa = smem_base + x_rd0 + kk_off[0];
+        const uint32_t wa = smem_base + w_rd0 + kk_off[0];
+        xf[0][0] = lds_read16<0>(xa);
+        wf[0][0] = lds_read16<0>(wa);
+        wf[0][1] = lds_read16<WT1>(wa);
+        wf[0][2] = lds_read16<WT2>(wa);
+        wf[0][3] = lds_read16<WT3>(wa);
+        xf[0][1] = lds_read16<1 * T16>(xa);
+        xf[0][2] = lds_read16<2 * T16>(xa);
+        xf[0][3] = lds_read16<3 * T16>(xa);
     }
-#undef TPAMD_WAIT_FRAGS
+    // Loads past the last tile are clamped to the last tile: they refill a stage nobody reads any more, which
+    // keeps the loop body free of branches (a branch here makes the compiler copy fragment registers around
+    // before the counted waits, i.e. before their data has landed).
+    gx(0, last < 1 ? last : 1, 1);
+    gx(1, last < 1 ? last : 1, 1);
+    for (int kt = 0; kt < last; ++kt) {
+        const int cur = (kt & 1) * STAGE, nxt = ((kt + 1) & 1) * STAGE;
+        const int ns = (kt + 1) & 1, k1 = kt + 1;
+        TPAMD_SUB_A(0, cur, 0, gx(2, k1, ns), gx(3, k1, ns), gw(0, k1, ns));
+        TPAMD_SUB_B(0, 1, cur, 1, gw(1, k1, ns), gw(2, k1, ns), gw(3, k1, ns));
+        TPAMD_SUB_A(1, cur, 1, NOP_, NOP_, NOP_);
+        // every wavefront is done reading this tile and the next one has landed
+        TPAMD_DRAIN_BARRIER();
+        const int k2 = kt + 2 < last ? kt + 2 : last, cs = kt & 1;
+        TPAMD_SUB_B(1, 0, nxt, 0, NOP_, gx(0, k2, cs), gx(1, k2, cs));
+    }
+    {
+        const int cur = (last & 1) * STAGE;
+        TPAMD_SUB_A(0, cur, 0, NOP_, NOP_, NOP_);
+        TPAMD_SUB_B(0, 1, cur, 1, NOP_, NOP_, NOP_);
+        TPAMD_SUB_A(1, cur, 1, NOP_, NOP_, NOP_);
+        TPAMD_DRAIN_BARRIER();  // also: no global->LDS load is in flight when the wavefront leaves the loop
+        TPAMD_WAIT(0, xf[1][0]); TPAMD_WAIT(0, xf[1][1]); TPAMD_WAIT(0, xf[1][2]); TPAMD_WAIT(0, xf[1][3]);
+        TPAMD_WAIT(0, wf[1][0]); TPAMD_WAIT(0, wf[1][1]); TPAMD_WAIT(0, wf[1][2]); TPAMD_WAIT(0, wf[1][3]);
+        TPAMD_ROW(1, 1, 4, 0); TPAMD_ROW(1, 1, 4, 1); TPAMD_ROW(1, 1, 4, 2); TPAMD_ROW(1, 1, 4, 3);
+    }
+#undef NOP_
+#undef TPAMD_SB
+#undef TPAMD_WAIT
+#undef TPAMD_MFMA
+#undef TPAMD_ROW
+#undef TPAMD_SUB_A
+#undef TPAMD_SUB_B
 #undef TPAMD_DRAIN_BARRIER
 
-    epilogue<DT, MODE, BM, BN, WAVES_M, WAVES_N>(p, acc, m0, n0, wm, wn, l32, lhi);
+    epilogue16<DT, MODE>(p, acc, m0 + wm * 128, n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq);
 }
 
 // ---- any dtype, any alignment: LDS-tiled FMA kernel, 64x64 tile, 256 threads, 4x4 outputs per thread ---------
@@ -555,7 +675,8 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     // 256x256 tiles once they fill the chip at least about once, else 128x128 tiles.
     const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
     if (big_tiles >= 200) {
-        if (p.K % 64 == 0 && p.K >= 64) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
+        // the direct kernel addresses a tile with 32-bit byte offsets from the tile origin
+        if (p.K % 64 == 0 && p.K >= 64 && p.ldx < (1ll << 22) && p.ldw < (1ll << 22)) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
         return swiglu ? launch_gemm<DT, MODE_SWIGLU, 256, 256, 2, 4>(p, s) : launch_gemm<DT, MODE_LINEAR, 256, 256, 2, 4>(p, s);
     }
     return swiglu ? launch_gemm<DT, MODE_SWIGLU, 128, 128, 2, 2>(p, s) : launch_gemm<DT, MODE_LINEAR, 128, 128, 2, 2>(p, s);
