@@ -22,6 +22,28 @@ from .slicing import concat_dim
 
 RENDEZVOUS_TIMEOUT_S = 600.0
 
+# Rank threads that share ONE device take turns on the host: a rank holds the "turn" lock while it runs module
+# code and gives it up only while it waits in a rendezvous. All ranks enqueue onto the same device anyway, so
+# nothing is lost, and host-side lazy initialisation inside torch (attention backends, BLAS handles) is never
+# entered by two rank threads at once. The lock of the running forward is published per thread here.
+_turn = threading.local()
+
+
+def set_turn_lock(lock: Optional[threading.Lock]) -> None:
+    _turn.lock = lock
+
+
+def _rendezvous(barrier: threading.Barrier, timeout: float) -> None:
+    lock = getattr(_turn, "lock", None)
+    if lock is None:
+        barrier.wait(timeout)
+        return
+    lock.release()
+    try:
+        barrier.wait(timeout)
+    finally:
+        lock.acquire()
+
 
 class CollectiveOpetationBase:
     def __call__(self, x: torch.Tensor, rank: int):
@@ -44,7 +66,7 @@ class CollectiveOperation(CollectiveOpetationBase):
     def __call__(self, x: Any, rank: int):
         try:
             self._inputs[rank] = x
-            self._barrier.wait(self.timeout)
+            _rendezvous(self._barrier, self.timeout)
             if rank == 0:
                 try:
                     result = self.func(*self._inputs)
@@ -53,7 +75,7 @@ class CollectiveOperation(CollectiveOpetationBase):
                     self._error = None
                 except BaseException as e:  # fan the failure out to every rank
                     self._error = e
-            self._barrier.wait(self.timeout)
+            _rendezvous(self._barrier, self.timeout)
             if self._error is not None:
                 raise self._error
             return self._outputs[rank]
@@ -61,7 +83,7 @@ class CollectiveOperation(CollectiveOpetationBase):
             self._inputs[rank] = None
             # the third rendezvous keeps a fast rank from starting the next call while a slow one still reads
             try:
-                self._barrier.wait(self.timeout)
+                _rendezvous(self._barrier, self.timeout)
             except threading.BrokenBarrierError:
                 pass
             self._outputs[rank] = None

@@ -78,7 +78,30 @@ __device__ __forceinline__ uint16_t f32_to_half(float f) {
     else return f32_to_f16(f);
 }
 
+// Two fp32 values rounded to nearest even and packed (a in the low half): v_cvt_pk_bf16_f32 for bf16.
+typedef float tpamd_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 tpamd_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 tpamd_f16x2 __attribute__((ext_vector_type(2)));
+template <int DT>
+__device__ __forceinline__ uint32_t pack2_half(float a, float b) {
+    const tpamd_f32x2 v = {a, b};
+    if constexpr (DT == TPAMD_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, tpamd_bf16x2));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, tpamd_f16x2));
+}
+template <int DT>
+__device__ __forceinline__ float lo_half_to_f32(uint32_t p) {
+    if constexpr (DT == TPAMD_BF16) return __uint_as_float(p << 16);
+    else return half_to_f32<DT>(static_cast<uint16_t>(p & 0xffffu));
+}
+template <int DT>
+__device__ __forceinline__ float hi_half_to_f32(uint32_t p) {
+    if constexpr (DT == TPAMD_BF16) return __uint_as_float(p & 0xffff0000u);
+    else return half_to_f32<DT>(static_cast<uint16_t>(p >> 16));
+}
+
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
-__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+// v_exp_f32 and v_rcp_f32 (1 ulp each) instead of the 10-instruction IEEE division sequence. Every kernel uses this
+// one definition, so a row's result does not depend on which kernel the batch size selects.
+__device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 }  // namespace tpamd

@@ -297,32 +297,35 @@ __device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[8][
         for (int b = 0; b < (MODE == MODE_SWIGLU ? 2 : 4); ++b) {
             const int n = n_wave + b * 16 + lq * 4;
             if (n >= p.N) continue;  // N is a multiple of 4: the group of 4 is all in or all out
-            uint16_t h[4];
+            uint2 o;
             if constexpr (MODE == MODE_SWIGLU) {
+                // gate and up products rounded to the tensor dtype, then silu and the product each rounded again
+                uint32_t out[2];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float g = half_to_f32<DT>(f32_to_half<DT>(acc[a][b][j]));
-                    const float u = half_to_f32<DT>(f32_to_half<DT>(acc[a][b + 2][j]));
-                    const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(g)));
-                    h[j] = f32_to_half<DT>(sl * u);
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t g2 = pack2_half<DT>(acc[a][b][2 * j], acc[a][b][2 * j + 1]);
+                    const uint32_t u2 = pack2_half<DT>(acc[a][b + 2][2 * j], acc[a][b + 2][2 * j + 1]);
+                    const uint32_t s2 = pack2_half<DT>(silu_f32(lo_half_to_f32<DT>(g2)), silu_f32(hi_half_to_f32<DT>(g2)));
+                    out[j] = pack2_half<DT>(lo_half_to_f32<DT>(s2) * lo_half_to_f32<DT>(u2), hi_half_to_f32<DT>(s2) * hi_half_to_f32<DT>(u2));
                 }
+                o.x = out[0];
+                o.y = out[1];
             } else {
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = acc[a][b][j];
                 if (p.bias) {
                     const uint2 braw = *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2);
-                    bv[0] = half_to_f32<DT>(braw.x & 0xffffu); bv[1] = half_to_f32<DT>(braw.x >> 16);
-                    bv[2] = half_to_f32<DT>(braw.y & 0xffffu); bv[3] = half_to_f32<DT>(braw.y >> 16);
+                    v[0] += lo_half_to_f32<DT>(braw.x); v[1] += hi_half_to_f32<DT>(braw.x);
+                    v[2] += lo_half_to_f32<DT>(braw.y); v[3] += hi_half_to_f32<DT>(braw.y);
                 }
+                if (p.act == TPAMD_ACT_GELU) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float v = acc[a][b][j] + bv[j];
-                    if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
-                    h[j] = f32_to_half<DT>(v);
+                    for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
                 }
+                o.x = pack2_half<DT>(v[0], v[1]);
+                o.y = pack2_half<DT>(v[2], v[3]);
             }
-            uint2 o;
-            o.x = h[0] | (static_cast<uint32_t>(h[1]) << 16);
-            o.y = h[2] | (static_cast<uint32_t>(h[3]) << 16);
             *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = o;
         }
     }

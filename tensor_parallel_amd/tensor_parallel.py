@@ -16,6 +16,7 @@ import torch
 from torch import nn
 
 from .autoconfig import get_default_config
+from .collectives import set_turn_lock
 from .config import Config
 from .shard import make_shard
 from .slicing import BatchSlicer, concat_specs
@@ -187,9 +188,23 @@ def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devi
     results: dict = {}
     lock = threading.Lock()
     grad_enabled = torch.is_grad_enabled()
+    # ranks that share one device take turns on the host (see collectives.set_turn_lock)
+    shared = len(modules) > 1 and all(d.type == "cuda" and d == devices[0] for d in devices)
+    turn = threading.Lock() if shared else None
 
     def worker(i, module, args, kwargs, device):
         torch.set_grad_enabled(grad_enabled)
+        if turn is not None:
+            turn.acquire()
+            set_turn_lock(turn)
+        try:
+            _run(i, module, args, kwargs, device)
+        finally:
+            if turn is not None:
+                set_turn_lock(None)
+                turn.release()
+
+    def _run(i, module, args, kwargs, device):
         try:
             if device.type == "cuda":
                 torch.cuda.set_device(device)

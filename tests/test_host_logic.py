@@ -315,3 +315,48 @@ def test_rendezvous_timeout_does_not_hang():
     op = CollectiveOperation(2, lambda *xs: list(xs), timeout=0.2)
     with pytest.raises(threading.BrokenBarrierError):
         op(1, 0)  # the peer never arrives
+
+
+def test_rank_threads_take_turns_between_rendezvous():
+    """With a turn lock published, only one rank runs host code at a time; the lock is given up inside a
+    rendezvous (otherwise the second rank could never arrive) and is free again afterwards."""
+    import threading
+    import time
+
+    from tensor_parallel_amd.collectives import CollectiveOperation, set_turn_lock
+
+    world = 3
+    op = CollectiveOperation(world, lambda *xs: [sum(xs)] * world, timeout=20.0)
+    turn = threading.Lock()
+    running, overlaps, results = [0], [0], {}
+
+    def critical():
+        running[0] += 1
+        if running[0] > 1:
+            overlaps[0] += 1
+        time.sleep(0.002)
+        running[0] -= 1
+
+    def worker(rank):
+        turn.acquire()
+        set_turn_lock(turn)
+        try:
+            total = 0
+            for step in range(5):
+                critical()
+                total += op(rank + step, rank)
+            results[rank] = total
+        finally:
+            set_turn_lock(None)
+            turn.release()
+
+    threads = [threading.Thread(target=worker, args=(r,)) for r in range(world)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(30)
+    assert not any(t.is_alive() for t in threads)
+    assert overlaps[0] == 0
+    want = sum(sum(r + step for r in range(world)) for step in range(5))
+    assert results == {r: want for r in range(world)}
+    assert turn.acquire(blocking=False)
