@@ -12,6 +12,7 @@
 // the activation dtype in registers, exact for |q| <= 128).
 #include "common.h"
 
+#include <stdlib.h>
 #include <type_traits>
 
 namespace tpamd {
@@ -79,23 +80,30 @@ __device__ __forceinline__ void cvt_i8x4(uint32_t q, uint32_t &lo, uint32_t &hi)
 // half-line requests, not by bytes (measured: 1.5-2x slower). So a load instruction here fetches 8 rows x 128
 // contiguous bytes (whole cache lines), and the loaded registers go through a wavefront-private LDS tile:
 // written in fetch order, read back in MFMA operand order. x takes the same route when the weights are 16-bit.
-template <int DT, bool W8, int MT, int MODE>
+//
+// CG = groups of 16 output columns per block. With CG > 1 the x fragments of a chunk are reused for CG weight
+// tiles, which divides the x bytes a block pulls from L2 per weight byte by CG (what limits this kernel once
+// M * 2 bytes of x per K element outweigh the 16 * itemsize(w) bytes of w); the registers this costs are taken
+// from the prefetch buffers, so CG > 1 loads a chunk, multiplies it and only then loads the next, and relies on
+// the 8 wavefronts of the block being out of phase. CG > 1 needs N % (16 * CG) == 0.
+template <int DT, bool W8, int MT, int MODE, int CG>
 __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     constexpr int NMAT = MODE == SK_SWIGLU ? 2 : 1;
+    constexpr int NA = NMAT * CG;             // weight tiles per chunk: index a = cg * NMAT + matrix
+    constexpr bool PRE = CG == 1;             // double-buffered loads
     constexpr int LANE_K = W8 ? 64 : 32;      // K elements per lane per chunk (64 bytes of w)
     constexpr int CHUNK_K = LANE_K * 4;       // K elements per chunk
     constexpr int WV = 4;                     // 16-byte loads of w per lane per chunk
     constexpr int XV = LANE_K / 8;            // 16-byte loads of x per lane per chunk per m-tile
-    constexpr int WK = W8 ? 16 : 8;           // K elements in one 16-byte load of w
 
     constexpr int TROW = 272;                 // staged row pitch: 256 bytes + 16 pad
-    constexpr bool XT = !W8;                  // x goes through the LDS tile too
     __shared__ float red[SK_WAVES][NMAT][MT][4][64];
     __shared__ __align__(16) char stage_all[SK_WAVES][16 * TROW];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 15, lg = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * 16 * CG;
+    const int64_t cg_stride = static_cast<int64_t>(16) * p.ldw * (W8 ? 1 : 2);  // bytes from one column group to the next
 
     int wrow = n0 + lr;
     wrow = wrow < p.N ? wrow : p.N - 1;
@@ -115,13 +123,11 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
         wp[h] = p.w + static_cast<int64_t>(r) * p.ldw * wbytes + cpiece * 16;
         if constexpr (NMAT == 2) wp2[h] = p.w2 + static_cast<int64_t>(r) * p.ldw * wbytes + cpiece * 16;
     }
-    const char *xp[MT];
     bool xok[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + lr;
         xok[t] = m < p.M;
-        xp[t] = p.x + (static_cast<int64_t>(xok[t] ? m : 0) * p.ldx + lg * WK) * 2;
     }
     const char *xpc[MT][2];
     bool xokc[MT][2];
@@ -134,9 +140,9 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
             xpc[t][h] = p.x + static_cast<int64_t>(xokc[t][h] ? m : 0) * p.ldx * 2 + cpiece * 16;
         }
 
-    f32x4 acc[NMAT][MT];
+    f32x4 acc[NA][MT];
 #pragma unroll
-    for (int a = 0; a < NMAT; ++a)
+    for (int a = 0; a < NA; ++a)
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[a][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -145,25 +151,42 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
 
     // Register double buffers for the weights (and for x when it is small enough). Buffer indices are
     // compile-time constants so that the arrays stay in registers.
-    constexpr bool XPRE = MT * XV <= 8;
-    uint4 wv[2][NMAT][WV];
+    constexpr bool XPRE = PRE && MT * XV <= 8;
+    uint4 wv[PRE ? 2 : 1][NA][WV];
     uint4 xv[XPRE ? 2 : 1][MT][XV];
     auto load_w = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
         const int64_t off = static_cast<int64_t>(c) * CHUNK_K * wbytes;
 #pragma unroll
-        for (int a = 0; a < NMAT; ++a)
+        for (int a = 0; a < NA; ++a)
 #pragma unroll
             for (int i = 0; i < WV; ++i) {
                 const int byte = (i >> 1) * 128 + cpiece * 16;            // inside the chunk's 256 bytes of the row
                 const bool ok = c * CHUNK_K + byte / wbytes < p.K;
-                const char *base = a == 0 ? wp[i & 1] : wp2[i & 1];
+                const char *base = (a % NMAT == 0 ? wp[i & 1] : wp2[i & 1]) + (a / NMAT) * cg_stride;
                 const uint4 raw = nt_load_u4(ok ? base + off + (i >> 1) * 128 : base - cpiece * 16);  // unconditional
                 wv[buf][a][i] = ok ? raw : zero4;
             }
     };
     // registers in fetch order -> registers in MFMA operand order, through this wavefront's LDS tile
-    auto transpose = [&](uint4 (&r)[WV]) {
+    auto transpose = [&](uint4 *r) {
+#pragma unroll
+        for (int i = 0; i < WV; ++i) *reinterpret_cast<uint4 *>(stage + st_wr + (i & 1) * 8 * TROW + (i >> 1) * 128) = r[i];
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+        if constexpr (W8) {
+            // (only x takes this branch with int8 weights, see compute) operand order that meets the int8 tile:
+            // lane slot lg holds k = v'*64 + lg*16 + h*8 .. +8 for register 2*v' + h of the 256-element chunk
+#pragma unroll
+            for (int v = 0; v < WV; ++v) r[v] = *reinterpret_cast<const uint4 *>(stage + lr * TROW + (v >> 1) * 128 + lg * 32 + (v & 1) * 16);
+        } else {
+#pragma unroll
+            for (int v = 0; v < WV; ++v) r[v] = *reinterpret_cast<const uint4 *>(stage + st_rd + v * 64);
+        }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    };
+    auto transpose_w = [&](uint4 *r) {
 #pragma unroll
         for (int i = 0; i < WV; ++i) *reinterpret_cast<uint4 *>(stage + st_wr + (i & 1) * 8 * TROW + (i >> 1) * 128) = r[i];
         __builtin_amdgcn_wave_barrier();
@@ -173,45 +196,36 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
         __builtin_amdgcn_wave_barrier();
         asm volatile("" ::: "memory");
     };
+    // x in fetch order too: load i covers rows (lane/8) + 8*(i&1), bytes (i/2)*128 + (lane%8)*16 of the chunk's
+    // 256 (16-bit weights) or 512 (int8 weights) bytes of the row
     auto load_x = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
-        const int kbase = c * CHUNK_K + lg * WK;
         const int64_t xoff = static_cast<int64_t>(c) * CHUNK_K * 2;
-        if constexpr (XT) {
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int i = 0; i < XV; ++i) {
-                    const int byte = (i >> 1) * 128 + cpiece * 16;
-                    const bool ok = xokc[t][i & 1] && c * CHUNK_K + byte / 2 < p.K;
-                    xv[buf][t][i] = ok ? *reinterpret_cast<const uint4 *>(xpc[t][i & 1] + xoff + (i >> 1) * 128) : zero4;
-                }
-            return;
-        }
 #pragma unroll
         for (int t = 0; t < MT; ++t)
 #pragma unroll
-            for (int v = 0; v < XV; ++v) {
-                // the x elements that meet w load v (bf16/f16 w) or half (v & 1) of w load v / 2 (int8 w)
-                const int krel = W8 ? (v / 2) * 64 + (v & 1) * 8 : v * 32;
-                xv[buf][t][v] = (xok[t] && kbase + krel < p.K) ? *reinterpret_cast<const uint4 *>(xp[t] + xoff + krel * 2) : zero4;
+            for (int i = 0; i < XV; ++i) {
+                const int byte = (i >> 1) * 128 + cpiece * 16;
+                const bool ok = xokc[t][i & 1] && c * CHUNK_K + byte / 2 < p.K;
+                xv[buf][t][i] = ok ? *reinterpret_cast<const uint4 *>(xpc[t][i & 1] + xoff + (i >> 1) * 128) : zero4;
             }
     };
     auto compute = [&](auto bufc) {
         constexpr int buf = decltype(bufc)::value;
         constexpr int xb = XPRE ? buf : 0;
 #pragma unroll
-        for (int a = 0; a < NMAT; ++a) transpose(wv[buf][a]);
-        if constexpr (XT) {
+        for (int a = 0; a < NA; ++a) transpose_w(wv[PRE ? buf : 0][a]);
 #pragma unroll
-            for (int t = 0; t < MT; ++t) transpose(xv[xb][t]);
+        for (int t = 0; t < MT; ++t) {
+            transpose(&xv[xb][t][0]);
+            if constexpr (W8) transpose(&xv[xb][t][4]);  // second 256 bytes of the row's chunk
         }
 #pragma unroll
-        for (int a = 0; a < NMAT; ++a) {
+        for (int a = 0; a < NA; ++a) {
             if constexpr (W8) {
 #pragma unroll
                 for (int v = 0; v < WV; ++v) {  // 16 int8 -> two operands of 8
-                    const uint4 q = wv[buf][a][v];
+                    const uint4 q = wv[PRE ? buf : 0][a][v];
                     uint4 w0, w1;
                     cvt_i8x4<DT>(q.x, w0.x, w0.y);
                     cvt_i8x4<DT>(q.y, w0.z, w0.w);
@@ -227,7 +241,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
 #pragma unroll
                 for (int v = 0; v < WV; ++v)
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) acc[a][t] = mfma16<DT>(wv[buf][a][v], xv[xb][t][v], acc[a][t]);
+                    for (int t = 0; t < MT; ++t) acc[a][t] = mfma16<DT>(wv[PRE ? buf : 0][a][v], xv[xb][t][v], acc[a][t]);
             }
         }
     };
@@ -238,41 +252,53 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
     // This wavefront's chunks are wave, wave + SK_WAVES, ... The next chunk's loads are issued before the
     // current one is multiplied. Loads return in order, so whatever the multiply waits for is issued
     // ahead of the prefetch.
-    int c = wave;
-    if (c < nchunks) {
-        load_w(B0{}, c);
-        if constexpr (XPRE) load_x(B0{}, c);
-    }
-    while (c < nchunks) {
-        int cn = c + SK_WAVES;
-        if constexpr (!XPRE) load_x(B0{}, c);
-        if (cn < nchunks) {
-            load_w(B1{}, cn);
-            if constexpr (XPRE) load_x(B1{}, cn);
+    if constexpr (PRE) {
+        int c = wave;
+        if (c < nchunks) {
+            load_w(B0{}, c);
+            if constexpr (XPRE) load_x(B0{}, c);
         }
-        compute(B0{});
-        c = cn;
-        if (c >= nchunks) break;
-        cn = c + SK_WAVES;
-        if constexpr (!XPRE) load_x(B0{}, c);
-        if (cn < nchunks) {
-            load_w(B0{}, cn);
-            if constexpr (XPRE) load_x(B0{}, cn);
+        while (c < nchunks) {
+            int cn = c + SK_WAVES;
+            if constexpr (!XPRE) load_x(B0{}, c);
+            if (cn < nchunks) {
+                load_w(B1{}, cn);
+                if constexpr (XPRE) load_x(B1{}, cn);
+            }
+            compute(B0{});
+            c = cn;
+            if (c >= nchunks) break;
+            cn = c + SK_WAVES;
+            if constexpr (!XPRE) load_x(B0{}, c);
+            if (cn < nchunks) {
+                load_w(B0{}, cn);
+                if constexpr (XPRE) load_x(B0{}, cn);
+            }
+            compute(B1{});
+            c = cn;
         }
-        compute(B1{});
-        c = cn;
+    } else {
+        for (int c = wave; c < nchunks; c += SK_WAVES) {
+            load_w(B0{}, c);
+            load_x(B0{}, c);
+            compute(B0{});
+        }
     }
 
     // ---- int8 path: the outlier columns, spread over the wavefronts in groups of 32 ----------------
-    f32x4 acc_o[MT];
     if constexpr (W8) {
+        f32x4 acc_o[CG][MT];
 #pragma unroll
-        for (int t = 0; t < MT; ++t) acc_o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc_o[g][t] = f32x4{0.f, 0.f, 0.f, 0.f};
         const uint16_t *xo = reinterpret_cast<const uint16_t *>(p.x);
         const uint16_t *wo = reinterpret_cast<const uint16_t *>(p.w_out);
         for (int s = wave; s * 32 < p.n_out; s += SK_WAVES) {
-            uint32_t wq[4] = {0, 0, 0, 0};
+            uint32_t wq[CG][4];
             uint32_t xq[MT][4];
+#pragma unroll
+            for (int g = 0; g < CG; ++g) wq[g][0] = wq[g][1] = wq[g][2] = wq[g][3] = 0;
 #pragma unroll
             for (int t = 0; t < MT; ++t) xq[t][0] = xq[t][1] = xq[t][2] = xq[t][3] = 0;
 #pragma unroll
@@ -280,8 +306,12 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
                 const int o = s * 32 + lg * 8 + j;
                 if (o < p.n_out) {
                     const int col = p.outlier_idx[o];
-                    const uint32_t wval = wo[static_cast<int64_t>(wrow) * p.ld_wout + o];
-                    wq[j >> 1] |= wval << ((j & 1) * 16);
+#pragma unroll
+                    for (int g = 0; g < CG; ++g) {
+                        const int wr = CG == 1 ? wrow : n0 + g * 16 + lr;  // CG > 1: every row of the block exists
+                        const uint32_t wval = wo[static_cast<int64_t>(wr) * p.ld_wout + o];
+                        wq[g][j >> 1] |= wval << ((j & 1) * 16);
+                    }
 #pragma unroll
                     for (int t = 0; t < MT; ++t)
                         if (xok[t]) {
@@ -291,59 +321,68 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(SkinnyParams p) {
                 }
             }
 #pragma unroll
+            for (int g = 0; g < CG; ++g)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    acc_o[g][t] = mfma16<DT>(make_uint4(wq[g][0], wq[g][1], wq[g][2], wq[g][3]),
+                                             make_uint4(xq[t][0], xq[t][1], xq[t][2], xq[t][3]), acc_o[g][t]);
+        }
+        // fold the per-row scale in before the partial sums meet, then add the outlier product.
+        // D[n_local][m_local]: lane -> m_local = lr, register i -> n_local = 4*lg + i
+#pragma unroll
+        for (int g = 0; g < CG; ++g) {
+            float sc[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int n = n0 + g * 16 + lg * 4 + i;
+                n = n < p.N ? n : p.N - 1;
+                sc[i] = p.scale[n];
+            }
+#pragma unroll
             for (int t = 0; t < MT; ++t)
-                acc_o[t] = mfma16<DT>(make_uint4(wq[0], wq[1], wq[2], wq[3]), make_uint4(xq[t][0], xq[t][1], xq[t][2], xq[t][3]), acc_o[t]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[g * NMAT][t][i] = acc[g * NMAT][t][i] * sc[i] + acc_o[g][t][i];
         }
     }
 
-    // ---- cross-wave reduction. D[n_local][m_local]: lane -> m_local = lr, register i -> n_local = 4*lg + i
-    if constexpr (W8) {
-        // fold the per-row scale in before the partial sums meet, then add the outlier product
-        float sc[4];
+    // ---- cross-wave reduction, one column group at a time through the same LDS array ------------------
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int n = n0 + lg * 4 + i;
-            n = n < p.N ? n : p.N - 1;
-            sc[i] = p.scale[n];
-        }
+    for (int g = 0; g < CG; ++g) {
+        if (g > 0) __syncthreads();
 #pragma unroll
-        for (int t = 0; t < MT; ++t)
+        for (int a = 0; a < NMAT; ++a)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[0][t][i] = acc[0][t][i] * sc[i] + acc_o[t][i];
-    }
+            for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int a = 0; a < NMAT; ++a)
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) red[wave][a][t][i][lane] = acc[a][t][i];
-    __syncthreads();
+                for (int i = 0; i < 4; ++i) red[wave][a][t][i][lane] = acc[g * NMAT + a][t][i];
+        __syncthreads();
 
-    // thread e -> output (m = e / 16, n_local = e % 16): 16 consecutive threads store one 32-byte row piece
-    for (int e = tid; e < MT * 256; e += SK_THREADS) {
-        const int m = e >> 4, nl = e & 15;
-        const int n = n0 + nl;
-        if (m >= p.M || n >= p.N) continue;
-        const int t = m >> 4, src_lane = (nl >> 2) * 16 + (m & 15), i = nl & 3;
-        float s0 = 0.f, s1 = 0.f;
+        // thread e -> output (m = e / 16, n_local = e % 16): 16 consecutive threads store one 32-byte row piece
+        for (int e = tid; e < MT * 256; e += SK_THREADS) {
+            const int m = e >> 4, nl = e & 15;
+            const int n = n0 + g * 16 + nl;
+            if (m >= p.M || n >= p.N) continue;
+            const int t = m >> 4, src_lane = (nl >> 2) * 16 + (m & 15), i = nl & 3;
+            float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-        for (int w = 0; w < SK_WAVES; ++w) {
-            s0 += red[w][0][t][i][src_lane];
-            if constexpr (NMAT == 2) s1 += red[w][1][t][i][src_lane];
+            for (int w = 0; w < SK_WAVES; ++w) {
+                s0 += red[w][0][t][i][src_lane];
+                if constexpr (NMAT == 2) s1 += red[w][1][t][i][src_lane];
+            }
+            uint16_t out;
+            if constexpr (MODE == SK_SWIGLU) {
+                const float gv = half_to_f32<DT>(f32_to_half<DT>(s0));
+                const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
+                const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(gv)));
+                out = f32_to_half<DT>(sl * u);
+            } else {
+                float v = s0;
+                if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
+                if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+                out = f32_to_half<DT>(v);
+            }
+            reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
         }
-        uint16_t out;
-        if constexpr (MODE == SK_SWIGLU) {
-            const float g = half_to_f32<DT>(f32_to_half<DT>(s0));
-            const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
-            const float s = half_to_f32<DT>(f32_to_half<DT>(silu_f32(g)));
-            out = f32_to_half<DT>(s * u);
-        } else {
-            float v = s0;
-            if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
-            if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
-            out = f32_to_half<DT>(v);
-        }
-        reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
     }
 }
 
@@ -517,12 +556,51 @@ int launch_gemv(const SkinnyParams &p, hipStream_t s) {
     return TPAMD_OK;
 }
 
+// Column groups per block: as many as keep at least one block per CU and divide N; they pay once x outweighs w.
+inline int pick_cg(const SkinnyParams &p, bool w8, bool swiglu) {
+    if (const char *e = getenv("TPAMD_SKINNY_CG")) return atoi(e) == 4 ? 4 : atoi(e) == 2 ? 2 : 1;
+    if (p.M < (w8 ? 4 : 12)) return 1;  // measured: below this the prefetching single-group kernel is faster
+    if (!swiglu && p.N % 64 == 0 && p.N / 64 >= 256) return 4;
+    if (p.N % 32 == 0 && p.N / 32 >= 256) return 2;
+    return 1;
+}
+
 template <int DT, bool W8, int MODE>
 int launch_skinny(const SkinnyParams &p, hipStream_t s) {
-    const unsigned grid = static_cast<unsigned>((p.N + 15) / 16);
-    if (p.M <= 16) hipLaunchKernelGGL((skinny_kernel<DT, W8, 1, MODE>), dim3(grid), dim3(SK_THREADS), 0, s, p);
-    else if (p.M <= 32) hipLaunchKernelGGL((skinny_kernel<DT, W8, 2, MODE>), dim3(grid), dim3(SK_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((skinny_kernel<DT, W8, 4, MODE>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    int cg = pick_cg(p, W8, MODE == SK_SWIGLU);
+    if (MODE == SK_SWIGLU && cg > 2) cg = 2;  // two matrices per group: registers for 2 groups
+    const unsigned grid = static_cast<unsigned>((p.N + 16 * cg - 1) / (16 * cg));
+    if (cg > 1 && p.M > 32) {
+        // the column-group kernels take 32 rows of x at a time; the weights of the later slabs come from L2 / the
+        // Infinity Cache rather than HBM when they fit
+        for (int m0 = 0; m0 < p.M; m0 += 32) {
+            SkinnyParams q = p;
+            q.x = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
+            q.y = p.y + static_cast<int64_t>(m0) * p.ldy * 2;
+            q.M = p.M - m0 < 32 ? p.M - m0 : 32;
+            const int rc = launch_skinny<DT, W8, MODE>(q, s);
+            if (rc != TPAMD_OK) return rc;
+        }
+        return TPAMD_OK;
+    }
+    if (cg > 1) {
+        TPAMD_REQUIRE(p.N % (16 * cg) == 0, "skinny: N %% %d != 0", 16 * cg);
+        if constexpr (MODE == SK_SWIGLU) {
+            if (p.M <= 16) hipLaunchKernelGGL((skinny_kernel<DT, W8, 1, MODE, 2>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+            else hipLaunchKernelGGL((skinny_kernel<DT, W8, 2, MODE, 2>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+        } else if (cg == 2) {
+            if (p.M <= 16) hipLaunchKernelGGL((skinny_kernel<DT, W8, 1, MODE, 2>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+            else hipLaunchKernelGGL((skinny_kernel<DT, W8, 2, MODE, 2>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+        } else {
+            if (p.M <= 16) hipLaunchKernelGGL((skinny_kernel<DT, W8, 1, MODE, 4>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+            else hipLaunchKernelGGL((skinny_kernel<DT, W8, 2, MODE, 4>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+        }
+    } else {
+        const unsigned grid1 = static_cast<unsigned>((p.N + 15) / 16);
+        if (p.M <= 16) hipLaunchKernelGGL((skinny_kernel<DT, W8, 1, MODE, 1>), dim3(grid1), dim3(SK_THREADS), 0, s, p);
+        else if (p.M <= 32) hipLaunchKernelGGL((skinny_kernel<DT, W8, 2, MODE, 1>), dim3(grid1), dim3(SK_THREADS), 0, s, p);
+        else hipLaunchKernelGGL((skinny_kernel<DT, W8, 4, MODE, 1>), dim3(grid1), dim3(SK_THREADS), 0, s, p);
+    }
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }

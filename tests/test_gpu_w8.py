@@ -70,3 +70,50 @@ def test_falcon_mlp_shard_full_shape():
     want_down = oq.linear_w8_f64(h.float().numpy(), wq2, s2, c2, o2)
     scale_y = float(np.abs(want_down).std())
     torch.testing.assert_close(down.double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * scale_y)
+
+
+@pytest.fixture
+def column_groups(monkeypatch):
+    """Forces the number of 16-column groups per block of the decode kernel (a debugging knob of the library;
+    by default it is chosen from the shape and only large N gets more than one)."""
+    def use(cg):
+        monkeypatch.setenv("TPAMD_SKINNY_CG", str(cg))
+    return use
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [5, 16, 17, 32, 40, 64])
+@pytest.mark.parametrize("cg", [2, 4])
+def test_linear_w8_column_groups_do_not_change_the_result(dtype, M, cg, column_groups):
+    """The same chunks meet the same MFMAs in the same order whatever the grouping: bit-identical results, and
+    both within tolerance of the definition."""
+    N, K, n_out = 192, 1296, 41  # K: 5 whole 256-element chunks and a ragged one
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, dtype, seed=3)
+    args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+            torch.from_numpy(cols.astype(np.int32)).to(DEV), torch.from_numpy(w_out).to(dtype).to(DEV))
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(5)) * 0.1).to(dtype).to(DEV)
+    column_groups(1)
+    one = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
+    column_groups(cg)
+    grouped = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
+    assert torch.equal(one, grouped)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out) + bias.double().cpu().numpy()
+    want = 0.5 * want * (1.0 + np.vectorize(math.erf)(want / math.sqrt(2.0)))
+    sigma = 0.02 * math.sqrt(K + 400 * n_out)
+    torch.testing.assert_close(grouped.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [4, 16, 25, 32])
+@pytest.mark.parametrize("cg", [2, 4])
+def test_16bit_decode_kernels_column_groups(dtype, M, cg, column_groups):
+    N, K = 128, 840
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+    w1, w2 = ((torch.randn(N, K, generator=g) * 0.05).to(dtype).to(DEV) for _ in range(2))
+    column_groups(1)
+    lin1, sw1 = _native.linear(x, w1), _native.swiglu_up(x, w1, w2)
+    column_groups(cg)
+    lin, sw = _native.linear(x, w1), _native.swiglu_up(x, w1, w2)  # the gated pair uses at most 2 groups
+    assert torch.equal(lin, lin1) and torch.equal(sw, sw1)
+    torch.testing.assert_close(lin.float(), torch.nn.functional.linear(x.float(), w1.float()), rtol=2e-2, atol=2e-2 * 0.05 * math.sqrt(K))
