@@ -24,7 +24,7 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
 namespace {
 
 // Largest M served by the weight-streaming kernel; above it the tiled MFMA kernel takes over.
-constexpr int64_t SKINNY_MAX_M = 32;
+constexpr int64_t SKINNY_MAX_M = 16;
 constexpr int64_t SKINNY_W8_SLAB = 64;
 
 // What the MFMA kernels need from 16-bit operands: 16-byte aligned rows of x and w, 8-byte aligned groups of 4

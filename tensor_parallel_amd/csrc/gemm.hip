@@ -12,7 +12,10 @@
 //                       K tile prefetched into registers while the current one is multiplied.
 #include "common.h"
 
+#include <stdlib.h>
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 namespace tpamd {
 namespace {
@@ -33,6 +36,8 @@ struct GemmParams {
     int64_t ldx, ldw, ldy;  // elements
     int act;
     int tiles_m, tiles_n;
+    float *ws;          // split-K: partial tiles, [split][tile][128 w rows][128 x rows] fp32
+    int kt_per_split;   // split-K: K tiles (of 64) per split
 };
 
 constexpr int BK = 64;            // K elements per stage (128 bytes of a row)
@@ -283,13 +288,49 @@ __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// Epilogue of the direct kernel. With w as the first MFMA operand a lane holds D[n = 4*(lane/16) + i][m = lane%16],
-// i = 0..3: four consecutive output columns of one output row, one 8-byte store.
-// acc[a][b]: a = 16-row tile of x (8 per wavefront), b = 16-row tile of w (4 per wavefront; swiglu: 2 gate + 2 up).
+// Four consecutive output columns n..n+3 of one row, from fp32 sums to the packed 16-bit store value.
+// linear: v = bias/activation of g; swiglu: g = gate sums, u = up sums.
 template <int DT, int MODE>
-__device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[8][4], int m_wave, int n_wave, int l16, int lq) {
+__device__ __forceinline__ uint2 finish4(const GemmParams &p, const float (&g)[4], const float (&u)[4], int n) {
+    uint2 o;
+    if constexpr (MODE == MODE_SWIGLU) {
+        // gate and up products rounded to the tensor dtype, then silu and the product each rounded again
+        uint32_t out[2];
 #pragma unroll
-    for (int a = 0; a < 8; ++a) {
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t g2 = pack2_half<DT>(g[2 * j], g[2 * j + 1]);
+            const uint32_t u2 = pack2_half<DT>(u[2 * j], u[2 * j + 1]);
+            const uint32_t s2 = pack2_half<DT>(silu_f32(lo_half_to_f32<DT>(g2)), silu_f32(hi_half_to_f32<DT>(g2)));
+            out[j] = pack2_half<DT>(lo_half_to_f32<DT>(s2) * lo_half_to_f32<DT>(u2), hi_half_to_f32<DT>(s2) * hi_half_to_f32<DT>(u2));
+        }
+        o.x = out[0];
+        o.y = out[1];
+    } else {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = g[j];
+        if (p.bias) {
+            const uint2 braw = *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2);
+            v[0] += lo_half_to_f32<DT>(braw.x); v[1] += hi_half_to_f32<DT>(braw.x);
+            v[2] += lo_half_to_f32<DT>(braw.y); v[3] += hi_half_to_f32<DT>(braw.y);
+        }
+        if (p.act == TPAMD_ACT_GELU) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
+        }
+        o.x = pack2_half<DT>(v[0], v[1]);
+        o.y = pack2_half<DT>(v[2], v[3]);
+    }
+    return o;
+}
+
+// Epilogue of the direct kernels. With w as the first MFMA operand a lane holds D[n = 4*(lane/16) + i][m = lane%16],
+// i = 0..3: four consecutive output columns of one output row, one 8-byte store.
+// acc[a][b]: a = 16-row tile of x (TMX per wavefront), b = 16-row tile of w (4 per wavefront; swiglu: 2 gate + 2 up).
+template <int DT, int MODE, int TMX>
+__device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[TMX][4], int m_wave, int n_wave, int l16, int lq) {
+#pragma unroll
+    for (int a = 0; a < TMX; ++a) {
         const int m = m_wave + a * 16 + l16;
         if (m >= p.M) continue;
         char *yrow = p.y + static_cast<int64_t>(m) * p.ldy * 2;
@@ -297,36 +338,13 @@ __device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[8][
         for (int b = 0; b < (MODE == MODE_SWIGLU ? 2 : 4); ++b) {
             const int n = n_wave + b * 16 + lq * 4;
             if (n >= p.N) continue;  // N is a multiple of 4: the group of 4 is all in or all out
-            uint2 o;
-            if constexpr (MODE == MODE_SWIGLU) {
-                // gate and up products rounded to the tensor dtype, then silu and the product each rounded again
-                uint32_t out[2];
+            float g[4], u[4];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t g2 = pack2_half<DT>(acc[a][b][2 * j], acc[a][b][2 * j + 1]);
-                    const uint32_t u2 = pack2_half<DT>(acc[a][b + 2][2 * j], acc[a][b + 2][2 * j + 1]);
-                    const uint32_t s2 = pack2_half<DT>(silu_f32(lo_half_to_f32<DT>(g2)), silu_f32(hi_half_to_f32<DT>(g2)));
-                    out[j] = pack2_half<DT>(lo_half_to_f32<DT>(s2) * lo_half_to_f32<DT>(u2), hi_half_to_f32<DT>(s2) * hi_half_to_f32<DT>(u2));
-                }
-                o.x = out[0];
-                o.y = out[1];
-            } else {
-                float v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = acc[a][b][j];
-                if (p.bias) {
-                    const uint2 braw = *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2);
-                    v[0] += lo_half_to_f32<DT>(braw.x); v[1] += hi_half_to_f32<DT>(braw.x);
-                    v[2] += lo_half_to_f32<DT>(braw.y); v[3] += hi_half_to_f32<DT>(braw.y);
-                }
-                if (p.act == TPAMD_ACT_GELU) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
-                }
-                o.x = pack2_half<DT>(v[0], v[1]);
-                o.y = pack2_half<DT>(v[2], v[3]);
+            for (int j = 0; j < 4; ++j) {
+                g[j] = acc[a][b][j];
+                u[j] = MODE == MODE_SWIGLU ? acc[a][(b + 2) & 3][j] : 0.f;
             }
-            *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = o;
+            *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = finish4<DT, MODE>(p, g, u, n);
         }
     }
 }
@@ -544,7 +562,228 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
 #undef TPAMD_SUB_B
 #undef TPAMD_DRAIN_BARRIER
 
-    epilogue16<DT, MODE>(p, acc, m0 + wm * 128, n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq);
+    epilogue16<DT, MODE, 8>(p, acc, m0 + wm * 128, n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq);
+}
+
+// gemm_direct128_kernel: 128 x 128 x 64 tiles for problems whose 256 x 256 tiling would leave CUs idle.
+// 4 wavefronts (2 x 2, 64 x-rows by 64 w-rows each), NS LDS stages of 36 KiB: NS = 2 lets two blocks share a CU,
+// NS = 4 gives one block three tiles of look-ahead. Same LDS layout, loads, fragment reads and hand-ordered loop
+// body as the 256 kernel; a K tile is two sub-steps of 16 MFMAs with the tile's barrier between them:
+//   S1 (k 0..31)   reads the fragments of k 32..63;           loads: second half of tile kt + NS - 1
+//   barrier        tile kt+1 has landed (at most (NS-2)*8 younger loads in flight), tile kt is read out
+//   S2 (k 32..63)  reads the fragments of k 0..31 of tile kt+1; loads: first half of tile kt + NS into the freed stage
+// SPLIT: the block covers K tiles [blockIdx.y * kt_per_split, ...) and leaves its fp32 partial tile in p.ws for
+// splitk_finish_kernel.
+template <int DT, int MODE, int NS, bool SPLIT>
+__global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
+    constexpr int BM = 128, BN = 128, WAVES_N = 2, NW = 4;
+    constexpr int BLK = 1152;
+    constexpr int XREG = (BM / 8) * BLK, WREG = (BN / 8) * BLK, STAGE = XREG + WREG;
+    constexpr int XB = BM / 8 / NW, WB = BN / 8 / NW;
+    static_assert(XB == 4 && WB == 4, "8 loads per wavefront per tile");
+    static_assert(NS == 2 || NS == 4, "stage index is taken with a mask");
+
+    extern __shared__ __align__(16) char smem[];
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * (MODE == MODE_SWIGLU ? BN / 2 : BN);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l16 = lane & 15, lq = lane >> 4;
+
+    const int rb = lane >> 3, slot = lane & 7;
+    const int lchunk = slot ^ rb;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
+    const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
+    const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : w_base;
+    uint32_t x_off[XB], w_off[WB];
+#pragma unroll
+    for (int i = 0; i < XB; ++i) {
+        int r = (wave_s + i * NW) * 8 + rb;
+        r = m0 + r < p.M ? r : p.M - 1 - m0;
+        x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < WB; ++i) {
+        int tr = (wave_s + i * NW) * 8 + rb;
+        if constexpr (MODE == MODE_SWIGLU) tr = tr < BN / 2 ? tr : tr - BN / 2;  // gate rows, then up rows
+        tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
+        w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
+    }
+    const int x_rows = p.M - m0 < BM ? p.M - m0 : BM;
+    const int w_rows = p.N - n0 < BN ? p.N - n0 : BN;
+    const uint32_t x_extent = static_cast<uint32_t>(x_rows - 1) * static_cast<uint32_t>(p.ldx * 2) + static_cast<uint32_t>(p.K) * 2;
+    const uint32_t w_extent = static_cast<uint32_t>(w_rows - 1) * static_cast<uint32_t>(p.ldw * 2) + static_cast<uint32_t>(p.K) * 2;
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x_base, x_extent);
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(w_base, w_extent);
+    const __amdgpu_buffer_rsrc_t w2_rsrc = make_rsrc(w2_base, w_extent);
+
+    // this block's K tiles: [kt0, kt0 + nk)
+    const int KT = p.K / BK;
+    const int kt0 = SPLIT ? static_cast<int>(blockIdx.y) * p.kt_per_split : 0;
+    const int nk = SPLIT ? (KT - kt0 < p.kt_per_split ? KT - kt0 : p.kt_per_split) : KT;
+    const int last = nk - 1;
+    // loads of local tile j (clamped to the last one: such loads refill a stage nobody reads any more and keep
+    // the loop free of branches)
+    auto gx = [&](int i, int j) {
+        const int jj = j < last ? j : last;
+        buffer_load16_to_lds(x_rsrc, x_off[i], static_cast<uint32_t>(kt0 + jj) * (BK * 2), smem + (j & (NS - 1)) * STAGE + (wave_s + i * NW) * BLK);
+    };
+    auto gw = [&](int i, int j) {
+        const int jj = j < last ? j : last;
+        const bool up = MODE == MODE_SWIGLU && (wave_s + i * NW) * 8 >= BN / 2;  // i >= 2: known at compile time
+        buffer_load16_to_lds(up ? w2_rsrc : w_rsrc, w_off[i], static_cast<uint32_t>(kt0 + jj) * (BK * 2),
+                             smem + (j & (NS - 1)) * STAGE + XREG + (wave_s + i * NW) * BLK);
+    };
+
+    constexpr int T16 = 2 * BLK;
+    constexpr int WT1 = T16;
+    constexpr int WT2 = MODE == MODE_SWIGLU ? (BN / 2 / 8) * BLK : 2 * T16;  // swiglu: first up tile, 64 staged rows on
+    constexpr int WT3 = WT2 + T16;
+    int x_rd0, w_rd0;
+    {
+        const int r = wm * 64 + l16;
+        x_rd0 = (r >> 3) * BLK + (r & 7) * 128;
+        const int row = (MODE == MODE_SWIGLU ? wn * 32 : wn * 64) + l16;
+        w_rd0 = XREG + (row >> 3) * BLK + (row & 7) * 128;
+    }
+    int kk_off[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) kk_off[kk] = ((kk * 4 + lq) ^ (l16 & 7)) * 16;
+
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 xf[2][4], wf[2][4];
+    const uint32_t smem_base = lds_addr_of(smem);
+#define TPAMD_SB __builtin_amdgcn_sched_barrier(0)
+#define TPAMD_WAIT(N, reg) asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(reg))
+#define TPAMD_MFMA(S, a, b) acc[a][b] = mfma16<DT>(wf[S][b], xf[S][a], acc[a][b])
+#define TPAMD_ROW(S, a) TPAMD_MFMA(S, a, 0); TPAMD_MFMA(S, a, 1); TPAMD_MFMA(S, a, 2); TPAMD_MFMA(S, a, 3)
+    // 16 MFMAs on fragment set MS (read in the order x0 w0 w1 w2 w3 x1 x2 x3); the same 8 reads of (stage_off, kk)
+    // into set RS follow the first 8 MFMAs one by one; L0..L3: loads or nothing
+#define TPAMD_SUB(MS, RS, stage_off, kk, L0, L1, L2, L3)                                                            \
+    {                                                                                                               \
+        const uint32_t xa = smem_base + (stage_off) + x_rd0 + kk_off[kk];                                           \
+        const uint32_t wa = smem_base + (stage_off) + w_rd0 + kk_off[kk];                                           \
+        TPAMD_SB;                                                                                                   \
+        TPAMD_WAIT(6, xf[MS][0]); TPAMD_WAIT(6, wf[MS][0]); TPAMD_SB;                                               \
+        TPAMD_MFMA(MS, 0, 0); TPAMD_SB; xf[RS][0] = lds_read16<0>(xa); TPAMD_SB;                                    \
+        TPAMD_WAIT(6, wf[MS][1]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(MS, 0, 1); TPAMD_SB; wf[RS][0] = lds_read16<0>(wa); TPAMD_SB;                                    \
+        TPAMD_WAIT(6, wf[MS][2]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(MS, 0, 2); TPAMD_SB; wf[RS][1] = lds_read16<WT1>(wa); TPAMD_SB;                                  \
+        TPAMD_WAIT(6, wf[MS][3]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(MS, 0, 3); TPAMD_SB; wf[RS][2] = lds_read16<WT2>(wa); TPAMD_SB;                                  \
+        TPAMD_WAIT(6, xf[MS][1]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(MS, 1, 0); TPAMD_SB; wf[RS][3] = lds_read16<WT3>(wa); TPAMD_SB;                                  \
+        TPAMD_MFMA(MS, 1, 1); TPAMD_SB; xf[RS][1] = lds_read16<1 * T16>(xa); TPAMD_SB;                              \
+        TPAMD_MFMA(MS, 1, 2); TPAMD_SB; xf[RS][2] = lds_read16<2 * T16>(xa); TPAMD_SB;                              \
+        TPAMD_MFMA(MS, 1, 3); TPAMD_SB; xf[RS][3] = lds_read16<3 * T16>(xa); TPAMD_SB;                              \
+        TPAMD_WAIT(9, xf[MS][2]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(MS, 2, 0); TPAMD_MFMA(MS, 2, 1); TPAMD_SB; L0; TPAMD_SB;                                         \
+        TPAMD_MFMA(MS, 2, 2); TPAMD_MFMA(MS, 2, 3); TPAMD_SB; L1; TPAMD_SB;                                         \
+        TPAMD_WAIT(8, xf[MS][3]); TPAMD_SB;                                                                         \
+        TPAMD_MFMA(MS, 3, 0); TPAMD_MFMA(MS, 3, 1); TPAMD_SB; L2; TPAMD_SB;                                         \
+        TPAMD_MFMA(MS, 3, 2); TPAMD_MFMA(MS, 3, 3); TPAMD_SB; L3; TPAMD_SB;                                         \
+    }
+    // the tile's barrier: all fragment reads of this wavefront done, all but the loads of the NS-2 youngest tiles landed
+#define TPAMD_TILE_BARRIER()                                                                                        \
+    if constexpr (NS == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");                 \
+    else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+    // prologue: tiles 0 .. NS-2 in flight, tile 0 landed, its first fragments read, first half of tile NS-1 issued
+#pragma unroll
+    for (int j = 0; j < NS - 1; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) gx(i, j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) gw(i, j);
+    }
+    TPAMD_TILE_BARRIER();
+    {
+        const uint32_t xa = smem_base + x_rd0 + kk_off[0];
+        const uint32_t wa = smem_base + w_rd0 + kk_off[0];
+        xf[0][0] = lds_read16<0>(xa);
+        wf[0][0] = lds_read16<0>(wa);
+        wf[0][1] = lds_read16<WT1>(wa);
+        wf[0][2] = lds_read16<WT2>(wa);
+        wf[0][3] = lds_read16<WT3>(wa);
+        xf[0][1] = lds_read16<1 * T16>(xa);
+        xf[0][2] = lds_read16<2 * T16>(xa);
+        xf[0][3] = lds_read16<3 * T16>(xa);
+    }
+    gx(0, NS - 1); gx(1, NS - 1); gx(2, NS - 1); gx(3, NS - 1);
+    for (int j = 0; j < last; ++j) {
+        const int cur = (j & (NS - 1)) * STAGE, nxt = ((j + 1) & (NS - 1)) * STAGE;
+        TPAMD_SUB(0, 1, cur, 1, gw(0, j + NS - 1), gw(1, j + NS - 1), gw(2, j + NS - 1), gw(3, j + NS - 1));
+        TPAMD_TILE_BARRIER();
+        TPAMD_SUB(1, 0, nxt, 0, gx(0, j + NS), gx(1, j + NS), gx(2, j + NS), gx(3, j + NS));
+    }
+    {
+        const int cur = (last & (NS - 1)) * STAGE;
+        TPAMD_SUB(0, 1, cur, 1, (void)0, (void)0, (void)0, (void)0);
+        // nothing may still be on its way into LDS when the block ends (the memory is handed to the next block)
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        TPAMD_WAIT(0, xf[1][0]); TPAMD_WAIT(0, xf[1][1]); TPAMD_WAIT(0, xf[1][2]); TPAMD_WAIT(0, xf[1][3]);
+        TPAMD_WAIT(0, wf[1][0]); TPAMD_WAIT(0, wf[1][1]); TPAMD_WAIT(0, wf[1][2]); TPAMD_WAIT(0, wf[1][3]);
+        TPAMD_ROW(1, 0); TPAMD_ROW(1, 1); TPAMD_ROW(1, 2); TPAMD_ROW(1, 3);
+    }
+#undef TPAMD_SB
+#undef TPAMD_WAIT
+#undef TPAMD_MFMA
+#undef TPAMD_ROW
+#undef TPAMD_SUB
+#undef TPAMD_TILE_BARRIER
+
+    if constexpr (SPLIT) {
+        // partial tile [w row][x row]: a lane's 4 values are 4 w rows of one x row; 16 lanes cover 16 consecutive x rows
+        const int tile = tile_m * p.tiles_n + tile_n;
+        float *ws = p.ws + (static_cast<int64_t>(blockIdx.y) * p.tiles_m * p.tiles_n + tile) * (BM * BN);
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int wr = (MODE == MODE_SWIGLU ? (b >> 1) * 64 + wn * 32 + (b & 1) * 16 : wn * 64 + b * 16) + lq * 4;
+                const int xr = wm * 64 + a * 16 + l16;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ws[(wr + i) * BM + xr] = acc[a][b][i];
+            }
+    } else {
+        epilogue16<DT, MODE, 4>(p, acc, m0 + wm * 64, n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq);
+    }
+}
+
+// Sums the split-K partial tiles of gemm_direct128_kernel and applies the epilogue. One thread = one x row and 4
+// consecutive output columns; the 128 x rows of a tile are the contiguous axis of a partial tile, so a block of
+// 256 threads reads two runs of 512 contiguous bytes per w row and split. Grid: (column-group pairs, tiles).
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(GemmParams p, int splits) {
+    const int tile = blockIdx.y;
+    const int tile_m = tile / p.tiles_n, tile_n = tile % p.tiles_n;
+    const int64_t ntiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    const int xr = threadIdx.x & 127, grp = blockIdx.x * 2 + (threadIdx.x >> 7);
+    const int m = tile_m * 128 + xr;
+    const int n = tile_n * (MODE == MODE_SWIGLU ? 64 : 128) + grp * 4;
+    if (m >= p.M || n >= p.N) return;
+    float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < splits; ++sp) {
+        const float *ws = p.ws + (sp * ntiles + tile) * (128 * 128);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            g[i] += ws[(grp * 4 + i) * 128 + xr];
+            if constexpr (MODE == MODE_SWIGLU) u[i] += ws[(64 + grp * 4 + i) * 128 + xr];
+        }
+    }
+    *reinterpret_cast<uint2 *>(p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2) = finish4<DT, MODE>(p, g, u, n);
 }
 
 // ---- any dtype, any alignment: LDS-tiled FMA kernel, 64x64 tile, 256 threads, 4x4 outputs per thread ---------
@@ -672,16 +911,110 @@ int launch_direct(GemmParams p, hipStream_t s) {
 
 }  // namespace
 
+// Split-K scratch: one buffer per device, allocated at first use with room for any split this file chooses, kept
+// until the process ends. Work on one stream is ordered, so consecutive calls can share it (callers that spread
+// such GEMMs over several streams of one device have to order those streams themselves); the mutex keeps the two
+// launches of a call together when several host threads enqueue onto one stream. *out stays NULL when there is no
+// buffer yet and the stream is being captured (allocating is not allowed then): the caller runs unsplit.
+inline std::mutex &splitk_mutex() {
+    static std::mutex m;
+    return m;
+}
+inline int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
+    struct Entry { int dev; void *ptr; size_t bytes; };
+    static std::vector<Entry> cache;  // guarded by splitk_mutex(), held by the caller
+    *out = nullptr;
+    for (Entry &e : cache)
+        if (e.dev == dev) {
+            if (e.bytes >= need) *out = e.ptr;  // `reserve` covers every shape; a larger need runs unsplit
+            return TPAMD_OK;
+        }
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    TPAMD_HIP(hipStreamIsCapturing(stream, &capturing));
+    if (capturing != hipStreamCaptureStatusNone) return TPAMD_OK;
+    const size_t bytes = need > reserve ? need : reserve;
+    void *ptr = nullptr;
+    TPAMD_HIP(hipMalloc(&ptr, bytes));
+    cache.push_back(Entry{dev, ptr, bytes});
+    *out = ptr;
+    return TPAMD_OK;
+}
+
+template <int DT, int MODE, int NS, bool SPLIT>
+int configure128(int dev) {
+    static thread_local int configured_dev = -1;
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct128_kernel<DT, MODE, NS, SPLIT>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, NS * 32 * 1152));
+        configured_dev = dev;
+    }
+    return TPAMD_OK;
+}
+
+// 128 x 128 tiles; split over K (fp32 partial tiles in stream-ordered scratch memory, then one finishing pass)
+// when the tiles alone would not give every CU two blocks.
+template <int DT, int MODE>
+int launch_direct128(GemmParams p, int cus, hipStream_t s) {
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    p.tiles_m = (p.M + 127) / 128;
+    constexpr int BN_OUT = MODE == MODE_SWIGLU ? 64 : 128;
+    p.tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+    const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    TPAMD_REQUIRE(tiles < 65536 || tiles >= 2 * cus, "gemm: too many tiles");  // the finishing pass indexes tiles with blockIdx.y
+    TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
+    const int KT = p.K / 64;
+    int splits = 1;
+    if (const char *e = getenv("TPAMD_GEMM_SPLITK")) splits = atoi(e);
+    else if (tiles < 2 * cus) splits = static_cast<int>((2 * cus + tiles - 1) / tiles);
+    if (splits > 8) splits = 8;
+    if (splits > KT / 8) splits = KT / 8 > 0 ? KT / 8 : 1;  // at least 8 K tiles per split
+    if (splits < 1) splits = 1;
+    p.kt_per_split = (KT + splits - 1) / splits;
+    splits = (KT + p.kt_per_split - 1) / p.kt_per_split;   // no empty split
+    constexpr int LDS2 = 2 * 32 * 1152;
+    if (splits > 1) {
+        int rc = configure128<DT, MODE, 2, true>(dev);
+        if (rc != TPAMD_OK) return rc;
+        const size_t ws_bytes = static_cast<size_t>(splits) * tiles * 128 * 128 * sizeof(float);
+        // the scratch buffer is ours until both launches are enqueued
+        std::lock_guard<std::mutex> hold(splitk_mutex());
+        void *ws = nullptr;
+        rc = splitk_scratch(dev, s, ws_bytes, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
+        if (rc != TPAMD_OK) return rc;
+        if (ws != nullptr) {
+            p.ws = static_cast<float *>(ws);
+            hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true>), dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits)), dim3(256), LDS2, s, p);
+            TPAMD_HIP(hipGetLastError());
+            hipLaunchKernelGGL((splitk_finish_kernel<DT, MODE>), dim3(MODE == MODE_SWIGLU ? 8 : 16, static_cast<unsigned>(tiles)), dim3(256), 0, s, p, splits);
+            TPAMD_HIP(hipGetLastError());
+            return TPAMD_OK;
+        }
+    }
+    int rc = configure128<DT, MODE, 2, false>(dev);
+    if (rc != TPAMD_OK) return rc;
+    hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, false>), dim3(static_cast<unsigned>(tiles)), dim3(256), LDS2, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 // Prefill-sized dispatch; called by linear.hip once M is above the skinny range.
 template <int DT>
 int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    // the direct kernels address a tile with 32-bit byte offsets from the tile origin and step K in tiles of 64
+    const bool direct_ok = p.K % 64 == 0 && p.K >= 64 && p.ldx < (1ll << 22) && p.ldw < (1ll << 22);
     // 256x256 tiles once they fill the chip at least about once, else 128x128 tiles.
     const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
-    if (big_tiles >= 200) {
-        // the direct kernel addresses a tile with 32-bit byte offsets from the tile origin
-        if (p.K % 64 == 0 && p.K >= 64 && p.ldx < (1ll << 22) && p.ldw < (1ll << 22)) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
-        return swiglu ? launch_gemm<DT, MODE_SWIGLU, 256, 256, 2, 4>(p, s) : launch_gemm<DT, MODE_LINEAR, 256, 256, 2, 4>(p, s);
+    const char *force = getenv("TPAMD_GEMM_TILE");
+    const bool big = force ? atoi(force) == 256 : big_tiles >= 200;
+    if (direct_ok) {
+        if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
+        return swiglu ? launch_direct128<DT, MODE_SWIGLU>(p, cus, s) : launch_direct128<DT, MODE_LINEAR>(p, cus, s);
     }
+    if (big) return swiglu ? launch_gemm<DT, MODE_SWIGLU, 256, 256, 2, 4>(p, s) : launch_gemm<DT, MODE_LINEAR, 256, 256, 2, 4>(p, s);
     return swiglu ? launch_gemm<DT, MODE_SWIGLU, 128, 128, 2, 2>(p, s) : launch_gemm<DT, MODE_LINEAR, 128, 128, 2, 2>(p, s);
 }
 
