@@ -163,3 +163,43 @@ def test_llama_mlp_shard_prefill_4096_sampled_rows():
     assert (sub != y[1024:1536]).float().mean().item() < 0.01
     # the same tiling twice: bit-identical
     assert torch.equal(_native.linear(h[1024:1536].contiguous(), wd), sub)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(40, 136, 5504), (130, 260, 1536), (300, 64, 2048), (17, 512, 1024)])
+@pytest.mark.parametrize("splits", [1, 3, 8])
+def test_split_k_tiles(dtype, M, N, K, splits, monkeypatch):
+    """The 128 x 128 tiling with K split `splits` ways (forced through the library's debugging knob; by default
+    the split is chosen from the tile count): ragged last split, tile rows past M, tile columns past N, bias and
+    GELU applied by the finishing pass."""
+    monkeypatch.setenv("TPAMD_GEMM_SPLITK", str(splits))
+    monkeypatch.setenv("TPAMD_GEMM_TILE", "128")
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
+    want = F.gelu(F.linear(x.float(), w.float(), b.float()))
+    check_half(got, want, K)
+    w2 = rnd((N, K), 5, 0.02, dtype)
+    h = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+
+
+def test_mid_sized_linear_inside_a_hip_graph():
+    """A split-K GEMM recorded into a HIP graph after a warm-up call (which allocates the library's scratch buffer)
+    replays to the eager result every time, with eager work in between."""
+    M, N, K = 64, 512, 4096
+    x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
+    eager = _native.linear(x, w)
+    torch.cuda.synchronize()
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out.copy_(_native.linear(x, w))
+    for i in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        assert torch.equal(_native.linear(x, w), eager)  # eager work between replays
