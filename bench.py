@@ -211,7 +211,20 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
         except Exception as e:  # noqa: BLE001 - the eager figure stands on its own
             entry["graph"] = {"error": str(e)[:200]}
         extra[f"decode_m{m}"] = entry
-    extra["w8_decode_m1"] = w8_decode(torch, _native, dev)
+    # the same shard at M = 512 (the prefill size of the configuration list between decode and the headline)
+    x512 = torch.randn(512, D_MODEL, device=dev).to(torch.bfloat16)
+
+    def fn512(i):
+        wg, wu, wd = sets[i % n_sets]
+        return _native.linear(_native.swiglu_up(x512, wg, wu), wd)
+
+    us = _time_us(torch, fn512, 10, 50)
+    flops = 6.0 * 512 * D_MODEL * FFN_SHARD
+    extra["prefill_m512"] = {"us_per_step": us, "tokens_per_s": 512 / us * 1e6, "TFLOPs": flops / us / 1e6,
+                             "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS, "algorithmic_flops": flops,
+                             "step": "swiglu_up + down (128x128 tiles, K split)"}
+    for m in (1, 32):
+        extra[f"w8_decode_m{m}"] = w8_decode(torch, _native, dev, m)
 
     from types import SimpleNamespace
 
@@ -244,8 +257,8 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     return extra
 
 
-def w8_decode(torch, _native, dev) -> dict:
-    """BASELINE config 5 at batch 1: int8 weight-only rank-0 shard of a Falcon-40B-shape MLP (up [16384 x 8192] + GELU,
+def w8_decode(torch, _native, dev, m=1) -> dict:
+    """BASELINE config 5 at batch m: int8 weight-only rank-0 shard of a Falcon-40B-shape MLP (up [16384 x 8192] + GELU,
     down [8192 x 16384], per-row scales, 41 / 82 outlier columns in fp16), fp16 activations. HBM-bound."""
     d, f, n_sets = 8192, 16384, 3
     g = torch.Generator(device=dev).manual_seed(0)
@@ -259,7 +272,7 @@ def w8_decode(torch, _native, dev) -> dict:
 
     ups = [make(f, d, 41) for _ in range(n_sets)]
     downs = [make(d, f, 82) for _ in range(n_sets)]
-    x = torch.randn(1, d, device=dev, generator=g).half()
+    x = torch.randn(m, d, device=dev, generator=g).half()
 
     def fn(i):
         u, dn = ups[i % n_sets], downs[i % n_sets]
@@ -268,7 +281,7 @@ def w8_decode(torch, _native, dev) -> dict:
 
     us = _time_us(torch, fn, 10, 100)
     by = 2.0 * f * d + (f * 41 + d * 82) * 2.0 + (f + d) * 4.0
-    return {"us_per_step": us, "tokens_per_s": 1e6 / us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
+    return {"us_per_step": us, "tokens_per_s": m * 1e6 / us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
             "algorithmic_bytes": by, "launch": "eager"}
 
 

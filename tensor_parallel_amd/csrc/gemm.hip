@@ -964,11 +964,25 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     TPAMD_REQUIRE(tiles < 65536 || tiles >= 2 * cus, "gemm: too many tiles");  // the finishing pass indexes tiles with blockIdx.y
     TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
     const int KT = p.K / 64;
+    // Split factor from a small cost model fitted on this part (microseconds): a block that has its CU to itself
+    // takes 0.8 per K tile, two blocks sharing a CU 1.0 each, blocks beyond two per CU wait for the next round; the
+    // partial tiles cost 3 + 0.18 per MB (written, read back and finished by a second launch).
     int splits = 1;
-    if (const char *e = getenv("TPAMD_GEMM_SPLITK")) splits = atoi(e);
-    else if (tiles < 2 * cus) splits = static_cast<int>((2 * cus + tiles - 1) / tiles);
+    if (const char *e = getenv("TPAMD_GEMM_SPLITK")) {
+        splits = atoi(e);
+    } else {
+        double best = 1e30;
+        for (int sp = 1; sp <= 8; ++sp) {
+            const int kt = (KT + sp - 1) / sp;
+            if (sp > 1 && (kt < 4 || tiles * sp > 4ll * cus)) break;  // too little K per split / more than the scratch buffer holds
+            const double units = static_cast<double>(tiles) * sp;
+            const double rounds = units <= cus ? 1.0 : static_cast<double>((static_cast<int64_t>(units) + 2 * cus - 1) / (2 * cus));
+            const double t = rounds * kt * (units <= cus ? 0.8 : 1.0) + (sp > 1 ? 3.0 + units * 0.065536 * 0.18 : 0.0);
+            if (t < best) { best = t; splits = sp; }
+        }
+    }
     if (splits > 8) splits = 8;
-    if (splits > KT / 8) splits = KT / 8 > 0 ? KT / 8 : 1;  // at least 8 K tiles per split
+    if (splits > KT) splits = KT;
     if (splits < 1) splits = 1;
     p.kt_per_split = (KT + splits - 1) / splits;
     splits = (KT + p.kt_per_split - 1) / p.kt_per_split;   // no empty split
