@@ -151,6 +151,25 @@ int tpamd_linear(const void *x_dev, const void *w_dev, const void *bias_dev, voi
 int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void *wu_dev, void *h_dev, int64_t M, int64_t N,
                     int64_t K, int64_t ldx, int64_t ldw, int64_t ldh, int dtype, void *stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * Rank-local attention core: out = softmax(scale * q k^T [+ causal mask]) v over the heads this rank owns.
+ * In the reference this is the attention of the wrapped transformers module, run per rank by
+ * TensorParallelWrapper.forward (src/tensor_parallel/wrapper.py:69-72) on the rank's share of the heads (head
+ * counts divided by the attr rules, e.g. src/tensor_parallel/slicing_configs.py:382-389 for Llama, :414-433 for
+ * RefinedWeb/Falcon with grouped key/value heads); the reference itself contains no attention code.
+ *   q   [B, Hq, Sq, D], k / v [B, Hkv, Skv, D], out [B, Sq, Hq, D]; Hq a multiple of Hkv (grouped-query: query head h
+ *   uses key/value head h / (Hq / Hkv)); D (contiguous) is 64 or 128; dtype BF16 or F16, fp32 accumulation.
+ *   strides: 12 element strides, {q batch, q head, q position, k batch, k head, k position, v batch, v head,
+ *   v position, out batch, out position, out head}.
+ *   causal != 0: query position i sees keys j <= i + (Skv - Sq) (the new tokens are the last Sq positions of the
+ *   key range: prefill with Sq == Skv, decode with Sq == 1). No other mask, no dropout.
+ * Few rows and many keys (decode) are split over the keys with partials in the per-device scratch buffer
+ * described above. Returns TPAMD_ERR_UNSUPPORTED for another head_dim or unaligned rows.
+ * ---------------------------------------------------------------------------------------------- */
+int tpamd_attention(const void *q_dev, const void *k_dev, const void *v_dev, void *out_dev, int64_t B, int64_t Hq,
+                    int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal,
+                    int dtype, void *stream);
+
 /* Weight-only int8 shard Linear with fp16/bf16 outlier columns:
  *   y[m,n] = act( scale[n] * sum_k x[m,k]*wq[n,k]  +  sum_j x[m,outlier_idx[j]] * w_out[n,j]  + bias[n] )
  * wq is int8 [N,K] (zero in the outlier columns), scale fp32 [N], outlier_idx int32 [n_out] (sorted,

@@ -28,6 +28,7 @@ EXPORTS = (
     "tpamd_linear",
     "tpamd_swiglu_up",
     "tpamd_linear_w8",
+    "tpamd_attention",
 )
 
 ABI_VERSION = 1
@@ -83,6 +84,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_linear.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
     lib.tpamd_swiglu_up.restype = ci
     lib.tpamd_swiglu_up.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+    lib.tpamd_attention.restype = ci
+    lib.tpamd_attention.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, c.POINTER(i64), c.c_float, ci, ci, vp]
     lib.tpamd_linear_w8.restype = ci
     lib.tpamd_linear_w8.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, i64, i64, i64, i64, i64, i64, i64, ci, ci, vp]
 
@@ -299,6 +302,31 @@ def swiglu_up(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor) -> torch.Tens
             "tpamd_swiglu_up",
         )
     return h.view(*x.shape[:-1], N)
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None, causal: bool = True) -> torch.Tensor:
+    """softmax(scale * q k^T [+ causal]) v. q [B, Hq, Sq, D], k / v [B, Hkv, Skv, D] -> [B, Sq, Hq, D] (the layout the
+    attention output projection consumes). Grouped-query heads when Hq > Hkv; causal is aligned to the END of the key
+    range (query i sees keys j <= i + Skv - Sq)."""
+    require_device(q, "attention")
+    if not (q.dtype == k.dtype == v.dtype) or q.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("attention: q, k, v must share bfloat16 or float16")
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
+        raise ValueError(f"attention: shapes q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit")
+    B, Hq, Sq, D = q.shape
+    Hkv, Skv = k.shape[1], k.shape[2]
+    q, k, v = (t if t.stride(3) == 1 else t.contiguous() for t in (q, k, v))
+    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    strides = (ctypes.c_int64 * 12)(q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                                    v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2))
+    with torch.cuda.device(q.device):
+        _check(
+            lib().tpamd_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, Hq, Hkv, Sq, Skv, D, strides,
+                                  float(scale if scale is not None else D ** -0.5), 1 if causal else 0, dtype_code(q.dtype),
+                                  ctypes.c_void_p(current_stream_ptr(q.device))),
+            "tpamd_attention",
+        )
+    return out
 
 
 def linear_w8(x: torch.Tensor, wq: torch.Tensor, scale_: torch.Tensor, outlier_idx: Optional[torch.Tensor],

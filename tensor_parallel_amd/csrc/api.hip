@@ -21,6 +21,9 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
                     int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
                     hipStream_t s);
 
+int attention_dispatch(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq,
+                       int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal, int dtype, hipStream_t s);
+
 namespace {
 
 // Largest M served by the weight-streaming kernel; above it the tiled MFMA kernel takes over.
@@ -82,6 +85,30 @@ extern "C" int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void
         return skinny_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw, ldh, 0,
                                dtype, TPAMD_ACT_NONE, true, false, s);
     return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true, !fast, s);
+}
+
+extern "C" int tpamd_attention(const void *q_dev, const void *k_dev, const void *v_dev, void *out_dev, int64_t B, int64_t Hq,
+                               int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal,
+                               int dtype, void *stream) {
+    const char *who = "tpamd_attention";
+    TPAMD_REQUIRE(dtype == TPAMD_BF16 || dtype == TPAMD_F16, "%s: dtype must be BF16 or F16", who);
+    TPAMD_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Sq >= 0 && Skv >= 0, "%s: bad dimension", who);
+    TPAMD_REQUIRE(Hq % Hkv == 0, "%s: %lld query heads are not a multiple of %lld key/value heads", who, (long long)Hq, (long long)Hkv);
+    TPAMD_REQUIRE(strides != nullptr, "%s: strides is NULL", who);
+    TPAMD_REQUIRE(!causal || Skv >= Sq, "%s: causal attention needs Skv >= Sq", who);
+    if (B == 0 || Sq == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(Skv > 0, "%s: no keys", who);
+    TPAMD_REQUIRE(q_dev && k_dev && v_dev && out_dev, "%s: null pointer", who);
+    TPAMD_REQUIRE(Hq * Sq / Hkv < (1ll << 30) && Skv < (1ll << 30), "%s: sequence too long", who);
+    bool ok = (D == 64 || D == 128) && aligned(q_dev, 16) && aligned(k_dev, 16) && aligned(v_dev, 16) && aligned(out_dev, 8);
+    for (int i = 0; i < 9; ++i) ok = ok && strides[i] % 8 == 0;   // 16-byte loads of q, k, v rows
+    for (int i = 9; i < 12; ++i) ok = ok && strides[i] % 4 == 0;  // 8-byte stores
+    if (!ok) {
+        set_error("%s: head_dim must be 64 or 128 and rows 16-byte aligned", who);
+        return TPAMD_ERR_UNSUPPORTED;
+    }
+    return attention_dispatch(q_dev, k_dev, v_dev, out_dev, B, Hq, Hkv, Sq, Skv, D, strides, scale, causal, dtype,
+                              static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,

@@ -1,0 +1,310 @@
+// Rank-local attention core: softmax(scale * Q K^T + causal mask) V for the heads one rank owns, grouped-query
+// layout (Hq = G * Hkv query heads share Hkv key/value heads), bf16/f16, head_dim 64 or 128.
+//
+// One kernel serves prefill and decode. The query rows that share a key/value head are put on one axis,
+// row = g * Sq + sq (g = query head inside the group): at decode (Sq = 1, G = 16) the 16 heads of a group fill
+// one MFMA tile and K / V of that head are read once for all of them; at prefill a tile is 64 consecutive
+// positions of one head. A block (4 wavefronts, 16 rows each) walks the keys in tiles of 64:
+//   S^T = K Q^T   v_mfma_f32_16x16x32 with K rows as the first operand: a lane then holds, for ONE query row,
+//                 4 keys per 16-key tile, so the row maximum / sum need two cross-lane steps only,
+//   online softmax in exp2 domain (scale * log2 e folded in),
+//   O^T += V^T P^T the lane's 8 probabilities of two key tiles are exactly the second operand of the next MFMA
+//                 (the K index of an MFMA may be permuted freely as long as both operands agree), the first
+//                 operand comes from a transposed copy of the V tile in LDS.
+// O^T leaves a lane with 4 consecutive head-dim elements of one query row: one 8-byte store into [B, Sq, Hq, D].
+//
+// Long key ranges with few rows (decode) are split over blockIdx.z; every split leaves (m, l, unnormalised O) in
+// the per-device scratch buffer and attention_combine_kernel merges them.
+#include "common.h"
+
+namespace tpamd {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
+    if constexpr (DT == TPAMD_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+struct AttnParams {
+    const char *q, *k, *v;
+    char *o;
+    float *part;  // split partials: [split][B*Hkv][rows_pad][D + 4] fp32 (O, then m, l, 2 unused)
+    int B, Hq, Hkv, Sq, Skv, G;
+    int64_t q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_ss, o_sh;  // elements; head_dim is contiguous
+    float scale_log2;  // scale * log2(e)
+    int causal;        // query position sq sees keys j <= sq + (Skv - Sq)
+    int nsplit, keys_per_split, rows_pad;
+};
+
+constexpr int AT_ROWS = 64;   // query rows per block
+constexpr int AT_KEYS = 64;   // keys per tile
+
+template <int DT, int D>
+__global__ __launch_bounds__(256) void attention_kernel(AttnParams p) {
+    constexpr int KP = D * 2 + 16;        // K tile row pitch (bytes): conflict-free 16-byte reads
+    constexpr int VP = AT_KEYS * 2 + 8;   // V^T tile row pitch (bytes), 8-byte aligned
+    constexpr int DT16 = D / 16, DK = D / 32;
+    __shared__ __align__(16) char ks[AT_KEYS * KP];
+    __shared__ __align__(16) char vt[D * VP];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int bh = blockIdx.y, b = bh / p.Hkv, hkv = bh % p.Hkv;
+    const int nrows = p.G * p.Sq;
+    const int row0 = blockIdx.x * AT_ROWS;
+    const int row = row0 + wave * 16 + l16;
+    const bool row_ok = row < nrows;
+    const int g = row_ok ? row / p.Sq : 0, sq = row_ok ? row % p.Sq : 0;
+    const int head = hkv * p.G + g;
+
+    // ---- Q fragments (second MFMA operand): lane = (query row l16, 8 head-dim elements at 32*kk + 8*lq)
+    uint4 qf[DK];
+    {
+        const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(head) * p.q_sh + static_cast<int64_t>(sq) * p.q_ss) * 2;
+#pragma unroll
+        for (int kk = 0; kk < DK; ++kk) qf[kk] = row_ok ? *reinterpret_cast<const uint4 *>(qrow + (32 * kk + 8 * lq) * 2) : make_uint4(0, 0, 0, 0);
+    }
+
+    // ---- key range of this block
+    int k_begin = blockIdx.z * p.keys_per_split;
+    int k_end = k_begin + p.keys_per_split < p.Skv ? k_begin + p.keys_per_split : p.Skv;
+    const int shift = p.Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
+    if (p.causal) {
+        // the largest position in this tile of rows (a tile that straddles two heads contains position Sq - 1)
+        const int last_row = row0 + AT_ROWS - 1 < nrows - 1 ? row0 + AT_ROWS - 1 : nrows - 1;
+        const int max_sq = (row0 / p.Sq != last_row / p.Sq) ? p.Sq - 1 : last_row % p.Sq;
+        const int lim = max_sq + shift + 1;
+        k_end = k_end < lim ? k_end : lim;
+    }
+    const int my_lim = p.causal ? sq + shift : p.Skv - 1;  // last key this lane's row may see
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4 acc[DT16];
+#pragma unroll
+    for (int dt = 0; dt < DT16; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const char *kbase = p.k + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh) * 2;
+    const char *vbase = p.v + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh) * 2;
+
+    for (int k0 = k_begin; k0 < k_end; k0 += AT_KEYS) {
+        // ---- stage K [key][D] and V^T [d][key]; keys past the end are zero (and masked below)
+        constexpr int CH = D / 8;  // 16-byte chunks per key
+        for (int e = tid; e < AT_KEYS * CH; e += 256) {
+            const int key = e / CH, c = e % CH;
+            const bool ok = k0 + key < k_end;
+            uint4 kv4 = make_uint4(0, 0, 0, 0), vv4 = make_uint4(0, 0, 0, 0);
+            if (ok) {
+                kv4 = *reinterpret_cast<const uint4 *>(kbase + (static_cast<int64_t>(k0 + key) * p.k_ss + c * 8) * 2);
+                vv4 = *reinterpret_cast<const uint4 *>(vbase + (static_cast<int64_t>(k0 + key) * p.v_ss + c * 8) * 2);
+            }
+            *reinterpret_cast<uint4 *>(ks + key * KP + c * 16) = kv4;
+            const uint32_t w[4] = {vv4.x, vv4.y, vv4.z, vv4.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * j) * VP + key * 2) = static_cast<uint16_t>(w[j] & 0xffffu);
+                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * j + 1) * VP + key * 2) = static_cast<uint16_t>(w[j] >> 16);
+            }
+        }
+        __syncthreads();
+
+        // ---- S^T = K Q^T: s[t][i] = score of key k0 + 16 t + 4 lq + i against this lane's query row
+        f32x4 s[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < DK; ++kk) {
+                const uint4 kf = *reinterpret_cast<const uint4 *>(ks + (16 * t + l16) * KP + (32 * kk + 8 * lq) * 2);
+                s[t] = mfma16<DT>(kf, qf[kk], s[t]);
+            }
+        }
+        // ---- online softmax for this lane's row (the 4 lanes l16 + 16 * {0..3} hold the same row)
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = k0 + 16 * t + 4 * lq + i;
+                const float x = (key <= my_lim && key < k_end) ? s[t][i] * p.scale_log2 : -INFINITY;
+                s[t][i] = x;
+                mx = fmaxf(mx, x);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with nothing visible yet: all p = 0
+        const float alpha = exp2f(m_run - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float pv = exp2f(s[t][i] - m_use);
+                s[t][i] = pv;
+                sum += pv;
+            }
+        sum += __shfl_xor(sum, 16);
+        sum += __shfl_xor(sum, 32);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+
+        // ---- O^T += V^T P^T. MFMA K slot (lq, e): e < 4 -> key 32 u + 4 lq + e, e >= 4 -> key 32 u + 16 + 4 lq + e - 4
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            uint4 pf;
+            pf.x = pack2_half<DT>(s[2 * u][0], s[2 * u][1]);
+            pf.y = pack2_half<DT>(s[2 * u][2], s[2 * u][3]);
+            pf.z = pack2_half<DT>(s[2 * u + 1][0], s[2 * u + 1][1]);
+            pf.w = pack2_half<DT>(s[2 * u + 1][2], s[2 * u + 1][3]);
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt) {
+                const char *vrow = vt + (16 * dt + l16) * VP + (32 * u + 4 * lq) * 2;
+                const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
+                const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 32);
+                acc[dt] = mfma16<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, acc[dt]);
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- acc[dt][i] = O[row = l16][d = 16 dt + 4 lq + i]
+    if (!row_ok) return;
+    if (p.nsplit == 1) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        char *orow = p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(sq) * p.o_ss + static_cast<int64_t>(head) * p.o_sh) * 2;
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt) {
+            uint2 o2;
+            o2.x = pack2_half<DT>(acc[dt][0] * inv, acc[dt][1] * inv);
+            o2.y = pack2_half<DT>(acc[dt][2] * inv, acc[dt][3] * inv);
+            *reinterpret_cast<uint2 *>(orow + (16 * dt + 4 * lq) * 2) = o2;
+        }
+    } else {
+        float *pr = p.part + ((static_cast<int64_t>(blockIdx.z) * gridDim.y + bh) * p.rows_pad + row) * (D + 4);
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt)
+            *reinterpret_cast<f32x4 *>(pr + 16 * dt + 4 * lq) = acc[dt];
+        if (lq == 0) {
+            pr[D] = m_run;
+            pr[D + 1] = l_run;
+        }
+    }
+}
+
+// out[row] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the key splits. One thread per (row, 4 head-dim elements).
+template <int DT, int D>
+__global__ __launch_bounds__(256) void attention_combine_kernel(AttnParams p) {
+    const int nrows = p.G * p.Sq;
+    const int per_row = D / 4;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int bh = blockIdx.y;
+    if (e >= static_cast<int64_t>(nrows) * per_row) return;
+    const int row = static_cast<int>(e / per_row), d4 = static_cast<int>(e % per_row) * 4;
+    float M = -INFINITY;
+    for (int s = 0; s < p.nsplit; ++s) {
+        const float *pr = p.part + ((static_cast<int64_t>(s) * gridDim.y + bh) * p.rows_pad + row) * (D + 4);
+        M = fmaxf(M, pr[D]);
+    }
+    const float m_use = M == -INFINITY ? 0.f : M;
+    float o[4] = {0.f, 0.f, 0.f, 0.f}, l = 0.f;
+    for (int s = 0; s < p.nsplit; ++s) {
+        const float *pr = p.part + ((static_cast<int64_t>(s) * gridDim.y + bh) * p.rows_pad + row) * (D + 4);
+        const float w = exp2f(pr[D] - m_use);
+        l += w * pr[D + 1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] += w * pr[d4 + i];
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const int b = bh / p.Hkv, hkv = bh % p.Hkv, g = row / p.Sq, sq = row % p.Sq;
+    const int head = hkv * p.G + g;
+    uint2 o2;
+    o2.x = pack2_half<DT>(o[0] * inv, o[1] * inv);
+    o2.y = pack2_half<DT>(o[2] * inv, o[3] * inv);
+    *reinterpret_cast<uint2 *>(p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(sq) * p.o_ss + static_cast<int64_t>(head) * p.o_sh + d4) * 2) = o2;
+}
+
+template <int DT, int D>
+int launch(AttnParams p, int cus, hipStream_t s) {
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    const int nrows = p.G * p.Sq;
+    const int row_tiles = (nrows + AT_ROWS - 1) / AT_ROWS;
+    const int64_t blocks = static_cast<int64_t>(row_tiles) * p.B * p.Hkv;
+    // split the keys when the rows alone leave CUs idle and there are enough keys to share out
+    int nsplit = 1;
+    if (blocks < cus) {
+        nsplit = static_cast<int>((2 * cus + blocks - 1) / blocks);
+        const int max_by_keys = (p.Skv + 255) / 256;  // at least 256 keys per split
+        if (nsplit > max_by_keys) nsplit = max_by_keys;
+        if (nsplit > 64) nsplit = 64;
+        if (nsplit < 1) nsplit = 1;
+    }
+    p.keys_per_split = ((p.Skv + nsplit - 1) / nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
+    nsplit = (p.Skv + p.keys_per_split - 1) / p.keys_per_split;
+    p.nsplit = nsplit;
+    p.rows_pad = row_tiles * AT_ROWS;
+    TPAMD_REQUIRE(p.B * p.Hkv < 65536 && nsplit < 65536, "attention: batch * kv heads too large for one launch");
+    const dim3 grid(row_tiles, p.B * p.Hkv, nsplit);
+    if (nsplit == 1) {
+        hipLaunchKernelGGL((attention_kernel<DT, D>), grid, dim3(256), 0, s, p);
+        TPAMD_HIP(hipGetLastError());
+        return TPAMD_OK;
+    }
+    const size_t need = static_cast<size_t>(nsplit) * p.B * p.Hkv * p.rows_pad * (D + 4) * sizeof(float);
+    std::lock_guard<std::mutex> hold(splitk_mutex());
+    void *ws = nullptr;
+    int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
+    if (rc != TPAMD_OK) return rc;
+    if (ws == nullptr) {  // no scratch (first use under stream capture, or more than it holds): one split
+        p.nsplit = 1;
+        p.keys_per_split = (p.Skv + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
+        hipLaunchKernelGGL((attention_kernel<DT, D>), dim3(row_tiles, p.B * p.Hkv, 1), dim3(256), 0, s, p);
+        TPAMD_HIP(hipGetLastError());
+        return TPAMD_OK;
+    }
+    p.part = static_cast<float *>(ws);
+    hipLaunchKernelGGL((attention_kernel<DT, D>), grid, dim3(256), 0, s, p);
+    TPAMD_HIP(hipGetLastError());
+    const unsigned cblocks = static_cast<unsigned>((static_cast<int64_t>(nrows) * (D / 4) + 255) / 256);
+    hipLaunchKernelGGL((attention_combine_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+}  // namespace
+
+int attention_dispatch(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq,
+                       int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal, int dtype, hipStream_t s) {
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    AttnParams p{};
+    p.q = static_cast<const char *>(q);
+    p.k = static_cast<const char *>(k);
+    p.v = static_cast<const char *>(v);
+    p.o = static_cast<char *>(o);
+    p.B = static_cast<int>(B); p.Hq = static_cast<int>(Hq); p.Hkv = static_cast<int>(Hkv);
+    p.Sq = static_cast<int>(Sq); p.Skv = static_cast<int>(Skv); p.G = static_cast<int>(Hq / Hkv);
+    p.q_sb = strides[0]; p.q_sh = strides[1]; p.q_ss = strides[2];
+    p.k_sb = strides[3]; p.k_sh = strides[4]; p.k_ss = strides[5];
+    p.v_sb = strides[6]; p.v_sh = strides[7]; p.v_ss = strides[8];
+    p.o_sb = strides[9]; p.o_ss = strides[10]; p.o_sh = strides[11];
+    p.scale_log2 = scale * 1.4426950408889634f;
+    p.causal = causal;
+    const bool bf = dtype == TPAMD_BF16;
+    if (D == 64) return bf ? launch<TPAMD_BF16, 64>(p, cus, s) : launch<TPAMD_F16, 64>(p, cus, s);
+    return bf ? launch<TPAMD_BF16, 128>(p, cus, s) : launch<TPAMD_F16, 128>(p, cus, s);
+}
+
+}  // namespace tpamd

@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <stdarg.h>
 
+#include <mutex>
+
 #include "../../include/tpamd.h"
 
 namespace tpamd {
@@ -30,6 +32,12 @@ void set_error(const char *fmt, ...);
             return TPAMD_ERR_HIP;                                                                \
         }                                                                                        \
     } while (0)
+
+// The per-device fp32 scratch buffer (split-K partial tiles, split-KV attention partials): defined in gemm.hip.
+// Callers hold splitk_mutex() from the lookup until their launches that use the buffer are enqueued and pass
+// reserve = 4 * CUs * 64 KiB, so that whoever comes first allocates the size everybody can live with.
+std::mutex &splitk_mutex();
+int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out);
 
 static inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 

@@ -916,11 +916,11 @@ int launch_direct(GemmParams p, hipStream_t s) {
 // such GEMMs over several streams of one device have to order those streams themselves); the mutex keeps the two
 // launches of a call together when several host threads enqueue onto one stream. *out stays NULL when there is no
 // buffer yet and the stream is being captured (allocating is not allowed then): the caller runs unsplit.
-inline std::mutex &splitk_mutex() {
+std::mutex &splitk_mutex() {
     static std::mutex m;
     return m;
 }
-inline int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
+int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
     struct Entry { int dev; void *ptr; size_t bytes; };
     static std::vector<Entry> cache;  // guarded by splitk_mutex(), held by the caller
     *out = nullptr;

@@ -1,0 +1,97 @@
+"""Rank-local attention core on the GPU against the oracle (float64 on the CPU): rtol 2e-2 on 16-bit inputs,
+plus an absolute floor of 2e-2 of the value scale (outputs are convex combinations of v rows)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as oat
+from tensor_parallel_amd import _native
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+RTOL = 2e-2
+
+
+def make(B, Hq, Hkv, Sq, Skv, D, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Hq, Sq, D, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, Skv, D, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, Skv, D, generator=g).to(dtype)
+    return q, k, v
+
+
+def check(q, k, v, causal, scale=None):
+    D = q.shape[-1]
+    scale = D ** -0.5 if scale is None else scale
+    got = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), scale=scale, causal=causal)
+    assert got.shape == (q.shape[0], q.shape[2], q.shape[1], D) and got.dtype == q.dtype
+    want = oat.attention_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale, causal)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL)
+    return got
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D", [
+    (2, 4, 4, 64, 64, 64),      # one tile of rows per head, equal heads
+    (1, 16, 2, 1, 300, 64),     # decode: a group of 8 heads in one MFMA tile, ragged key count
+    (2, 8, 2, 3, 200, 64),      # a few new positions on a cache
+    (1, 2, 1, 70, 70, 64),      # row tiles that straddle heads, ragged
+    (1, 4, 2, 130, 130, 128),   # head_dim 128
+    (3, 6, 3, 1, 17, 128),      # fewer keys than a tile
+])
+def test_attention_matches_oracle(dtype, causal, B, Hq, Hkv, Sq, Skv, D):
+    check(*make(B, Hq, Hkv, Sq, Skv, D, dtype), causal)
+
+
+def test_strided_inputs_as_projection_outputs_produce_them():
+    """q / k / v as views of [B, S, H, D] projection outputs (what the attention modules pass), sliced cache."""
+    B, Hq, Hkv, S, D = 2, 8, 2, 96, 64
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn(B, S, (Hq + 2 * Hkv) * D, generator=g).to(torch.bfloat16).to(DEV)
+    q = qkv[..., : Hq * D].view(B, S, Hq, D).transpose(1, 2)
+    k = qkv[..., Hq * D: (Hq + Hkv) * D].view(B, S, Hkv, D).transpose(1, 2)
+    v = qkv[..., (Hq + Hkv) * D:].view(B, S, Hkv, D).transpose(1, 2)
+    assert not q.is_contiguous()
+    got = _native.attention(q, k, v, causal=True)
+    want = oat.attention_f64(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), D ** -0.5, True)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL)
+    assert torch.equal(got, _native.attention(q.contiguous(), k.contiguous(), v.contiguous(), causal=True))
+
+
+def test_falcon_40b_rank_shard_decode_and_prefill():
+    """BASELINE config 4 at W = 2: 64 query heads and 4 key/value heads per rank, head_dim 64; decode batch 8 on 2048
+    cached keys (split over the keys), prefill of 1024 positions (sampled rows against the oracle)."""
+    q, k, v = make(8, 64, 4, 1, 2048, 64, torch.bfloat16, seed=1)
+    check(q, k, v, True)
+    q, k, v = make(1, 64, 4, 1024, 1024, 64, torch.bfloat16, seed=2)
+    got = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=True)
+    assert torch.isfinite(got.float()).all()
+    heads = [0, 17, 63]
+    want = oat.attention_f64(q[:, heads].float().numpy(), k[:, [0, 1, 3]].float().numpy(), v[:, [0, 1, 3]].float().numpy(), 64 ** -0.5, True)
+    torch.testing.assert_close(got[:, :, heads].double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL)
+
+
+def test_split_and_unsplit_key_ranges_agree():
+    """The same decode rows with many keys (split over blocks, merged by the second kernel) and as part of a batch
+    large enough not to be split."""
+    q, k, v = make(1, 16, 1, 1, 4096, 64, torch.float16, seed=4)
+    one = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=False)
+    B = 300
+    many = _native.attention(q.expand(B, -1, -1, -1).contiguous().to(DEV), k.expand(B, -1, -1, -1).contiguous().to(DEV),
+                             v.expand(B, -1, -1, -1).contiguous().to(DEV), causal=False)
+    torch.testing.assert_close(many[7].float(), one[0].float(), rtol=2e-3, atol=2e-3)
+
+
+def test_argument_errors():
+    q, k, v = make(1, 4, 3, 2, 2, 64, torch.float16)
+    with pytest.raises(ValueError):
+        _native.attention(q.to(DEV), k.to(DEV), v.to(DEV))  # 4 query heads over 3 key/value heads
+    q, k, v = make(1, 2, 2, 5, 3, 64, torch.float16)
+    with pytest.raises(ValueError):
+        _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=True)  # more queries than keys
+    q, k, v = make(1, 2, 2, 4, 4, 32, torch.float16)
+    with pytest.raises(RuntimeError):
+        _native.attention(q.to(DEV), k.to(DEV), v.to(DEV))  # head_dim 32: no kernel
+    with pytest.raises(TypeError):
+        _native.attention(q.float().to(DEV), k.float().to(DEV), v.float().to(DEV))
