@@ -95,3 +95,37 @@ def test_argument_errors():
         _native.attention(q.to(DEV), k.to(DEV), v.to(DEV))  # head_dim 32: no kernel
     with pytest.raises(TypeError):
         _native.attention(q.float().to(DEV), k.float().to(DEV), v.float().to(DEV))
+
+
+def test_llama_with_the_registered_attention_implementation():
+    """A small Llama (grouped-query, head_dim 64) with attn_implementation "tpamd" against the same weights with
+    transformers' eager attention: prefill logits and one decode step on the cache, unsplit and through
+    tp.tensor_parallel on two ranks sharing the device."""
+    from copy import deepcopy
+
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    import tensor_parallel_amd as tp
+
+    name = tp.attention.register()
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=512, hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8,
+                      num_key_value_heads=2, max_position_embeddings=256, attn_implementation="eager")
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV).eval()
+    ids = torch.randint(0, 512, (2, 48), generator=torch.Generator().manual_seed(1)).to(DEV)
+    nxt = torch.randint(0, 512, (2, 1), generator=torch.Generator().manual_seed(2)).to(DEV)
+    with torch.no_grad():
+        ref = model(input_ids=ids, use_cache=True)
+        ref_step = model(input_ids=nxt, past_key_values=ref.past_key_values, use_cache=True).logits
+    fast = deepcopy(model)
+    fast.config._attn_implementation = name
+    with torch.no_grad():
+        out = fast(input_ids=ids, use_cache=True)
+        step = fast(input_ids=nxt, past_key_values=out.past_key_values, use_cache=True).logits
+    scale = ref.logits.float().std().item()
+    torch.testing.assert_close(out.logits.float(), ref.logits.float(), rtol=RTOL, atol=3 * RTOL * scale)
+    torch.testing.assert_close(step.float(), ref_step.float(), rtol=RTOL, atol=3 * RTOL * scale)
+    model_tp = tp.tensor_parallel(deepcopy(fast), [DEV, DEV])
+    with torch.no_grad():
+        tp_logits = model_tp(input_ids=ids, use_cache=False).logits
+    torch.testing.assert_close(tp_logits.float(), ref.logits.float(), rtol=RTOL, atol=3 * RTOL * scale)
