@@ -17,6 +17,8 @@
 // the per-device scratch buffer and attention_combine_kernel merges them.
 #include "common.h"
 
+#include <stdlib.h>
+
 namespace tpamd {
 namespace {
 
@@ -43,14 +45,19 @@ struct AttnParams {
     int nsplit, keys_per_split, rows_pad;
 };
 
-constexpr int AT_ROWS = 64;   // query rows per block
 constexpr int AT_KEYS = 64;   // keys per tile
 
-template <int DT, int D>
-__global__ __launch_bounds__(256) void attention_kernel(AttnParams p) {
+// RT = 16-row tiles per wavefront: 1 for few rows (decode), 2 for prefill, where every K and V^T fragment read
+// from LDS then feeds two MFMAs (with one tile the fragment reads alone would need the whole LDS bandwidth).
+// A block owns 64 * RT consecutive rows.
+// At least two wavefronts per SIMD are asked for: that caps a wavefront at 256 registers, and with no need for
+// AGPRs the compiler keeps MFMA results in ordinary VGPRs, where the softmax can use them without copies.
+template <int DT, int D, int RT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) void attention_kernel(AttnParams p) {
     constexpr int KP = D * 2 + 16;        // K tile row pitch (bytes): conflict-free 16-byte reads
     constexpr int VP = AT_KEYS * 2 + 8;   // V^T tile row pitch (bytes), 8-byte aligned
     constexpr int DT16 = D / 16, DK = D / 32;
+    constexpr int ROWS = 64 * RT;
     __shared__ __align__(16) char ks[AT_KEYS * KP];
     __shared__ __align__(16) char vt[D * VP];
 
@@ -58,146 +65,207 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams p) {
     const int l16 = lane & 15, lq = lane >> 4;
     const int bh = blockIdx.y, b = bh / p.Hkv, hkv = bh % p.Hkv;
     const int nrows = p.G * p.Sq;
-    const int row0 = blockIdx.x * AT_ROWS;
-    const int row = row0 + wave * 16 + l16;
-    const bool row_ok = row < nrows;
-    const int g = row_ok ? row / p.Sq : 0, sq = row_ok ? row % p.Sq : 0;
-    const int head = hkv * p.G + g;
+    // causal: blocks with the highest positions have the longest key ranges; they are launched first
+    const int row_tile = p.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+    const int row0 = row_tile * ROWS;
+    const int shift = p.Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
 
-    // ---- Q fragments (second MFMA operand): lane = (query row l16, 8 head-dim elements at 32*kk + 8*lq)
-    uint4 qf[DK];
-    {
-        const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(head) * p.q_sh + static_cast<int64_t>(sq) * p.q_ss) * 2;
+    // ---- this lane's query rows and their Q fragments (second MFMA operand): 8 head-dim elements at 32*kk + 8*lq
+    int row[RT], sq[RT], head[RT], my_lim[RT];
+    bool row_ok[RT];
+    uint4 qf[RT][DK];
 #pragma unroll
-        for (int kk = 0; kk < DK; ++kk) qf[kk] = row_ok ? *reinterpret_cast<const uint4 *>(qrow + (32 * kk + 8 * lq) * 2) : make_uint4(0, 0, 0, 0);
+    for (int r = 0; r < RT; ++r) {
+        row[r] = row0 + (wave * RT + r) * 16 + l16;
+        row_ok[r] = row[r] < nrows;
+        const int g = row_ok[r] ? row[r] / p.Sq : 0;
+        sq[r] = row_ok[r] ? row[r] % p.Sq : 0;
+        head[r] = hkv * p.G + g;
+        my_lim[r] = p.causal ? sq[r] + shift : p.Skv - 1;  // last key this row may see
+        const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(head[r]) * p.q_sh + static_cast<int64_t>(sq[r]) * p.q_ss) * 2;
+#pragma unroll
+        for (int kk = 0; kk < DK; ++kk)
+            qf[r][kk] = row_ok[r] ? *reinterpret_cast<const uint4 *>(qrow + (32 * kk + 8 * lq) * 2) : make_uint4(0, 0, 0, 0);
     }
 
     // ---- key range of this block
     int k_begin = blockIdx.z * p.keys_per_split;
     int k_end = k_begin + p.keys_per_split < p.Skv ? k_begin + p.keys_per_split : p.Skv;
-    const int shift = p.Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
     if (p.causal) {
-        // the largest position in this tile of rows (a tile that straddles two heads contains position Sq - 1)
-        const int last_row = row0 + AT_ROWS - 1 < nrows - 1 ? row0 + AT_ROWS - 1 : nrows - 1;
+        // the largest position among this block's rows (a block that straddles two heads contains position Sq - 1)
+        const int last_row = row0 + ROWS - 1 < nrows - 1 ? row0 + ROWS - 1 : nrows - 1;
         const int max_sq = (row0 / p.Sq != last_row / p.Sq) ? p.Sq - 1 : last_row % p.Sq;
         const int lim = max_sq + shift + 1;
         k_end = k_end < lim ? k_end : lim;
     }
-    const int my_lim = p.causal ? sq + shift : p.Skv - 1;  // last key this lane's row may see
 
-    float m_run = -INFINITY, l_run = 0.f;
-    f32x4 acc[DT16];
+    float m_run[RT];
+    f32x4 acc[RT][DT16], l_acc[RT];  // l_acc[r][i]: the row sum of this lane's row r, the same in all four elements
+    const uint32_t one2 = DT == TPAMD_BF16 ? 0x3f803f80u : 0x3c003c00u;  // two 1.0 in the tensor dtype
+    const uint4 ones = make_uint4(one2, one2, one2, one2);
 #pragma unroll
-    for (int dt = 0; dt < DT16; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < RT; ++r) {
+        m_run[r] = -INFINITY;
+        l_acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt) acc[r][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
     const char *kbase = p.k + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh) * 2;
     const char *vbase = p.v + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh) * 2;
 
-    for (int k0 = k_begin; k0 < k_end; k0 += AT_KEYS) {
-        // ---- stage K [key][D] and V^T [d][key]; keys past the end are zero (and masked below)
-        constexpr int CH = D / 8;  // 16-byte chunks per key
-        for (int e = tid; e < AT_KEYS * CH; e += 256) {
-            const int key = e / CH, c = e % CH;
-            const bool ok = k0 + key < k_end;
-            uint4 kv4 = make_uint4(0, 0, 0, 0), vv4 = make_uint4(0, 0, 0, 0);
-            if (ok) {
-                kv4 = *reinterpret_cast<const uint4 *>(kbase + (static_cast<int64_t>(k0 + key) * p.k_ss + c * 8) * 2);
-                vv4 = *reinterpret_cast<const uint4 *>(vbase + (static_cast<int64_t>(k0 + key) * p.v_ss + c * 8) * 2);
-            }
-            *reinterpret_cast<uint4 *>(ks + key * KP + c * 16) = kv4;
-            const uint32_t w[4] = {vv4.x, vv4.y, vv4.z, vv4.w};
+    // K / V tiles travel global -> registers -> LDS; the registers of tile i+1 are requested before tile i is
+    // multiplied, so the loads fly during the MFMAs and the softmax. Keys past the end are zero (and masked below).
+    constexpr int CH = D / 8;                    // 16-byte chunks per key
+    constexpr int LPT = AT_KEYS * CH / 256;      // chunks per thread per tile (2 for head_dim 64, 4 for 128)
+    uint4 kreg[LPT], vreg[LPT];
+    const int key_j0 = tid / CH, chunk = tid % CH;  // thread's key inside a tile for j = 0; j adds 256 / CH keys
+    const char *kthr = kbase + chunk * 16, *vthr = vbase + chunk * 16;
+    const int64_t k_pitch = p.k_ss * 2, v_pitch = p.v_ss * 2;
+    auto fetch = [&](int k0) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * j) * VP + key * 2) = static_cast<uint16_t>(w[j] & 0xffffu);
-                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * j + 1) * VP + key * 2) = static_cast<uint16_t>(w[j] >> 16);
+        for (int j = 0; j < LPT; ++j) {
+            const int key = k0 + key_j0 + j * (256 / CH);
+            const bool ok = key < k_end;
+            // unconditional loads (first key of the range when out of it) keep all of them in flight together
+            const int64_t kr = ok ? key : k_begin;
+            const uint4 kv4 = *reinterpret_cast<const uint4 *>(kthr + kr * k_pitch);
+            const uint4 vv4 = *reinterpret_cast<const uint4 *>(vthr + kr * v_pitch);
+            kreg[j] = ok ? kv4 : make_uint4(0, 0, 0, 0);
+            vreg[j] = ok ? vv4 : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int j = 0; j < LPT; ++j) {
+            const int e = tid + j * 256, key = e / CH, c = e % CH;
+            *reinterpret_cast<uint4 *>(ks + key * KP + c * 16) = kreg[j];
+            const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * i) * VP + key * 2) = static_cast<uint16_t>(w[i] & 0xffffu);
+                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * i + 1) * VP + key * 2) = static_cast<uint16_t>(w[i] >> 16);
             }
         }
+    };
+    if (k_begin < k_end) fetch(k_begin);
+    for (int k0 = k_begin; k0 < k_end; k0 += AT_KEYS) {
+        stage();
         __syncthreads();
+        if (k0 + AT_KEYS < k_end) fetch(k0 + AT_KEYS);
 
-        // ---- S^T = K Q^T: s[t][i] = score of key k0 + 16 t + 4 lq + i against this lane's query row
-        f32x4 s[4];
+        // ---- S^T = K Q^T: s[r][t][i] = score of key k0 + 16 t + 4 lq + i against query row r of this lane
+        f32x4 s[RT][4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int r = 0; r < RT; ++r) s[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < DK; ++kk) {
                 const uint4 kf = *reinterpret_cast<const uint4 *>(ks + (16 * t + l16) * KP + (32 * kk + 8 * lq) * 2);
-                s[t] = mfma16<DT>(kf, qf[kk], s[t]);
+#pragma unroll
+                for (int r = 0; r < RT; ++r) s[r][t] = mfma16<DT>(kf, qf[r][kk], s[r][t]);
             }
         }
-        // ---- online softmax for this lane's row (the 4 lanes l16 + 16 * {0..3} hold the same row)
-        float mx = -INFINITY;
+        // ---- online softmax per row (the 4 lanes l16 + 16 * {0..3} hold the same row).
+        // Probabilities are taken relative to a reference maximum m_run (in units of scale * log2 e) that is only
+        // raised when the running maximum outgrows it by more than 2^LAZY: then the accumulators (which live in
+        // AGPRs: rescaling them costs three instructions per element) are rescaled; otherwise
+        // p = 2^(x - m_run) <= 2^LAZY, well inside what 16-bit p and fp32 sums hold. A tile fully visible to every
+        // row of the wavefront skips the masking. The row sums come out of the MFMA pipe (a row of ones appended
+        // to V^T) instead of 16 additions per row and tile.
+        constexpr float LAZY = 6.0f;
+        uint4 pf[RT][2];
+        bool tile_free = k0 + AT_KEYS <= k_end;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int r = 0; r < RT; ++r) tile_free = tile_free && (k0 + AT_KEYS - 1 <= my_lim[r]);
+        const bool no_mask = __all(tile_free);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = k0 + 16 * t + 4 * lq + i;
-                const float x = (key <= my_lim && key < k_end) ? s[t][i] * p.scale_log2 : -INFINITY;
-                s[t][i] = x;
-                mx = fmaxf(mx, x);
+        for (int r = 0; r < RT; ++r) {
+            if (!no_mask) {
+                // keys of this tile visible to the row: the first `vis`; key (t, i) of this lane sits at 16 t + 4 lq + i
+                const int last = my_lim[r] < k_end - 1 ? my_lim[r] : k_end - 1;
+                const int vis = last - k0 + 1 - 4 * lq;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[r][t][i] = (16 * t + i < vis) ? s[r][t][i] : -INFINITY;
             }
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with nothing visible yet: all p = 0
-        const float alpha = exp2f(m_run - m_use);
-        float sum = 0.f;
+            float mx = fmaxf(fmaxf(s[r][0][0], s[r][0][1]), fmaxf(s[r][0][2], s[r][0][3]));
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 1; t < 4; ++t) mx = fmaxf(mx, fmaxf(fmaxf(s[r][t][0], s[r][t][1]), fmaxf(s[r][t][2], s[r][t][3])));
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            mx *= p.scale_log2;  // scale > 0: the maximum of the scaled scores
+            if (__any(mx > m_run[r] + LAZY)) {  // wavefront-uniform: some row's maximum outgrew its reference
+                const float m_new = mx > m_run[r] + LAZY ? mx : m_run[r];
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with nothing visible yet
+                const float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_use);
+                m_run[r] = m_new;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float pv = exp2f(s[t][i] - m_use);
-                s[t][i] = pv;
-                sum += pv;
+                for (int i = 0; i < 4; ++i) l_acc[r][i] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT16; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[r][dt][i] *= alpha;
             }
-        sum += __shfl_xor(sum, 16);
-        sum += __shfl_xor(sum, 32);
-        l_run = l_run * alpha + sum;
-        m_run = m_new;
+            const float neg_ref = m_run[r] == -INFINITY ? 0.f : -m_run[r];
 #pragma unroll
-        for (int dt = 0; dt < DT16; ++dt)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+                for (int i = 0; i < 4; ++i) s[r][t][i] = __builtin_amdgcn_exp2f(fmaf(s[r][t][i], p.scale_log2, neg_ref));
+            // the lane's probabilities as the second MFMA operand. K slot (lq, e): e < 4 -> key 32 u + 4 lq + e,
+            // e >= 4 -> key 32 u + 16 + 4 lq + e - 4
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                pf[r][u].x = pack2_half<DT>(s[r][2 * u][0], s[r][2 * u][1]);
+                pf[r][u].y = pack2_half<DT>(s[r][2 * u][2], s[r][2 * u][3]);
+                pf[r][u].z = pack2_half<DT>(s[r][2 * u + 1][0], s[r][2 * u + 1][1]);
+                pf[r][u].w = pack2_half<DT>(s[r][2 * u + 1][2], s[r][2 * u + 1][3]);
+            }
+        }
 
-        // ---- O^T += V^T P^T. MFMA K slot (lq, e): e < 4 -> key 32 u + 4 lq + e, e >= 4 -> key 32 u + 16 + 4 lq + e - 4
+        // ---- O^T += V^T P^T, and the row sums: ones . P^T (every row of that product is the same sum)
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            uint4 pf;
-            pf.x = pack2_half<DT>(s[2 * u][0], s[2 * u][1]);
-            pf.y = pack2_half<DT>(s[2 * u][2], s[2 * u][3]);
-            pf.z = pack2_half<DT>(s[2 * u + 1][0], s[2 * u + 1][1]);
-            pf.w = pack2_half<DT>(s[2 * u + 1][2], s[2 * u + 1][3]);
 #pragma unroll
             for (int dt = 0; dt < DT16; ++dt) {
                 const char *vrow = vt + (16 * dt + l16) * VP + (32 * u + 4 * lq) * 2;
                 const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
                 const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 32);
-                acc[dt] = mfma16<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, acc[dt]);
+                const uint4 vf = make_uint4(lo.x, lo.y, hi.x, hi.y);
+#pragma unroll
+                for (int r = 0; r < RT; ++r) acc[r][dt] = mfma16<DT>(vf, pf[r][u], acc[r][dt]);
             }
+#pragma unroll
+            for (int r = 0; r < RT; ++r) l_acc[r] = mfma16<DT>(ones, pf[r][u], l_acc[r]);
         }
         __syncthreads();
     }
 
-    // ---- acc[dt][i] = O[row = l16][d = 16 dt + 4 lq + i]
-    if (!row_ok) return;
-    if (p.nsplit == 1) {
-        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-        char *orow = p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(sq) * p.o_ss + static_cast<int64_t>(head) * p.o_sh) * 2;
+    // ---- acc[r][dt][i] = O[row r of this lane][d = 16 dt + 4 lq + i]
 #pragma unroll
-        for (int dt = 0; dt < DT16; ++dt) {
-            uint2 o2;
-            o2.x = pack2_half<DT>(acc[dt][0] * inv, acc[dt][1] * inv);
-            o2.y = pack2_half<DT>(acc[dt][2] * inv, acc[dt][3] * inv);
-            *reinterpret_cast<uint2 *>(orow + (16 * dt + 4 * lq) * 2) = o2;
-        }
-    } else {
-        float *pr = p.part + ((static_cast<int64_t>(blockIdx.z) * gridDim.y + bh) * p.rows_pad + row) * (D + 4);
+    for (int r = 0; r < RT; ++r) {
+        if (!row_ok[r]) continue;
+        if (p.nsplit == 1) {
+            const float l_row = l_acc[r][0];
+            const float inv = l_row > 0.f ? 1.0f / l_row : 0.f;
+            char *orow = p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(sq[r]) * p.o_ss + static_cast<int64_t>(head[r]) * p.o_sh) * 2;
 #pragma unroll
-        for (int dt = 0; dt < DT16; ++dt)
-            *reinterpret_cast<f32x4 *>(pr + 16 * dt + 4 * lq) = acc[dt];
-        if (lq == 0) {
-            pr[D] = m_run;
-            pr[D + 1] = l_run;
+            for (int dt = 0; dt < DT16; ++dt) {
+                uint2 o2;
+                o2.x = pack2_half<DT>(acc[r][dt][0] * inv, acc[r][dt][1] * inv);
+                o2.y = pack2_half<DT>(acc[r][dt][2] * inv, acc[r][dt][3] * inv);
+                *reinterpret_cast<uint2 *>(orow + (16 * dt + 4 * lq) * 2) = o2;
+            }
+        } else {
+            float *pr = p.part + ((static_cast<int64_t>(blockIdx.z) * gridDim.y + bh) * p.rows_pad + row[r]) * (D + 4);
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt) *reinterpret_cast<f32x4 *>(pr + 16 * dt + 4 * lq) = acc[r][dt];
+            if (lq == 0) {
+                pr[D] = m_run[r];
+                pr[D + 1] = l_acc[r][0];
+            }
         }
     }
 }
@@ -239,25 +307,31 @@ int launch(AttnParams p, int cus, hipStream_t s) {
     int dev = 0;
     TPAMD_HIP(hipGetDevice(&dev));
     const int nrows = p.G * p.Sq;
-    const int row_tiles = (nrows + AT_ROWS - 1) / AT_ROWS;
+    // 128 rows per block (two 16-row tiles per wavefront) once that still leaves every CU a few blocks
+    const bool wide = nrows >= 128 && static_cast<int64_t>((nrows + 127) / 128) * p.B * p.Hkv >= 2 * cus;
+    const int block_rows = wide ? 128 : 64;
+    const int row_tiles = (nrows + block_rows - 1) / block_rows;
     const int64_t blocks = static_cast<int64_t>(row_tiles) * p.B * p.Hkv;
     // split the keys when the rows alone leave CUs idle and there are enough keys to share out
     int nsplit = 1;
-    if (blocks < cus) {
-        nsplit = static_cast<int>((2 * cus + blocks - 1) / blocks);
-        const int max_by_keys = (p.Skv + 255) / 256;  // at least 256 keys per split
+    if (blocks < 2 * cus) {
+        // several blocks per CU hide each other's load latency: aim at 4 per CU, at least 128 keys per split
+        nsplit = static_cast<int>((4 * cus + blocks - 1) / blocks);
+        const int max_by_keys = (p.Skv + 127) / 128;
         if (nsplit > max_by_keys) nsplit = max_by_keys;
         if (nsplit > 64) nsplit = 64;
         if (nsplit < 1) nsplit = 1;
     }
+    if (const char *e = getenv("TPAMD_ATTN_SPLITS")) nsplit = atoi(e) > 0 ? atoi(e) : 1;
     p.keys_per_split = ((p.Skv + nsplit - 1) / nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
     nsplit = (p.Skv + p.keys_per_split - 1) / p.keys_per_split;
     p.nsplit = nsplit;
-    p.rows_pad = row_tiles * AT_ROWS;
+    p.rows_pad = row_tiles * block_rows;
     TPAMD_REQUIRE(p.B * p.Hkv < 65536 && nsplit < 65536, "attention: batch * kv heads too large for one launch");
     const dim3 grid(row_tiles, p.B * p.Hkv, nsplit);
     if (nsplit == 1) {
-        hipLaunchKernelGGL((attention_kernel<DT, D>), grid, dim3(256), 0, s, p);
+        if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2>), grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((attention_kernel<DT, D, 1>), grid, dim3(256), 0, s, p);
         TPAMD_HIP(hipGetLastError());
         return TPAMD_OK;
     }
@@ -269,12 +343,14 @@ int launch(AttnParams p, int cus, hipStream_t s) {
     if (ws == nullptr) {  // no scratch (first use under stream capture, or more than it holds): one split
         p.nsplit = 1;
         p.keys_per_split = (p.Skv + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
-        hipLaunchKernelGGL((attention_kernel<DT, D>), dim3(row_tiles, p.B * p.Hkv, 1), dim3(256), 0, s, p);
+        if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2>), dim3(row_tiles, p.B * p.Hkv, 1), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((attention_kernel<DT, D, 1>), dim3(row_tiles, p.B * p.Hkv, 1), dim3(256), 0, s, p);
         TPAMD_HIP(hipGetLastError());
         return TPAMD_OK;
     }
     p.part = static_cast<float *>(ws);
-    hipLaunchKernelGGL((attention_kernel<DT, D>), grid, dim3(256), 0, s, p);
+    if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2>), grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((attention_kernel<DT, D, 1>), grid, dim3(256), 0, s, p);
     TPAMD_HIP(hipGetLastError());
     const unsigned cblocks = static_cast<unsigned>((static_cast<int64_t>(nrows) * (D / 4) + 255) / 256);
     hipLaunchKernelGGL((attention_combine_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
