@@ -12,6 +12,8 @@ Modules and the reference code each one follows:
   reduce.py         the "sum" rule's arithmetic (src/tensor_parallel/cross_device_ops.py:49), bit-level
   shard_forward.py  rank-shard Linears, the SiLU-gated MLP shard and the W-thread forward
                     (src/tensor_parallel/wrapper.py:69-72, tensor_parallel.py:237-287), torch on CPU
+  attention.py      the attention core the wrapped module runs on a rank's heads (softmax(q k^T) v, grouped-query,
+                    causal aligned to the end of the keys), float64; the reference has no attention code of its own
   quant.py          int8 weight-only quantisation with outlier columns - NOT in the reference: parity
                     unpinned against it; defined in closed form and checked against fp64 matmul
 
@@ -23,5 +25,7 @@ How each function is pinned (tests/test_oracle_*.py):
   reduce       torch CPU bf16/fp16 addition (a third-party routine), W = 2 and chained W = 3..8
   forward      sum of row-parallel partials == unsplit Linear, concat of column-parallel == unsplit Linear,
                both in fp64
+  attention    torch's CPU scaled_dot_product_attention where it covers the case, explicit loops on tiny inputs for
+               grouped heads and Sq < Skv causal, rows of probabilities sum to one, a single visible key returns its value
   quant        dequantised weights within scale/2 of the originals; fp64 matmul of the definition
 """
