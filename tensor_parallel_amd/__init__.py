@@ -10,12 +10,14 @@ from . import _native, attention, state_actions
 from .config import Config
 from .dispatch import convert_state_dict, infer_sharded_device_map, save_tensor_parallel
 from .factory import tensor_parallel
+from .legacy import Sharded
 from .state_actions import Scale, Split, SplitInChunks, SplitInGroupedChunks, StateAction
 from .tensor_parallel import TensorParallel
 
 __all__ = [
     "Config",
     "Scale",
+    "Sharded",
     "Split",
     "SplitInChunks",
     "SplitInGroupedChunks",

@@ -17,6 +17,7 @@ from itertools import chain
 from typing import Any, Callable, Dict, Iterable, Mapping, Sequence, Union
 
 import torch
+from torch import nn
 
 from .collectives import DeviceAllGather, DeviceAllReduce
 from .state_actions import LegacyStateAction, StateAction
@@ -85,6 +86,41 @@ def create_collective_ops(rules: dict, devices: Sequence[torch.device], distribu
                 ops[rule] = DeviceAllGather(world_size, int(opts[0]) if opts else -1)
     return {pattern: {key: ops.get(rule, rule) if isinstance(rule, str) else rule for key, rule in actions.items()}
             for pattern, actions in rules.items()}
+
+
+def add_lora_rules(model: nn.Module, config: Config) -> Config:
+    """Extend `config`, in place, for the low-rank branches of peft LoRA Linears (config.py:128-154).
+
+    A LoRA Linear adds lora_B(lora_A(x)) to its base Linear. If the base weight is split on its output axis, lora_B's
+    weight takes the same split and lora_A stays whole. If it is split on its input axis, every rank sees only its
+    part of x: lora_A's input is gathered back to the full x and its output divided by the world size, so that the
+    sum over ranks that follows the base layer counts the low-rank branch once."""
+    from .state_actions import Split
+    from .utils import check_lora
+
+    state_rules, input_rules, output_rules = {}, {}, {}
+    for name, module in model.named_modules():
+        if not check_lora(module):
+            continue
+        for pattern, action in config.state_rules.items():
+            if pattern.search(name + ".weight") is None:
+                continue
+            if not isinstance(action, Split):
+                raise Exception(
+                    f"Can't apply action {action} since it uses LoRA. The only actions with LoRA support are Split and it's variations."
+                )
+            if action.dim == 0:
+                state_rules[re.compile(rf"^{re.escape(name)}\.lora_B")] = action
+            elif action.dim == 1:
+                branch = re.compile(rf"^{re.escape(name)}\.lora_A\..+")
+                input_rules[branch] = {0: "gather -1"}
+                output_rules[branch] = {0: "scale"}
+            else:
+                raise Exception(f"Expected dim in [0, 1]. Don't know what to do with LoRA linear split along dim {action.dim}")
+    config.state_rules.update(state_rules)
+    config.input_rules.update(input_rules)
+    config.output_rules.update(output_rules)
+    return config
 
 
 def get_parameter_name_mapping(names: Iterable[str], tensor_parallel_config: Config) -> Mapping[str, str]:

@@ -3,13 +3,14 @@
 
 Construction slices the whole state for all ranks with one launch of the region mover. A forward runs the
 W shards on W host threads, as the reference does (tensor_parallel.py:237-287); the threads meet in the
-"sum" / "gather" ops, which are single-device kernels here. The ZeRO-3 side-car of the reference
-(`sharded=True`) is not part of this package: the argument is accepted, and `apply_sharding` raises.
+"sum" / "gather" ops, which are single-device kernels here. `sharded=True` keeps the parameters the rule table
+leaves replicated as flat per-rank shards (`sharding.Sharded`) and recombines them on the device before a forward.
 """
 from __future__ import annotations
 
 import logging
 import threading
+from operator import attrgetter
 from typing import Any, Collection, Optional, Sequence, Union
 
 import torch
@@ -17,8 +18,9 @@ from torch import nn
 
 from .autoconfig import get_default_config
 from .collectives import set_turn_lock
-from .config import Config
+from .config import Config, add_lora_rules
 from .shard import make_shard
+from .sharding import Sharded
 from .slicing import BatchSlicer, concat_specs
 from .state_actions import SegmentedAction
 from .utils import nested_flatten, nested_pack
@@ -84,6 +86,7 @@ class TensorParallel(nn.Module):
         if tensor_parallel_config is None:
             tensor_parallel_config = get_default_config(module, self.devices)
             logger.info("Using automatic config: sharding individual linear/emb layers")
+        tensor_parallel_config = add_lora_rules(module, tensor_parallel_config)
         self.tensor_parallel_config = tensor_parallel_config
         config_with_ops = tensor_parallel_config.create_collective_ops(self.devices, distributed)
 
@@ -121,10 +124,14 @@ class TensorParallel(nn.Module):
         )
         self.preserve_shards_when_saving: bool = True
         if sharded:
-            logger.info("sharded=True (ZeRO-3 of the replicated parameters) is not available; parameters stay replicated")
+            self.apply_sharding(sharded_param_names)
 
     def apply_sharding(self, replicated_param_names: Optional[Collection[str]] = None):
-        raise NotImplementedError("ZeRO-3 sharding of replicated parameters is not part of tensor_parallel_amd")
+        if self.sharding_manager is not None:
+            raise Exception(
+                "Trying to apply sharding for the second time. If you wish NOT to apply sharding during model initialization, pass `sharded=False`."
+            )
+        self.sharding_manager = Sharded(self, len(self.devices), replicated_param_names)
 
     def prepare_args_kwargs_for_forward(self, *args, **kwargs):
         """One copy of (args, kwargs) per rank; every tensor is moved to that rank's device (tensor_parallel.py:121-137)."""
@@ -136,6 +143,8 @@ class TensorParallel(nn.Module):
         return zip(*per_rank)
 
     def forward(self, *args, **kwargs):
+        if self.sharding_manager is not None:
+            self.sharding_manager.synchronize_weights(self.all_cuda)
         if len(self.module_shards) <= 1:
             return [self.module_shards[0](*args, **kwargs)][self.output_device_index]
         if not all(p.device == d for p, d in zip(self._sanity_check_params, self.devices) if p.device.type != "meta"):
@@ -148,6 +157,8 @@ class TensorParallel(nn.Module):
 
     def set_preserve_shards_when_saving(self, value: bool):
         self.preserve_shards_when_saving = value
+        if self.sharding_manager is not None:
+            self.sharding_manager.preserve_shards_when_saving = value
 
     def state_dict(self, *args, **kwargs):
         """Sharded names by default; inside `save_tensor_parallel` the original model's names and full tensors,
@@ -162,8 +173,8 @@ class TensorParallel(nn.Module):
             state_dict[name.replace("tp_wrapped_module.", "")] = state_dict.pop(name)
         marker = "module_shards."
         first = next((n for n in state_dict if marker in n), None)
-        if first is None:
-            return state_dict
+        if first is None:  # nothing is tensor parallel
+            return self.process_sharded_state_dict(state_dict, kwargs.get("prefix", ""))
         shards_prefix = first[: first.find(marker) + len(marker)]
         module_prefix = shards_prefix[: -len(marker)]
         rank0 = shards_prefix + "0."
@@ -176,7 +187,17 @@ class TensorParallel(nn.Module):
                     break
             else:
                 state_dict[module_prefix + unsharded] = pieces[0]
-        return state_dict
+        return self.process_sharded_state_dict(state_dict, kwargs.get("prefix", ""))
+
+    def process_sharded_state_dict(self, destination, prefix):
+        """The ZeRO-3 parameters, recombined, under their names in the original model (tensor_parallel.py:223-234)."""
+        manager = self.sharding_manager
+        if manager is not None and hasattr(manager, "flat_shards"):
+            manager.synchronize_weights(self.all_cuda)
+            for name in manager.sharded_param_names:
+                value = attrgetter(name)(self.module_shards[0])
+                destination[prefix + name.replace("tp_wrapped_module.", "")] = value
+        return destination
 
 
 def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devices: Sequence[torch.device]):

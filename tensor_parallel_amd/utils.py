@@ -63,3 +63,27 @@ def find_tied_weight_aliases(module: nn.Module, destination: Optional[Dict[int, 
         if child is not None:
             find_tied_weight_aliases(child, destination, prefix + name + ".")
     return destination
+
+
+def verify_peft_version() -> None:
+    """LoRA layers are only understood in the layout of peft >= 0.3.0 (imports.py:4-7)."""
+    import sys
+
+    try:
+        from importlib.metadata import version
+
+        found = version("peft")
+    except Exception:
+        found = getattr(sys.modules.get("peft"), "__version__", None)
+    if found is None:
+        raise ImportError("tensor_parallel only works with peft>=0.3.0")
+    if tuple(int(x) for x in found.split(".")[:2] if x.isdigit()) < (0, 3):
+        raise ImportError("tensor_parallel only works with peft>=0.3.0")
+
+
+def check_lora(module: nn.Module) -> bool:
+    """True for peft's LoRA-augmented Linear: a class named `Linear` defined in `peft.tuners.lora` (utils.py:131-144)."""
+    if type(module).__module__ != "peft.tuners.lora":
+        return False
+    verify_peft_version()
+    return type(module).__name__ == "Linear"
