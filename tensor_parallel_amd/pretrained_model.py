@@ -1,17 +1,17 @@
-"""Thin Hugging Face wrapper: picks the model family's rule table and delegates forward
-(reference: src/tensor_parallel/pretrained_model.py:21-76). Generation helpers, cache reordering and the
-encoder wrapper of the reference are not carried."""
+"""Hugging Face wrapper: picks the model family's rule table, delegates forward, and lets `generate` drive the
+rank shards (reference: src/tensor_parallel/pretrained_model.py:21-165). The attention cache is rank-local
+(see kv_cache): there is no cache reordering hook here, the cache objects reorder themselves."""
 from __future__ import annotations
 
 import logging
 from typing import Optional, Sequence
 
 import torch
-from transformers import PretrainedConfig, PreTrainedModel
+from transformers import GenerationMixin, PretrainedConfig, PreTrainedModel
 
 from .config import Config
 from .slicing_configs import PREDEFINED_CONFIGS
-from .tensor_parallel import TensorParallel, check_device_ids
+from .tensor_parallel import TensorParallel, check_device_ids, parallel_apply_simple
 
 logger = logging.getLogger(__file__)
 
@@ -25,7 +25,25 @@ def find_predefined_tensor_parallel_config(model_config: PretrainedConfig, devic
     return getter(model_config, device_ids)
 
 
-class TensorParallelPreTrainedModel(PreTrainedModel):
+class _EncoderWrapper(torch.nn.Module):
+    """The encoders of all rank shards, run side by side like the whole model (pretrained_model.py:108-165)."""
+
+    def __init__(self, tp_model: "TensorParallelPreTrainedModel"):
+        super().__init__()
+        self.__dict__["tp_model"] = tp_model  # not a submodule: the model owns the shards
+        shards = tp_model.wrapped_model.module_shards
+        self.__dict__["encoder_shards"] = [shard.get_encoder() for shard in shards]
+        self.main_input_name = getattr(self.encoder_shards[0], "main_input_name", "input_ids")
+
+    def forward(self, *args, **kwargs):
+        wrapped = self.tp_model.wrapped_model
+        if wrapped.sharding_manager is not None:
+            wrapped.sharding_manager.synchronize_weights(wrapped.all_cuda)
+        inputs, kwargs_tup = wrapped.prepare_args_kwargs_for_forward(*args, **kwargs)
+        return parallel_apply_simple(self.encoder_shards, inputs, kwargs_tup, wrapped.devices)[wrapped.output_device_index]
+
+
+class TensorParallelPreTrainedModel(PreTrainedModel, GenerationMixin):
     is_parallelizable = model_parallel = True
     # the wrapper only delegates to the wrapped model, whatever attention implementation that one runs
     _supports_sdpa = _supports_flash_attn = _supports_flex_attn = _supports_attention_backend = True
@@ -42,7 +60,16 @@ class TensorParallelPreTrainedModel(PreTrainedModel):
         super().__init__(module.config)
         if tensor_parallel_config is None:
             tensor_parallel_config = find_predefined_tensor_parallel_config(module.config, device_ids)
+        if hasattr(module, "_hf_hook"):
+            from accelerate.hooks import remove_hook_from_module
+
+            remove_hook_from_module(module, recurse=True)
+        self.main_input_name = module.main_input_name
+        generation_config = getattr(module, "generation_config", None)
         self.wrapped_model = TensorParallel(module, device_ids, output_device, output_device_index, tensor_parallel_config, **kwargs)
+        if generation_config is not None:
+            self.generation_config = generation_config
+        self._encoder_wrapper: Optional[_EncoderWrapper] = None
 
     @property
     def devices(self):
@@ -60,6 +87,31 @@ class TensorParallelPreTrainedModel(PreTrainedModel):
 
     def forward(self, *args, **kwargs):
         return self.wrapped_model(*args, **kwargs)
+
+    # ---- what `generate` asks the model itself: answered by the first rank shard, which is the model class
+    def _validate_model_class(self):
+        return self.wrapped_model.module_shards[0]._validate_model_class()
+
+    def _validate_model_kwargs(self, model_kwargs):
+        return self.wrapped_model.module_shards[0]._validate_model_kwargs(model_kwargs)
+
+    def _prepare_model_inputs(self, *args, **kwargs):
+        return self.wrapped_model.module_shards[0]._prepare_model_inputs(*args, **kwargs)
+
+    def prepare_inputs_for_generation(self, *args, **kwargs):
+        return self.wrapped_model.module_shards[0].prepare_inputs_for_generation(*args, **kwargs)
+
+    def _supports_default_dynamic_cache(self) -> bool:
+        return self.wrapped_model.module_shards[0]._supports_default_dynamic_cache()
+
+    def get_encoder(self, *args, **kwargs):
+        shards = self.wrapped_model.module_shards
+        assert len(shards), "Can't get encoder since no module shards present"
+        if len(shards) == 1:
+            return shards[0].get_encoder(*args, **kwargs)
+        if self._encoder_wrapper is None:
+            self.__dict__["_encoder_wrapper"] = _EncoderWrapper(self)
+        return self._encoder_wrapper
 
     def state_dict(self, *args, **kwargs):
         state_dict = super().state_dict(*args, **kwargs)

@@ -2,8 +2,9 @@
 
 Carried here: BLOOM (slicing_configs.py:32-72), T5 (:75-137), BERT (:140-177), GPT-2 (:180-238), GPT-NeoX (:241-282),
 CodeGen (:285-342), Llama (:345-406) and Falcon / RefinedWeb (:409-462). The state rules - which tensor is split
-how - are those of the reference. The KV-cache rules of the reference (`select_kv_for_rank`, `gather_kv`) are not
-carried: shards are run without a cache, so an attention module's cache output stays rank-local.
+how - are those of the reference. The KV-cache rules of the reference (`select_kv_for_rank`, `gather_kv`) have no
+counterpart in the tables: every rank is handed its own cache object (see kv_cache), so an attention module's cache
+stays rank-local without a rule.
 Attribute rules name the attributes of the model classes the reference was written against; attributes
 a given transformers version no longer has are skipped when the shard is built.
 """

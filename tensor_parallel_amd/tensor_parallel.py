@@ -19,6 +19,7 @@ from torch import nn
 from .autoconfig import get_default_config
 from .collectives import set_turn_lock
 from .config import Config, add_lora_rules
+from .kv_cache import is_kv_cache, rank_caches
 from .shard import make_shard
 from .sharding import Sharded
 from .slicing import BatchSlicer, concat_specs
@@ -134,11 +135,17 @@ class TensorParallel(nn.Module):
         self.sharding_manager = Sharded(self, len(self.devices), replicated_param_names)
 
     def prepare_args_kwargs_for_forward(self, *args, **kwargs):
-        """One copy of (args, kwargs) per rank; every tensor is moved to that rank's device (tensor_parallel.py:121-137)."""
+        """One copy of (args, kwargs) per rank; every tensor is moved to that rank's device (tensor_parallel.py:121-137).
+        An attention cache object becomes that rank's own cache (see kv_cache)."""
         structure = (args, kwargs)
+        flat = list(nested_flatten(structure))
+        caches = {i: rank_caches(x, len(self.devices)) for i, x in enumerate(flat) if is_kv_cache(x)}
         per_rank = []
-        for device in self.devices:
-            leaves = [x.to(device, non_blocking=True) if isinstance(x, torch.Tensor) else x for x in nested_flatten(structure)]
+        for rank, device in enumerate(self.devices):
+            leaves = [
+                x.to(device, non_blocking=True) if isinstance(x, torch.Tensor) else (caches[i][rank] if i in caches else x)
+                for i, x in enumerate(flat)
+            ]
             per_rank.append(nested_pack(leaves, structure))
         return zip(*per_rank)
 
