@@ -6,8 +6,9 @@
 // Two kernels share the tiling (block tile BM x BN x 64, WAVES_M x WAVES_N wavefronts of 64 lanes, two LDS
 // stages, one barrier per K tile):
 //   gemm_direct_kernel  256x256 tiles, K % 64 == 0, v_mfma_f32_16x16x32. Global loads go straight into LDS (no
-//                       register staging), operand fragments are read one sub-step ahead of the MFMAs that use
-//                       them, and the loop body is scheduled by hand (see the comment on the kernel).
+//                       register staging); one block per CU walks through several output tiles; the two
+//                       wavefronts of a SIMD alternate between a read phase and a multiply phase (see the
+//                       comment on the kernel).
 //   gemm_kernel         any K (multiple of 8) and the 128x128 tiling for small problems, v_mfma_f32_32x32x16; next
 //                       K tile prefetched into registers while the current one is multiplied.
 #include "common.h"
@@ -361,18 +362,14 @@ __device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[TMX
 // fetches one whole 128-byte row segment.
 //
 // Global->LDS loads go through buffer descriptors (wavefront-uniform base and K offset, 32-bit per-lane offset
-// computed once), fragment reads are inline ds_read_b128 with counted waits, and the loop body is written out
-// instruction by instruction: one fragment read or one load between MFMAs, so LDS, the load path and the matrix
-// pipe see a steady trickle. A K tile is four sub-steps of 16 MFMAs:
-//   S1 (k 0..31, x tiles 0-3)   reads x tiles 4-7 of k 0..31
-//   S2 (k 0..31, x tiles 4-7)   reads x tiles 0-3 and the 4 w tiles of k 32..63
-//   S3 (k 32..63, x tiles 0-3)  reads x tiles 4-7 of k 32..63; then the one barrier of the tile
-//   S4 (k 32..63, x tiles 4-7)  reads x tiles 0-3 and w of k 0..31 of the NEXT tile
-// The loads of the tile after next are issued in S4, S1 and S2 (2 + 3 + 3 per wavefront) into the stage the
-// barrier has just freed.
+// computed once), fragment reads are inline ds_read_b128. The main loop runs in phases that end at workgroup
+// barriers (described where it is written out): the two wavefronts of a SIMD alternate between reading fragments
+// and multiplying. Measured against a loop that interleaved one read or load between MFMAs inside every wavefront:
+// same speed on a single round of tiles, 3-7 % faster when a CU runs several tiles in a row.
 template <int DT, int MODE>
 __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
     constexpr int BM = 256, BN = 256, WAVES_N = 4, NW = 8;
+    constexpr int BN_OUT = MODE == MODE_SWIGLU ? BN / 2 : BN;
     constexpr int BLK = 1152;
     constexpr int XREG = (BM / 8) * BLK, WREG = (BN / 8) * BLK, STAGE = XREG + WREG;
     constexpr int XB = BM / 8 / NW, WB = BN / 8 / NW;  // 1 KiB blocks per wavefront per operand
@@ -380,45 +377,55 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
 
     extern __shared__ __align__(16) char smem[];
 
-    int tile_m, tile_n;
-    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * BM;
-    const int n0 = tile_n * (MODE == MODE_SWIGLU ? BN / 2 : BN);
-
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l16 = lane & 15, lq = lane >> 4;
 
-    // ---- global -> LDS: lane (rb, slot) of a load fetches chunk slot ^ rb of row rb of its block
+    // ---- output tiles of this block: the launch has at most one block per CU and a block walks through tile
+    // ids blockIdx.x, blockIdx.x + gridDim.x, ... (gridDim.x is a multiple of 8 whenever there is more than one
+    // round, so a block stays with one XCD's share of the tiles)
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    const int KT = p.K / BK;
+    const int last = KT - 1;
+
+    // ---- global -> LDS: lane (rb, slot) of a load fetches chunk slot ^ rb of row rb of its block. The load
+    // context (offsets and descriptors) belongs to the tile whose K tiles are being fetched, which is the next
+    // output tile while the last K tile of the current one is multiplied.
     const int rb = lane >> 3, slot = lane & 7;
     const int lchunk = slot ^ rb;
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-    const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
-    const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
-    const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : w_base;
     uint32_t x_off[XB], w_off[WB];
+    __amdgpu_buffer_rsrc_t x_rsrc, w_rsrc, w2_rsrc;
+    auto set_load_tile = [&](int tile_id) {
+        int tile_m, tile_n;
+        tile_of_block(tile_id, total_tiles, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        const int m0 = tile_m * BM, n0 = tile_n * BN_OUT;
+        const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
+        const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
+        const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : w_base;
 #pragma unroll
-    for (int i = 0; i < XB; ++i) {
-        int r = (wave_s + i * NW) * 8 + rb;
-        r = m0 + r < p.M ? r : p.M - 1 - m0;  // clamp to the last valid row of x
-        x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16;
-    }
+        for (int i = 0; i < XB; ++i) {
+            int r = (wave_s + i * NW) * 8 + rb;
+            r = m0 + r < p.M ? r : p.M - 1 - m0;  // clamp to the last valid row of x
+            x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16;
+        }
 #pragma unroll
-    for (int i = 0; i < WB; ++i) {
-        int tr = (wave_s + i * NW) * 8 + rb;
-        if constexpr (MODE == MODE_SWIGLU) tr = tr < BN / 2 ? tr : tr - BN / 2;  // gate rows, then up rows
-        tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
-        w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
-    }
-    // descriptor extents: up to the end of the last valid row below the tile origin
-    const int x_rows = p.M - m0 < BM ? p.M - m0 : BM;
-    const int w_rows = p.N - n0 < BN ? p.N - n0 : BN;
-    const uint32_t x_extent = static_cast<uint32_t>(x_rows - 1) * static_cast<uint32_t>(p.ldx * 2) + static_cast<uint32_t>(p.K) * 2;
-    const uint32_t w_extent = static_cast<uint32_t>(w_rows - 1) * static_cast<uint32_t>(p.ldw * 2) + static_cast<uint32_t>(p.K) * 2;
-    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(x_base, x_extent);
-    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(w_base, w_extent);
-    const __amdgpu_buffer_rsrc_t w2_rsrc = make_rsrc(w2_base, w_extent);
+        for (int i = 0; i < WB; ++i) {
+            int tr = (wave_s + i * NW) * 8 + rb;
+            if constexpr (MODE == MODE_SWIGLU) tr = tr < BN / 2 ? tr : tr - BN / 2;  // gate rows, then up rows
+            tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
+            w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
+        }
+        // descriptor extents: up to the end of the last valid row below the tile origin
+        const int x_rows = p.M - m0 < BM ? p.M - m0 : BM;
+        const int w_rows = p.N - n0 < BN ? p.N - n0 : BN;
+        const uint32_t x_extent = static_cast<uint32_t>(x_rows - 1) * static_cast<uint32_t>(p.ldx * 2) + static_cast<uint32_t>(p.K) * 2;
+        const uint32_t w_extent = static_cast<uint32_t>(w_rows - 1) * static_cast<uint32_t>(p.ldw * 2) + static_cast<uint32_t>(p.K) * 2;
+        x_rsrc = make_rsrc(x_base, x_extent);
+        w_rsrc = make_rsrc(w_base, w_extent);
+        w2_rsrc = make_rsrc(w2_base, w_extent);
+    };
     auto gx = [&](int i, int kt, int stage) {
         buffer_load16_to_lds(x_rsrc, x_off[i], static_cast<uint32_t>(kt) * (BK * 2), smem + stage * STAGE + (wave_s + i * NW) * BLK);
     };
@@ -446,123 +453,99 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
     for (int kk = 0; kk < 2; ++kk) kk_off[kk] = ((kk * 4 + lq) ^ (l16 & 7)) * 16;
 
     f32x4 acc[8][4];
-#pragma unroll
-    for (int a = 0; a < 8; ++a)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    u32x4 xf[2][4], wf[2][4];
     const uint32_t smem_base = lds_addr_of(smem);
-    // LDS reads return in order: "lgkmcnt(N)" = everything but the N youngest reads has landed. The counts below
-    // include the reads of the following sub-step issued in between. Naming a fragment as an operand of the wait
-    // keeps the MFMAs that consume it behind the wait. Everything is pinned in source order by the scheduling
-    // barriers: the compiler must not move a fragment register before its wait.
-#define TPAMD_SB __builtin_amdgcn_sched_barrier(0)
-#define TPAMD_WAIT(N, reg) asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(reg))
-#define TPAMD_MFMA(XS, WS, A0, a, b) acc[(A0) + (a)][b] = mfma16<DT>(wf[WS][b], xf[XS][a], acc[(A0) + (a)][b])
-#define TPAMD_DRAIN_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
-#define TPAMD_ROW(XS, WS, A0, a) TPAMD_MFMA(XS, WS, A0, a, 0); TPAMD_MFMA(XS, WS, A0, a, 1); TPAMD_MFMA(XS, WS, A0, a, 2); TPAMD_MFMA(XS, WS, A0, a, 3)
-    // Sub-step on x tiles 0-3 (fragments xf[0], read in the order x0 w0 w1 w2 w3 x1 x2 x3 by the sub-step before);
-    // reads x tiles 4-7 of the same k range into xf[1]; L0..L2: loads or nothing.
-#define TPAMD_SUB_A(WS, stage_off, kk, L0, L1, L2)                                                                  \
-    {                                                                                                               \
-        const uint32_t xa = smem_base + (stage_off) + x_rd0 + kk_off[kk];                                           \
-        TPAMD_SB;                                                                                                   \
-        TPAMD_WAIT(6, xf[0][0]); TPAMD_WAIT(6, wf[WS][0]); TPAMD_SB;                                                \
-        TPAMD_MFMA(0, WS, 0, 0, 0); TPAMD_SB; xf[1][0] = lds_read16<4 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_WAIT(6, wf[WS][1]); TPAMD_SB;                                                                         \
-        TPAMD_MFMA(0, WS, 0, 0, 1); TPAMD_SB; xf[1][1] = lds_read16<5 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_WAIT(6, wf[WS][2]); TPAMD_SB;                                                                         \
-        TPAMD_MFMA(0, WS, 0, 0, 2); TPAMD_SB; xf[1][2] = lds_read16<6 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_WAIT(6, wf[WS][3]); TPAMD_SB;                                                                         \
-        TPAMD_MFMA(0, WS, 0, 0, 3); TPAMD_SB; xf[1][3] = lds_read16<7 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_WAIT(6, xf[0][1]); TPAMD_SB;                                                                          \
-        TPAMD_ROW(0, WS, 0, 1); TPAMD_SB; L0; TPAMD_SB;                                                             \
-        TPAMD_WAIT(5, xf[0][2]); TPAMD_SB;                                                                          \
-        TPAMD_ROW(0, WS, 0, 2); TPAMD_SB; L1; TPAMD_SB;                                                             \
-        TPAMD_WAIT(4, xf[0][3]); TPAMD_SB;                                                                          \
-        TPAMD_ROW(0, WS, 0, 3); TPAMD_SB; L2; TPAMD_SB;                                                             \
-    }
-    // Sub-step on x tiles 4-7 (fragments xf[1]) with the same w fragments; reads x tiles 0-3 and the w tiles of
-    // (stage_off, kk) into xf[0] and wf[WR].
-#define TPAMD_SUB_B(WS, WR, stage_off, kk, L0, L1, L2)                                                              \
+
+    // Phased schedule: a K step of 32 is a read phase (12 fragment reads; in the first step also the 8 loads of the
+    // following K tile) and a multiply phase (32 MFMAs), every phase ends at a workgroup barrier, and wavefronts
+    // 4-7 run one phase behind wavefronts 0-3. Wavefronts w and w + 4 share a SIMD, so on every SIMD one wavefront
+    // multiplies while the other reads. g counts K tiles across the output tiles of the block, stage = g & 1:
+    //   phase      4g         4g+1       4g+2       4g+3       4g+4
+    //   waves 0-3  R(g,0)+L   M(g,0)     R(g,1)     M(g,1)+V   R(g+1,0)+L
+    //   waves 4-7  M(g-1,1)   R(g,0)+L   M(g,0)     R(g,1)+V   M(g,1)
+    // L = loads of K tile g+1 into the other stage (all of its readers finished before the barrier that starts
+    // phase 4g), V = wait for those loads, before the barrier that starts phase 4g+4 where K tile g+1 is read.
+    // K tile g+1 is the first K tile of the block's next output tile when g is the last of the current one, so a
+    // new output tile starts without a pipeline fill; the epilogue of wavefronts 0-3 runs under the last multiply
+    // phase of wavefronts 4-7.
+    u32x4 xq[8], wq[4];
+#define TPAMD_PP_BARRIER() asm volatile("s_barrier" ::: "memory")
+#define TPAMD_PP_READ(stage_off, kk)                                                                                \
     {                                                                                                               \
         const uint32_t xa = smem_base + (stage_off) + x_rd0 + kk_off[kk];                                           \
         const uint32_t wa = smem_base + (stage_off) + w_rd0 + kk_off[kk];                                           \
-        TPAMD_SB;                                                                                                   \
-        TPAMD_WAIT(3, xf[1][0]); TPAMD_SB;                                                                          \
-        TPAMD_MFMA(1, WS, 4, 0, 0); TPAMD_SB; xf[0][0] = lds_read16<0>(xa); TPAMD_SB;                               \
-        TPAMD_MFMA(1, WS, 4, 0, 1); TPAMD_SB; wf[WR][0] = lds_read16<0>(wa); TPAMD_SB;                              \
-        TPAMD_MFMA(1, WS, 4, 0, 2); TPAMD_SB; wf[WR][1] = lds_read16<WT1>(wa); TPAMD_SB;                            \
-        TPAMD_MFMA(1, WS, 4, 0, 3); TPAMD_SB; wf[WR][2] = lds_read16<WT2>(wa); TPAMD_SB;                            \
-        TPAMD_WAIT(6, xf[1][1]); TPAMD_SB;                                                                          \
-        TPAMD_MFMA(1, WS, 4, 1, 0); TPAMD_SB; wf[WR][3] = lds_read16<WT3>(wa); TPAMD_SB;                            \
-        TPAMD_MFMA(1, WS, 4, 1, 1); TPAMD_SB; xf[0][1] = lds_read16<1 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_MFMA(1, WS, 4, 1, 2); TPAMD_SB; xf[0][2] = lds_read16<2 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_MFMA(1, WS, 4, 1, 3); TPAMD_SB; xf[0][3] = lds_read16<3 * T16>(xa); TPAMD_SB;                         \
-        TPAMD_WAIT(9, xf[1][2]); TPAMD_SB;                                                                          \
-        TPAMD_ROW(1, WS, 4, 2); TPAMD_SB; L0; TPAMD_SB;                                                             \
-        TPAMD_WAIT(8, xf[1][3]); TPAMD_SB;                                                                          \
-        TPAMD_MFMA(1, WS, 4, 3, 0); TPAMD_MFMA(1, WS, 4, 3, 1); TPAMD_SB; L1; TPAMD_SB;                             \
-        TPAMD_MFMA(1, WS, 4, 3, 2); TPAMD_MFMA(1, WS, 4, 3, 3); TPAMD_SB; L2; TPAMD_SB;                             \
+        wq[0] = lds_read16<0>(wa); wq[1] = lds_read16<WT1>(wa); wq[2] = lds_read16<WT2>(wa); wq[3] = lds_read16<WT3>(wa); \
+        xq[0] = lds_read16<0>(xa); xq[1] = lds_read16<1 * T16>(xa); xq[2] = lds_read16<2 * T16>(xa);                \
+        xq[3] = lds_read16<3 * T16>(xa); xq[4] = lds_read16<4 * T16>(xa); xq[5] = lds_read16<5 * T16>(xa);          \
+        xq[6] = lds_read16<6 * T16>(xa); xq[7] = lds_read16<7 * T16>(xa);                                           \
     }
-#define NOP_ (void)0
+#define TPAMD_PP_FRAGS                                                                                              \
+    "+v"(xq[0]), "+v"(xq[1]), "+v"(xq[2]), "+v"(xq[3]), "+v"(xq[4]), "+v"(xq[5]), "+v"(xq[6]), "+v"(xq[7]),         \
+        "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3])
+#define TPAMD_PP_LANDED(VM)                                                                                         \
+    if (VM) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : TPAMD_PP_FRAGS::"memory");                               \
+    else asm volatile("s_waitcnt lgkmcnt(0)" : TPAMD_PP_FRAGS::"memory")
+#define TPAMD_PP_MMA()                                                                                              \
+    _Pragma("unroll") for (int a = 0; a < 8; ++a) _Pragma("unroll") for (int b = 0; b < 4; ++b)                     \
+        acc[a][b] = mfma16<DT>(wq[b], xq[a], acc[a][b]);
+    // one K tile: reads from stage g & 1, loads K tile `kload` of the load context into the other stage
+#define TPAMD_PP_KTILE(LATE, kload)                                                                                 \
+    {                                                                                                               \
+        const int cur = (g & 1) * STAGE, ns = (g + 1) & 1;                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                                          \
+        TPAMD_PP_READ(cur, 0);                                                                                      \
+        gx(0, kload, ns); gx(1, kload, ns); gx(2, kload, ns); gx(3, kload, ns);                                     \
+        gw(0, kload, ns); gw(1, kload, ns); gw(2, kload, ns); gw(3, kload, ns);                                     \
+        TPAMD_PP_LANDED(false); TPAMD_PP_BARRIER();                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                          \
+        TPAMD_PP_MMA();                                                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                          \
+        TPAMD_PP_BARRIER();                                                                                         \
+        TPAMD_PP_READ(cur, 1);                                                                                      \
+        TPAMD_PP_LANDED(LATE); TPAMD_PP_BARRIER();                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                          \
+        TPAMD_PP_MMA();                                                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                          \
+        if (!LATE) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                 \
+        TPAMD_PP_BARRIER();                                                                                         \
+        ++g;                                                                                                        \
+    }
+    // all output tiles of the block; LATE = this wavefront runs one phase behind
+#define TPAMD_PP_RUN(LATE)                                                                                          \
+    for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {                                            \
+        int tile_m, tile_n;                                                                                         \
+        tile_of_block(tile, total_tiles, p.tiles_m, p.tiles_n, tile_m, tile_n);                                     \
+        _Pragma("unroll") for (int a = 0; a < 8; ++a) _Pragma("unroll") for (int b = 0; b < 4; ++b)                 \
+            acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};                                                                  \
+        for (int kt = 0; kt < last; ++kt) TPAMD_PP_KTILE(LATE, kt + 1);                                             \
+        const bool more = tile + static_cast<int>(gridDim.x) < total_tiles;                                         \
+        if (more) set_load_tile(tile + gridDim.x);                                                                  \
+        /* without a next tile the last K tile is fetched again, into the stage nobody reads any more */            \
+        const int kfirst = more ? 0 : last;                                                                         \
+        TPAMD_PP_KTILE(LATE, kfirst);                                                                               \
+        epilogue16<DT, MODE, 8>(p, acc, tile_m * BM + wm * 128, tile_n * BN_OUT + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq); \
+    }
 
-    const int KT = p.K / BK;  // K is a multiple of 64 here
-    const int last = KT - 1;
+    int g = 0;
+    set_load_tile(blockIdx.x);
 #pragma unroll
     for (int i = 0; i < XB; ++i) gx(i, 0, 0);
 #pragma unroll
     for (int i = 0; i < WB; ++i) gw(i, 0, 0);
     drain_and_barrier();
-    {
-        const uint32_t xa = smem_base + x_rd0 + kk_off[0];
-        const uint32_t wa = smem_base + w_rd0 + kk_off[0];
-        xf[0][0] = lds_read16<0>(xa);
-        wf[0][0] = lds_read16<0>(wa);
-        wf[0][1] = lds_read16<WT1>(wa);
-        wf[0][2] = lds_read16<WT2>(wa);
-        wf[0][3] = lds_read16<WT3>(wa);
-        xf[0][1] = lds_read16<1 * T16>(xa);
-        xf[0][2] = lds_read16<2 * T16>(xa);
-        xf[0][3] = lds_read16<3 * T16>(xa);
+    if (wave_s < 4) {
+        TPAMD_PP_RUN(false);
+        TPAMD_PP_BARRIER();
+    } else {
+        TPAMD_PP_BARRIER();
+        TPAMD_PP_RUN(true);
     }
-    // Loads past the last tile are clamped to the last tile: they refill a stage nobody reads any more, which
-    // keeps the loop body free of branches (a branch here makes the compiler copy fragment registers around
-    // before the counted waits, i.e. before their data has landed).
-    gx(0, last < 1 ? last : 1, 1);
-    gx(1, last < 1 ? last : 1, 1);
-    for (int kt = 0; kt < last; ++kt) {
-        const int cur = (kt & 1) * STAGE, nxt = ((kt + 1) & 1) * STAGE;
-        const int ns = (kt + 1) & 1, k1 = kt + 1;
-        TPAMD_SUB_A(0, cur, 0, gx(2, k1, ns), gx(3, k1, ns), gw(0, k1, ns));
-        TPAMD_SUB_B(0, 1, cur, 1, gw(1, k1, ns), gw(2, k1, ns), gw(3, k1, ns));
-        TPAMD_SUB_A(1, cur, 1, NOP_, NOP_, NOP_);
-        // every wavefront is done reading this tile and the next one has landed
-        TPAMD_DRAIN_BARRIER();
-        const int k2 = kt + 2 < last ? kt + 2 : last, cs = kt & 1;
-        TPAMD_SUB_B(1, 0, nxt, 0, NOP_, gx(0, k2, cs), gx(1, k2, cs));
-    }
-    {
-        const int cur = (last & 1) * STAGE;
-        TPAMD_SUB_A(0, cur, 0, NOP_, NOP_, NOP_);
-        TPAMD_SUB_B(0, 1, cur, 1, NOP_, NOP_, NOP_);
-        TPAMD_SUB_A(1, cur, 1, NOP_, NOP_, NOP_);
-        TPAMD_DRAIN_BARRIER();  // also: no global->LDS load is in flight when the wavefront leaves the loop
-        TPAMD_WAIT(0, xf[1][0]); TPAMD_WAIT(0, xf[1][1]); TPAMD_WAIT(0, xf[1][2]); TPAMD_WAIT(0, xf[1][3]);
-        TPAMD_WAIT(0, wf[1][0]); TPAMD_WAIT(0, wf[1][1]); TPAMD_WAIT(0, wf[1][2]); TPAMD_WAIT(0, wf[1][3]);
-        TPAMD_ROW(1, 1, 4, 0); TPAMD_ROW(1, 1, 4, 1); TPAMD_ROW(1, 1, 4, 2); TPAMD_ROW(1, 1, 4, 3);
-    }
-#undef NOP_
-#undef TPAMD_SB
-#undef TPAMD_WAIT
-#undef TPAMD_MFMA
-#undef TPAMD_ROW
-#undef TPAMD_SUB_A
-#undef TPAMD_SUB_B
-#undef TPAMD_DRAIN_BARRIER
-
-    epilogue16<DT, MODE, 8>(p, acc, m0 + wm * 128, n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq);
+#undef TPAMD_PP_BARRIER
+#undef TPAMD_PP_READ
+#undef TPAMD_PP_FRAGS
+#undef TPAMD_PP_LANDED
+#undef TPAMD_PP_MMA
+#undef TPAMD_PP_KTILE
+#undef TPAMD_PP_RUN
 }
 
 // gemm_direct128_kernel: 128 x 128 x 64 tiles for problems whose 256 x 256 tiling would leave CUs idle.
@@ -889,7 +872,7 @@ int launch_gemm(GemmParams p, hipStream_t s) {
 }
 
 template <int DT, int MODE>
-int launch_direct(GemmParams p, hipStream_t s) {
+int launch_direct(GemmParams p, int cus, hipStream_t s) {
     constexpr int LDS = 2 * 64 * 1152;
     auto kern = gemm_direct_kernel<DT, MODE>;
     static thread_local int configured_dev = -1;
@@ -902,8 +885,12 @@ int launch_direct(GemmParams p, hipStream_t s) {
     p.tiles_m = (p.M + 255) / 256;
     constexpr int BN_OUT = MODE == MODE_SWIGLU ? 128 : 256;
     p.tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
-    const int64_t blocks = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-    TPAMD_REQUIRE(blocks < (1ll << 31), "gemm: too many tiles");
+    const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
+    // one block per CU at most (a block needs most of a CU's LDS anyway); a multiple of 8 when blocks take several
+    // tiles, so that a block's tiles all belong to one XCD's share
+    int64_t blocks = tiles;
+    if (tiles > cus) blocks = cus >= 8 ? (cus / 8) * 8 : cus;
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(512), LDS, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
@@ -1025,7 +1012,7 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     const char *force = getenv("TPAMD_GEMM_TILE");
     const bool big = force ? atoi(force) == 256 : big_tiles >= 200;
     if (direct_ok) {
-        if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, s) : launch_direct<DT, MODE_LINEAR>(p, s);
+        if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, s) : launch_direct<DT, MODE_LINEAR>(p, cus, s);
         return swiglu ? launch_direct128<DT, MODE_SWIGLU>(p, cus, s) : launch_direct128<DT, MODE_LINEAR>(p, cus, s);
     }
     if (big) return swiglu ? launch_gemm<DT, MODE_SWIGLU, 256, 256, 2, 4>(p, s) : launch_gemm<DT, MODE_LINEAR, 256, 256, 2, 4>(p, s);
