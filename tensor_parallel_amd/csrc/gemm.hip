@@ -548,6 +548,209 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
 #undef TPAMD_PP_RUN
 }
 
+// gemm_direct4_kernel: the same 256 x 256 x 64 tile with 4 wavefronts (2 x 2, 128 x-rows by 128 w-rows each), one
+// per SIMD with its 64 accumulator tiles in the upper half of the register file. A 128 x 128 wavefront tile reads 16
+// fragments per 64 MFMAs where the 128 x 64 tile of the 8-wavefront kernel reads 12 per 32: a third less LDS traffic
+// per flop, and half the wavefronts to issue loads and waits for. With a single wavefront per SIMD the reads and
+// loads of the next step have to be spread between the MFMAs of the current one by hand:
+//   step (g,0)  64 MFMAs on buffer 0; the 16 fragment reads of (g,1) follow the first 32, one per pair
+//   barrier     every wavefront has read stage g&1 for the last time; K tile g+1 has landed
+//   step (g,1)  64 MFMAs on buffer 1; the 16 reads of (g+1,0) follow the first 32; the 16 loads of K tile g+2 (into
+//               stage g&1) are spread evenly over the step: bunched up they queue in the load path and land late
+// Loads run two K tiles ahead of the multiplies, across output tiles (persistent blocks, as in the 8-wavefront kernel).
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
+    constexpr int BM = 256, BN = 256, NW = 4;
+    constexpr int BN_OUT = MODE == MODE_SWIGLU ? BN / 2 : BN;
+    constexpr int BLK = 1152;
+    constexpr int XREG = (BM / 8) * BLK, WREG = (BN / 8) * BLK, STAGE = XREG + WREG;
+    constexpr int XB = BM / 8 / NW, WB = BN / 8 / NW;
+    static_assert(XB == 8 && WB == 8, "16 loads per wavefront per tile");
+
+    extern __shared__ __align__(16) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    const int KT = p.K / BK;  // at least 2
+    const int last = KT - 1;
+
+    const int rb = lane >> 3, slot = lane & 7;
+    const int lchunk = slot ^ rb;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t x_off[XB], w_off[WB];
+    __amdgpu_buffer_rsrc_t x_rsrc, w_rsrc, w2_rsrc;
+    auto set_load_tile = [&](int tile_id) {
+        int tile_m, tile_n;
+        tile_of_block(tile_id, total_tiles, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        const int m0 = tile_m * BM, n0 = tile_n * BN_OUT;
+        const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
+        const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
+        const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : w_base;
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+            int r = (wave_s + i * NW) * 8 + rb;
+            r = m0 + r < p.M ? r : p.M - 1 - m0;
+            x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16;
+        }
+#pragma unroll
+        for (int i = 0; i < WB; ++i) {
+            int tr = (wave_s + i * NW) * 8 + rb;
+            if constexpr (MODE == MODE_SWIGLU) tr = tr < BN / 2 ? tr : tr - BN / 2;
+            tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
+            w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
+        }
+        const int x_rows = p.M - m0 < BM ? p.M - m0 : BM;
+        const int w_rows = p.N - n0 < BN ? p.N - n0 : BN;
+        const uint32_t x_extent = static_cast<uint32_t>(x_rows - 1) * static_cast<uint32_t>(p.ldx * 2) + static_cast<uint32_t>(p.K) * 2;
+        const uint32_t w_extent = static_cast<uint32_t>(w_rows - 1) * static_cast<uint32_t>(p.ldw * 2) + static_cast<uint32_t>(p.K) * 2;
+        x_rsrc = make_rsrc(x_base, x_extent);
+        w_rsrc = make_rsrc(w_base, w_extent);
+        w2_rsrc = make_rsrc(w2_base, w_extent);
+    };
+    auto gx = [&](int i, int kt, int stage) {
+        buffer_load16_to_lds(x_rsrc, x_off[i], static_cast<uint32_t>(kt) * (BK * 2), smem + stage * STAGE + (wave_s + i * NW) * BLK);
+    };
+    auto gw = [&](int i, int kt, int stage) {
+        const bool up = MODE == MODE_SWIGLU && (wave_s + i * NW) * 8 >= BN / 2;  // i >= 4: known at compile time
+        buffer_load16_to_lds(up ? w2_rsrc : w_rsrc, w_off[i], static_cast<uint32_t>(kt) * (BK * 2),
+                             smem + stage * STAGE + XREG + (wave_s + i * NW) * BLK);
+    };
+
+    constexpr int T16 = 2 * BLK;  // 16 staged rows
+    constexpr int WHI = MODE == MODE_SWIGLU ? (BN / 2 / 8) * BLK : 4 * T16;  // w tiles 4-7: the up rows / the next 64 rows
+    int x_rd0, w_rd0;
+    {
+        const int r = wm * 128 + l16;
+        x_rd0 = (r >> 3) * BLK + (r & 7) * 128;
+        const int row = (MODE == MODE_SWIGLU ? wn * 64 : wn * 128) + l16;
+        w_rd0 = XREG + (row >> 3) * BLK + (row & 7) * 128;
+    }
+    int kk_off[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) kk_off[kk] = ((kk * 4 + lq) ^ (l16 & 7)) * 16;
+
+    f32x4 acc[8][8];
+    u32x4 xq[2][8], wq[2][8];
+    const uint32_t smem_base = lds_addr_of(smem);
+
+#define T4_SB __builtin_amdgcn_sched_barrier(0)
+#define T4_MFMA(buf, a, b) acc[a][b] = mfma16<DT>(wq[buf][b], xq[buf][a], acc[a][b])
+#define T4_PAIR(buf, a, b) T4_MFMA(buf, a, b); T4_MFMA(buf, a, (b) + 1); T4_SB
+#define T4_LANDED(buf)                                                                                              \
+    asm volatile("s_waitcnt lgkmcnt(0)"                                                                             \
+                 : "+v"(xq[buf][0]), "+v"(xq[buf][1]), "+v"(xq[buf][2]), "+v"(xq[buf][3]), "+v"(xq[buf][4]),        \
+                   "+v"(xq[buf][5]), "+v"(xq[buf][6]), "+v"(xq[buf][7]), "+v"(wq[buf][0]), "+v"(wq[buf][1]),        \
+                   "+v"(wq[buf][2]), "+v"(wq[buf][3]), "+v"(wq[buf][4]), "+v"(wq[buf][5]), "+v"(wq[buf][6]),        \
+                   "+v"(wq[buf][7])::"memory")
+    // 64 MFMAs on fragment buffer CUR; reads the fragments of (rd_stage_off, rd_kk) into buffer NXT; L0..L15: loads
+#define T4_STEP(CUR, NXT, rd_stage_off, rd_kk, L0, L1, L2, L3, L4, L5, L6, L7, L8, L9, L10, L11, L12, L13, L14, L15) \
+    {                                                                                                               \
+        const uint32_t xa = smem_base + (rd_stage_off) + x_rd0 + kk_off[rd_kk];                                     \
+        const uint32_t wa = smem_base + (rd_stage_off) + w_rd0 + kk_off[rd_kk];                                     \
+        T4_SB; T4_LANDED(CUR); T4_SB;                                                                               \
+        T4_PAIR(CUR, 0, 0); wq[NXT][0] = lds_read16<0>(wa); T4_SB;                                                  \
+        T4_PAIR(CUR, 0, 2); wq[NXT][1] = lds_read16<1 * T16>(wa); T4_SB; L0; T4_SB;                                 \
+        T4_PAIR(CUR, 0, 4); wq[NXT][2] = lds_read16<2 * T16>(wa); T4_SB;                                            \
+        T4_PAIR(CUR, 0, 6); wq[NXT][3] = lds_read16<3 * T16>(wa); T4_SB; L1; T4_SB;                                 \
+        T4_PAIR(CUR, 1, 0); wq[NXT][4] = lds_read16<WHI>(wa); T4_SB;                                                \
+        T4_PAIR(CUR, 1, 2); wq[NXT][5] = lds_read16<WHI + 1 * T16>(wa); T4_SB; L2; T4_SB;                           \
+        T4_PAIR(CUR, 1, 4); wq[NXT][6] = lds_read16<WHI + 2 * T16>(wa); T4_SB;                                      \
+        T4_PAIR(CUR, 1, 6); wq[NXT][7] = lds_read16<WHI + 3 * T16>(wa); T4_SB; L3; T4_SB;                           \
+        T4_PAIR(CUR, 2, 0); xq[NXT][0] = lds_read16<0>(xa); T4_SB;                                                  \
+        T4_PAIR(CUR, 2, 2); xq[NXT][1] = lds_read16<1 * T16>(xa); T4_SB; L4; T4_SB;                                 \
+        T4_PAIR(CUR, 2, 4); xq[NXT][2] = lds_read16<2 * T16>(xa); T4_SB;                                            \
+        T4_PAIR(CUR, 2, 6); xq[NXT][3] = lds_read16<3 * T16>(xa); T4_SB; L5; T4_SB;                                 \
+        T4_PAIR(CUR, 3, 0); xq[NXT][4] = lds_read16<4 * T16>(xa); T4_SB;                                            \
+        T4_PAIR(CUR, 3, 2); xq[NXT][5] = lds_read16<5 * T16>(xa); T4_SB; L6; T4_SB;                                 \
+        T4_PAIR(CUR, 3, 4); xq[NXT][6] = lds_read16<6 * T16>(xa); T4_SB;                                            \
+        T4_PAIR(CUR, 3, 6); xq[NXT][7] = lds_read16<7 * T16>(xa); T4_SB; L7; T4_SB;                                 \
+        T4_PAIR(CUR, 4, 0); T4_PAIR(CUR, 4, 2); L8; T4_SB; T4_PAIR(CUR, 4, 4); T4_PAIR(CUR, 4, 6); L9; T4_SB;       \
+        T4_PAIR(CUR, 5, 0); T4_PAIR(CUR, 5, 2); L10; T4_SB; T4_PAIR(CUR, 5, 4); T4_PAIR(CUR, 5, 6); L11; T4_SB;     \
+        T4_PAIR(CUR, 6, 0); T4_PAIR(CUR, 6, 2); L12; T4_SB; T4_PAIR(CUR, 6, 4); T4_PAIR(CUR, 6, 6); L13; T4_SB;     \
+        T4_PAIR(CUR, 7, 0); T4_PAIR(CUR, 7, 2); L14; T4_SB; T4_PAIR(CUR, 7, 4); T4_PAIR(CUR, 7, 6); L15; T4_SB;     \
+    }
+#define T4_NOP (void)0
+    // one K tile; kload = K tile (of the load context) fetched into the stage this one leaves
+#define T4_KTILE(kload)                                                                                             \
+    {                                                                                                               \
+        const int cur = (g & 1) * STAGE, nxt = ((g + 1) & 1) * STAGE, cs = g & 1;                                   \
+        T4_STEP(0, 1, cur, 1, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, \
+                T4_NOP, T4_NOP, T4_NOP);                                                                            \
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                    \
+        T4_STEP(1, 0, nxt, 0, gx(0, kload, cs), gw(0, kload, cs), gx(1, kload, cs), gw(1, kload, cs), gx(2, kload, cs), gw(2, kload, cs), \
+                gx(3, kload, cs), gw(3, kload, cs), gx(4, kload, cs), gw(4, kload, cs), gx(5, kload, cs), gw(5, kload, cs),    \
+                gx(6, kload, cs), gw(6, kload, cs), gx(7, kload, cs), gw(7, kload, cs));                            \
+        ++g;                                                                                                        \
+    }
+
+    int g = 0;
+    set_load_tile(blockIdx.x);
+#pragma unroll
+    for (int i = 0; i < XB; ++i) gx(i, 0, 0);
+#pragma unroll
+    for (int i = 0; i < WB; ++i) gw(i, 0, 0);
+    drain_and_barrier();
+#pragma unroll
+    for (int i = 0; i < XB; ++i) gx(i, 1, 1);
+#pragma unroll
+    for (int i = 0; i < WB; ++i) gw(i, 1, 1);
+    {
+        const uint32_t xa = smem_base + x_rd0 + kk_off[0];
+        const uint32_t wa = smem_base + w_rd0 + kk_off[0];
+        wq[0][0] = lds_read16<0>(wa); wq[0][1] = lds_read16<1 * T16>(wa); wq[0][2] = lds_read16<2 * T16>(wa); wq[0][3] = lds_read16<3 * T16>(wa);
+        wq[0][4] = lds_read16<WHI>(wa); wq[0][5] = lds_read16<WHI + 1 * T16>(wa); wq[0][6] = lds_read16<WHI + 2 * T16>(wa); wq[0][7] = lds_read16<WHI + 3 * T16>(wa);
+        xq[0][0] = lds_read16<0>(xa); xq[0][1] = lds_read16<1 * T16>(xa); xq[0][2] = lds_read16<2 * T16>(xa); xq[0][3] = lds_read16<3 * T16>(xa);
+        xq[0][4] = lds_read16<4 * T16>(xa); xq[0][5] = lds_read16<5 * T16>(xa); xq[0][6] = lds_read16<6 * T16>(xa); xq[0][7] = lds_read16<7 * T16>(xa);
+    }
+    for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+        int tile_m, tile_n;
+        tile_of_block(tile, total_tiles, p.tiles_m, p.tiles_n, tile_m, tile_n);
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+            for (int b = 0; b < 8; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int kt = 0; kt + 2 < KT; ++kt) T4_KTILE(kt + 2);
+        const bool more = tile + static_cast<int>(gridDim.x) < total_tiles;
+        if (more) set_load_tile(tile + gridDim.x);
+        // without a next tile the last K tile is fetched again, into stages nobody reads any more
+        const int k0 = more ? 0 : last, k1 = more ? 1 : last;
+        T4_KTILE(k0);
+        T4_KTILE(k1);
+        // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up
+        const int m_wave = tile_m * BM + wm * 128;
+        const int n_wave = tile_n * BN_OUT + (MODE == MODE_SWIGLU ? wn * 64 : wn * 128);
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+            const int m = m_wave + a * 16 + l16;
+            if (m >= p.M) continue;
+            char *yrow = p.y + static_cast<int64_t>(m) * p.ldy * 2;
+#pragma unroll
+            for (int b = 0; b < (MODE == MODE_SWIGLU ? 4 : 8); ++b) {
+                const int n = n_wave + b * 16 + lq * 4;
+                if (n >= p.N) continue;
+                float gsum[4], usum[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    gsum[j] = acc[a][b][j];
+                    usum[j] = MODE == MODE_SWIGLU ? acc[a][(b + 4) & 7][j] : 0.f;
+                }
+                *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = finish4<DT, MODE>(p, gsum, usum, n);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no global->LDS load in flight when the wavefront leaves
+#undef T4_SB
+#undef T4_MFMA
+#undef T4_PAIR
+#undef T4_LANDED
+#undef T4_STEP
+#undef T4_NOP
+#undef T4_KTILE
+}
+
 // gemm_direct128_kernel: 128 x 128 x 64 tiles for problems whose 256 x 256 tiling would leave CUs idle.
 // 4 wavefronts (2 x 2, 64 x-rows by 64 w-rows each), NS LDS stages of 36 KiB: NS = 2 lets two blocks share a CU,
 // NS = 4 gives one block three tiles of look-ahead. Same LDS layout, loads, fragment reads and hand-ordered loop
@@ -874,12 +1077,15 @@ int launch_gemm(GemmParams p, hipStream_t s) {
 template <int DT, int MODE>
 int launch_direct(GemmParams p, int cus, hipStream_t s) {
     constexpr int LDS = 2 * 64 * 1152;
-    auto kern = gemm_direct_kernel<DT, MODE>;
+    const char *w4 = getenv("TPAMD_GEMM_W4");
+    const bool four = w4 != nullptr && atoi(w4) != 0 && p.K >= 128;
+    auto kern = four ? gemm_direct4_kernel<DT, MODE> : gemm_direct_kernel<DT, MODE>;
     static thread_local int configured_dev = -1;
     int dev = 0;
     TPAMD_HIP(hipGetDevice(&dev));
     if (configured_dev != dev) {
-        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct_kernel<DT, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct4_kernel<DT, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         configured_dev = dev;
     }
     p.tiles_m = (p.M + 255) / 256;
@@ -891,7 +1097,7 @@ int launch_direct(GemmParams p, int cus, hipStream_t s) {
     // tiles, so that a block's tiles all belong to one XCD's share
     int64_t blocks = tiles;
     if (tiles > cus) blocks = cus >= 8 ? (cus / 8) * 8 : cus;
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(512), LDS, s, p);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(four ? 256 : 512), LDS, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }
