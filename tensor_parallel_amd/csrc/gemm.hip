@@ -680,9 +680,9 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         T4_STEP(0, 1, cur, 1, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, \
                 T4_NOP, T4_NOP, T4_NOP);                                                                            \
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                    \
-        T4_STEP(1, 0, nxt, 0, gx(0, kload, cs), gw(0, kload, cs), gx(1, kload, cs), gw(1, kload, cs), gx(2, kload, cs), gw(2, kload, cs), \
-                gx(3, kload, cs), gw(3, kload, cs), gx(4, kload, cs), gw(4, kload, cs), gx(5, kload, cs), gw(5, kload, cs),    \
-                gx(6, kload, cs), gw(6, kload, cs), gx(7, kload, cs), gw(7, kload, cs));                            \
+        T4_STEP(1, 0, nxt, 0, gx(0, kload, cs), gx(1, kload, cs), gx(2, kload, cs), gx(3, kload, cs), gx(4, kload, cs), gx(5, kload, cs), \
+                gx(6, kload, cs), gx(7, kload, cs), gw(0, kload, cs), gw(1, kload, cs), gw(2, kload, cs), gw(3, kload, cs),    \
+                gw(4, kload, cs), gw(5, kload, cs), gw(6, kload, cs), gw(7, kload, cs));                            \
         ++g;                                                                                                        \
     }
 
