@@ -673,13 +673,22 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         T4_PAIR(CUR, 7, 0); T4_PAIR(CUR, 7, 2); L14; T4_SB; T4_PAIR(CUR, 7, 4); T4_PAIR(CUR, 7, 6); L15; T4_SB;     \
     }
 #define T4_NOP (void)0
+#if defined(T4_ABL_NOVM)
+#define T4_TILE_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#elif defined(T4_ABL_NOBAR)
+#define T4_TILE_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory")
+#elif defined(T4_ABL_NOSYNC)
+#define T4_TILE_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
+#else
+#define T4_TILE_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#endif
     // one K tile; kload = K tile (of the load context) fetched into the stage this one leaves
 #define T4_KTILE(kload)                                                                                             \
     {                                                                                                               \
         const int cur = (g & 1) * STAGE, nxt = ((g + 1) & 1) * STAGE, cs = g & 1;                                   \
         T4_STEP(0, 1, cur, 1, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, \
                 T4_NOP, T4_NOP, T4_NOP);                                                                            \
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");                                    \
+        T4_TILE_BARRIER();                                                                                          \
         T4_STEP(1, 0, nxt, 0, gx(0, kload, cs), gx(1, kload, cs), gx(2, kload, cs), gx(3, kload, cs), gx(4, kload, cs), gx(5, kload, cs), \
                 gx(6, kload, cs), gx(7, kload, cs), gw(0, kload, cs), gw(1, kload, cs), gw(2, kload, cs), gw(3, kload, cs),    \
                 gw(4, kload, cs), gw(5, kload, cs), gw(6, kload, cs), gw(7, kload, cs));                            \
@@ -749,6 +758,7 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
 #undef T4_STEP
 #undef T4_NOP
 #undef T4_KTILE
+#undef T4_TILE_BARRIER
 }
 
 // gemm_direct128_kernel: 128 x 128 x 64 tiles for problems whose 256 x 256 tiling would leave CUs idle.
@@ -1078,7 +1088,10 @@ template <int DT, int MODE>
 int launch_direct(GemmParams p, int cus, hipStream_t s) {
     constexpr int LDS = 2 * 64 * 1152;
     const char *w4 = getenv("TPAMD_GEMM_W4");
-    const bool four = w4 != nullptr && atoi(w4) != 0 && p.K >= 128;
+#ifndef TPAMD_W4_DEFAULT
+#define TPAMD_W4_DEFAULT 0
+#endif
+    const bool four = (w4 != nullptr ? atoi(w4) != 0 : TPAMD_W4_DEFAULT != 0) && p.K >= 128;
     auto kern = four ? gemm_direct4_kernel<DT, MODE> : gemm_direct_kernel<DT, MODE>;
     static thread_local int configured_dev = -1;
     int dev = 0;
