@@ -5,10 +5,13 @@
 //
 // Two kernels share the tiling (block tile BM x BN x 64, WAVES_M x WAVES_N wavefronts of 64 lanes, two LDS
 // stages, one barrier per K tile):
-//   gemm_direct_kernel  256x256 tiles, K % 64 == 0, v_mfma_f32_16x16x32. Global loads go straight into LDS (no
-//                       register staging); one block per CU walks through several output tiles; the two
-//                       wavefronts of a SIMD alternate between a read phase and a multiply phase (see the
-//                       comment on the kernel).
+//   gemm_direct4_kernel 256x256 tiles, K % 64 == 0, K >= 128, v_mfma_f32_16x16x32. Global loads go straight into LDS
+//                       (no register staging); one block of 4 wavefronts (128x128 outputs each, accumulators in
+//                       AGPRs) per CU walks through several output tiles; reads and loads of the next step are
+//                       placed by hand between the MFMAs of the current one. The default for large problems.
+//   gemm_direct_kernel  the same tile with 8 wavefronts (128x64 each): the two wavefronts of a SIMD alternate
+//                       between a read phase and a multiply phase. Takes K == 64; within 1-8 % of the 4-wavefront
+//                       kernel elsewhere (TPAMD_GEMM_W4=0 selects it).
 //   gemm_kernel         any K (multiple of 8) and the 128x128 tiling for small problems, v_mfma_f32_32x32x16; next
 //                       K tile prefetched into registers while the current one is multiplied.
 #include "common.h"
@@ -1089,7 +1092,7 @@ int launch_direct(GemmParams p, int cus, hipStream_t s) {
     constexpr int LDS = 2 * 64 * 1152;
     const char *w4 = getenv("TPAMD_GEMM_W4");
 #ifndef TPAMD_W4_DEFAULT
-#define TPAMD_W4_DEFAULT 0
+#define TPAMD_W4_DEFAULT 1
 #endif
     const bool four = (w4 != nullptr ? atoi(w4) != 0 : TPAMD_W4_DEFAULT != 0) && p.K >= 128;
     auto kern = four ? gemm_direct4_kernel<DT, MODE> : gemm_direct_kernel<DT, MODE>;
