@@ -592,18 +592,24 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
         const char *w_base = p.w + static_cast<int64_t>(n0) * p.ldw * 2;
         const char *w2_base = MODE == MODE_SWIGLU ? p.w2 + static_cast<int64_t>(n0) * p.ldw * 2 : w_base;
+        // A wavefront fetches 8 consecutive 1 KiB blocks (64 rows) of each operand. Four consecutive blocks share one
+        // LDS base (M0) and differ in the instruction's immediate offset, which the hardware also adds to the global
+        // address: it is taken off the per-lane offset here. A valid row is at least 8 * (i % 4) rows into the tile,
+        // i.e. at least (i % 4) * 2048 bytes (K >= 128), so the difference stays non-negative; rows past the end are
+        // clamped to the last valid row first, and if the difference then wraps, the range check returns zeros for
+        // them, which is as good as any other value for rows whose outputs are not stored.
 #pragma unroll
         for (int i = 0; i < XB; ++i) {
-            int r = (wave_s + i * NW) * 8 + rb;
+            int r = (wave_s * XB + i) * 8 + rb;
             r = m0 + r < p.M ? r : p.M - 1 - m0;
-            x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16;
+            x_off[i] = static_cast<uint32_t>(r) * static_cast<uint32_t>(p.ldx * 2) + lchunk * 16 - (i & 3) * BLK;
         }
 #pragma unroll
         for (int i = 0; i < WB; ++i) {
-            int tr = (wave_s + i * NW) * 8 + rb;
+            int tr = (wave_s * WB + i) * 8 + rb;
             if constexpr (MODE == MODE_SWIGLU) tr = tr < BN / 2 ? tr : tr - BN / 2;
             tr = n0 + tr < p.N ? tr : p.N - 1 - n0;
-            w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16;
+            w_off[i] = static_cast<uint32_t>(tr) * static_cast<uint32_t>(p.ldw * 2) + lchunk * 16 - (i & 3) * BLK;
         }
         const int x_rows = p.M - m0 < BM ? p.M - m0 : BM;
         const int w_rows = p.N - n0 < BN ? p.N - n0 : BN;
@@ -613,14 +619,18 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         w_rsrc = make_rsrc(w_base, w_extent);
         w2_rsrc = make_rsrc(w2_base, w_extent);
     };
-    auto gx = [&](int i, int kt, int stage) {
-        buffer_load16_to_lds(x_rsrc, x_off[i], static_cast<uint32_t>(kt) * (BK * 2), smem + stage * STAGE + (wave_s + i * NW) * BLK);
+    auto gx = [&](auto ic, int kt, int stage) {
+        constexpr int i = decltype(ic)::value;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (lds_void *)(smem + stage * STAGE + (wave_s * XB + (i & ~3)) * BLK), 16,
+                                                 static_cast<int>(x_off[i]), kt * (BK * 2), (i & 3) * BLK, 0);
     };
-    auto gw = [&](int i, int kt, int stage) {
-        const bool up = MODE == MODE_SWIGLU && (wave_s + i * NW) * 8 >= BN / 2;  // i >= 4: known at compile time
-        buffer_load16_to_lds(up ? w2_rsrc : w_rsrc, w_off[i], static_cast<uint32_t>(kt) * (BK * 2),
-                             smem + stage * STAGE + XREG + (wave_s + i * NW) * BLK);
+    auto gw = [&](auto ic, int kt, int stage) {
+        constexpr int i = decltype(ic)::value;
+        const bool up = MODE == MODE_SWIGLU && wave_s >= NW / 2;  // wavefronts 2 and 3 fetch the up rows
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(up ? w2_rsrc : w_rsrc, (lds_void *)(smem + stage * STAGE + XREG + (wave_s * WB + (i & ~3)) * BLK), 16,
+                                                 static_cast<int>(w_off[i]), kt * (BK * 2), (i & 3) * BLK, 0);
     };
+#define IC(n) std::integral_constant<int, n>{}
 
     constexpr int T16 = 2 * BLK;  // 16 staged rows
     constexpr int WHI = MODE == MODE_SWIGLU ? (BN / 2 / 8) * BLK : 4 * T16;  // w tiles 4-7: the up rows / the next 64 rows
@@ -692,23 +702,23 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         T4_STEP(0, 1, cur, 1, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, T4_NOP, \
                 T4_NOP, T4_NOP, T4_NOP);                                                                            \
         T4_TILE_BARRIER();                                                                                          \
-        T4_STEP(1, 0, nxt, 0, gx(0, kload, cs), gx(1, kload, cs), gx(2, kload, cs), gx(3, kload, cs), gx(4, kload, cs), gx(5, kload, cs), \
-                gx(6, kload, cs), gx(7, kload, cs), gw(0, kload, cs), gw(1, kload, cs), gw(2, kload, cs), gw(3, kload, cs),    \
-                gw(4, kload, cs), gw(5, kload, cs), gw(6, kload, cs), gw(7, kload, cs));                            \
+        T4_STEP(1, 0, nxt, 0, gx(IC(0), kload, cs), gx(IC(1), kload, cs), gx(IC(2), kload, cs), gx(IC(3), kload, cs), gx(IC(4), kload, cs), gx(IC(5), kload, cs), \
+                gx(IC(6), kload, cs), gx(IC(7), kload, cs), gw(IC(0), kload, cs), gw(IC(1), kload, cs), gw(IC(2), kload, cs), gw(IC(3), kload, cs),    \
+                gw(IC(4), kload, cs), gw(IC(5), kload, cs), gw(IC(6), kload, cs), gw(IC(7), kload, cs));                            \
         ++g;                                                                                                        \
     }
 
     int g = 0;
     set_load_tile(blockIdx.x);
-#pragma unroll
-    for (int i = 0; i < XB; ++i) gx(i, 0, 0);
-#pragma unroll
-    for (int i = 0; i < WB; ++i) gw(i, 0, 0);
+#define T4_ALL_LOADS(kt, stage)                                                                                     \
+    gx(IC(0), kt, stage); gx(IC(1), kt, stage); gx(IC(2), kt, stage); gx(IC(3), kt, stage); gx(IC(4), kt, stage);   \
+    gx(IC(5), kt, stage); gx(IC(6), kt, stage); gx(IC(7), kt, stage); gw(IC(0), kt, stage); gw(IC(1), kt, stage);   \
+    gw(IC(2), kt, stage); gw(IC(3), kt, stage); gw(IC(4), kt, stage); gw(IC(5), kt, stage); gw(IC(6), kt, stage);   \
+    gw(IC(7), kt, stage)
+    T4_ALL_LOADS(0, 0);
     drain_and_barrier();
-#pragma unroll
-    for (int i = 0; i < XB; ++i) gx(i, 1, 1);
-#pragma unroll
-    for (int i = 0; i < WB; ++i) gw(i, 1, 1);
+    T4_ALL_LOADS(1, 1);
+#undef T4_ALL_LOADS
     {
         const uint32_t xa = smem_base + x_rd0 + kk_off[0];
         const uint32_t wa = smem_base + w_rd0 + kk_off[0];
@@ -761,6 +771,7 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
 #undef T4_STEP
 #undef T4_NOP
 #undef T4_KTILE
+#undef IC
 #undef T4_TILE_BARRIER
 }
 
