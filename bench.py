@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # Fabric bytes per launch of the fused gate/up GEMM at M = 4096, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
 # each scaled by what the same counter reads for the slicing kernel's known 13.476 GB (factors 1.994 and 1.000):
 # profiles/pmc_fetch_write_bench_kernels.txt. A counter reading cannot be taken inside this script.
-MEASURED_TRAFFIC_BYTES_M4096 = 637.2e6
+MEASURED_TRAFFIC_BYTES_M4096 = 649.0e6
 
 
 def cpu_baseline(seconds_budget: float = 15.0) -> dict:
@@ -126,7 +126,7 @@ def main() -> int:
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_M4096 if M == 4096 else None,
                     "traffic_unit": "bytes per launch (L2<->fabric, rocprofv3 --pmc; algorithmic 168.8e6)",
-                    "kernel": "gemm_direct_kernel<bf16, swiglu> (tpamd_swiglu_up)", "avg_launch_ms": up_ms,
+                    "kernel": "gemm_direct4_kernel<bf16, swiglu> (tpamd_swiglu_up)", "avg_launch_ms": up_ms,
                     "algorithmic_flops_per_launch": up_flops}
     else:
         up_bytes = 2.0 * FFN_SHARD * D_MODEL * 2 + M * D_MODEL * 2 + M * FFN_SHARD * 2
