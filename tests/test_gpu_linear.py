@@ -203,3 +203,41 @@ def test_mid_sized_linear_inside_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         assert torch.equal(_native.linear(x, w), eager)  # eager work between replays
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(300, 520, 128), (513, 260, 192), (700, 1028, 320), (256, 256, 64), (1030, 772, 1088)])
+@pytest.mark.parametrize("waves", [4, 8])
+def test_256_tiles_on_ragged_shapes(dtype, M, N, K, waves, monkeypatch):
+    """The 256 x 256 tiling (forced through the library's debugging knobs; by default it is taken from about 200
+    tiles on) with 4 and with 8 wavefronts per block: two-tile K (the pipeline's minimum), tile rows past M, tile
+    columns past N, bias and GELU, the gated pair, and a strided x. K = 64 is always served by the 8-wavefront
+    kernel. Blocks that walk through several tiles are covered by the next test and by the full-shape tests."""
+    monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
+    monkeypatch.setenv("TPAMD_GEMM_W4", "1" if waves == 4 else "0")
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
+    check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
+    w2 = rnd((N, K), 5, 0.02, dtype)
+    h = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    wide = rnd((M, 2 * K), 3, 1.0, dtype).to(DEV)
+    strided = wide[:, K:]  # row pitch 2K: what a row-parallel shard sees of an unsplit activation
+    got = _native.linear(strided, w.to(DEV))
+    check_half(got, F.linear(strided.float().cpu(), w.float()), K)
+
+
+def test_both_256_tile_kernels_agree_bit_for_bit(monkeypatch):
+    """Same products added in the same order: the 4- and the 8-wavefront kernel must give identical results, also
+    when a block walks through several tiles (3 x 96 = 288 tiles on at most 256 blocks)."""
+    M, N, K = 700, 24500, 256
+    x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
+    monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
+    monkeypatch.setenv("TPAMD_GEMM_W4", "1")
+    four = _native.linear(x, w)
+    monkeypatch.setenv("TPAMD_GEMM_W4", "0")
+    eight = _native.linear(x, w)
+    assert torch.equal(four, eight)
+    check_half(four[:, :512], F.linear(x.float().cpu(), w[:512].float().cpu()), K)
+    check_half(four[:, -512:], F.linear(x.float().cpu(), w[-512:].float().cpu()), K)
