@@ -1171,6 +1171,24 @@ int configure128(int dev) {
     return TPAMD_OK;
 }
 
+// Predicted time (microseconds) of the 128 x 128 tiling and the K split that gives it, from a small cost model
+// fitted on this part: a block that has its CU to itself takes 0.8 per K tile, two blocks sharing a CU 1.0 each
+// (the pace of the CU's global->LDS path), blocks beyond two per CU wait for the next round; the partial tiles cost
+// 3 + 0.18 per MB (written, read back and finished by a second launch).
+inline double estimate128(int64_t tiles, int KT, int cus, int *splits) {
+    double best = 1e30;
+    *splits = 1;
+    for (int sp = 1; sp <= 8; ++sp) {
+        const int kt = (KT + sp - 1) / sp;
+        if (sp > 1 && (kt < 4 || tiles * sp > 4ll * cus)) break;  // too little K per split / more than the scratch buffer holds
+        const double units = static_cast<double>(tiles) * sp;
+        const double rounds = units <= cus ? 1.0 : static_cast<double>((static_cast<int64_t>(units) + 2 * cus - 1) / (2 * cus));
+        const double t = rounds * kt * (units <= cus ? 0.8 : 1.0) + (sp > 1 ? 3.0 + units * 0.065536 * 0.18 : 0.0);
+        if (t < best) { best = t; *splits = sp; }
+    }
+    return best;
+}
+
 // 128 x 128 tiles; split over K (fp32 partial tiles in stream-ordered scratch memory, then one finishing pass)
 // when the tiles alone would not give every CU two blocks.
 template <int DT, int MODE>
@@ -1184,23 +1202,9 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     TPAMD_REQUIRE(tiles < 65536 || tiles >= 2 * cus, "gemm: too many tiles");  // the finishing pass indexes tiles with blockIdx.y
     TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
     const int KT = p.K / 64;
-    // Split factor from a small cost model fitted on this part (microseconds): a block that has its CU to itself
-    // takes 0.8 per K tile, two blocks sharing a CU 1.0 each, blocks beyond two per CU wait for the next round; the
-    // partial tiles cost 3 + 0.18 per MB (written, read back and finished by a second launch).
     int splits = 1;
-    if (const char *e = getenv("TPAMD_GEMM_SPLITK")) {
-        splits = atoi(e);
-    } else {
-        double best = 1e30;
-        for (int sp = 1; sp <= 8; ++sp) {
-            const int kt = (KT + sp - 1) / sp;
-            if (sp > 1 && (kt < 4 || tiles * sp > 4ll * cus)) break;  // too little K per split / more than the scratch buffer holds
-            const double units = static_cast<double>(tiles) * sp;
-            const double rounds = units <= cus ? 1.0 : static_cast<double>((static_cast<int64_t>(units) + 2 * cus - 1) / (2 * cus));
-            const double t = rounds * kt * (units <= cus ? 0.8 : 1.0) + (sp > 1 ? 3.0 + units * 0.065536 * 0.18 : 0.0);
-            if (t < best) { best = t; splits = sp; }
-        }
-    }
+    if (const char *e = getenv("TPAMD_GEMM_SPLITK")) splits = atoi(e);
+    else estimate128(tiles, KT, cus, &splits);
     if (splits > 8) splits = 8;
     if (splits > KT) splits = KT;
     if (splits < 1) splits = 1;
@@ -1240,10 +1244,18 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     // the direct kernels address a tile with 32-bit byte offsets from the tile origin and step K in tiles of 64
     const bool direct_ok = p.K % 64 == 0 && p.K >= 64 && p.ldx < (1ll << 22) && p.ldw < (1ll << 22);
-    // 256x256 tiles once they fill the chip at least about once, else 128x128 tiles.
+    // 256 x 256 tiles or 128 x 128 tiles (with K split): whichever the cost models predict to be faster. The 256 tiles
+    // run in rounds of one per CU; a K tile takes about 1.45 us in a full round (the part is power-limited then) and
+    // 1.3 us in a round that fills at most three quarters of the CUs; fill and epilogue add about 8 us.
     const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
+    const int64_t small_tiles = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128));
+    const int KT = static_cast<int>(p.K / 64);
+    const int64_t full_rounds = big_tiles / cus, last_round = big_tiles % cus;
+    const double t256 = 8.0 + KT * (full_rounds * 1.45 + (last_round == 0 ? 0.0 : last_round * 4 <= 3ll * cus ? 1.3 : 1.45));
+    int unused_splits = 1;
+    const double t128 = estimate128(small_tiles, KT, cus, &unused_splits);
     const char *force = getenv("TPAMD_GEMM_TILE");
-    const bool big = force ? atoi(force) == 256 : big_tiles >= 200;
+    const bool big = force ? atoi(force) == 256 : (t256 < t128 || small_tiles >= 65536);
     if (direct_ok) {
         if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, s) : launch_direct<DT, MODE_LINEAR>(p, cus, s);
         return swiglu ? launch_direct128<DT, MODE_SWIGLU>(p, cus, s) : launch_direct128<DT, MODE_LINEAR>(p, cus, s);
