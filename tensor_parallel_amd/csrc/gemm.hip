@@ -42,6 +42,7 @@ struct GemmParams {
     int tiles_m, tiles_n;
     float *ws;          // split-K: partial tiles, [split][tile][128 w rows][128 x rows] fp32
     int kt_per_split;   // split-K: K tiles (of 64) per split
+    int splits;         // split-K of the 256 x 256 kernel: work units = tiles x splits
 };
 
 constexpr int BK = 64;            // K elements per stage (128 bytes of a row)
@@ -561,7 +562,10 @@ __global__ __launch_bounds__(512) void gemm_direct_kernel(GemmParams p) {
 //   step (g,1)  64 MFMAs on buffer 1; the 16 reads of (g+1,0) follow the first 32; the 16 loads of K tile g+2 (into
 //               stage g&1) are spread evenly over the step: bunched up they queue in the load path and land late
 // Loads run two K tiles ahead of the multiplies, across output tiles (persistent blocks, as in the 8-wavefront kernel).
-template <int DT, int MODE>
+// SPLIT: a block's unit of work is (tile, K range of p.kt_per_split K tiles, at least 2); unit u is tile u % tiles,
+// split u / tiles. Each wavefront leaves its 128 x 128 fp32 sums as one partial tile of the 128 x 128 tiling in p.ws,
+// in the layout splitk_finish_kernel reads.
+template <int DT, int MODE, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
     constexpr int BM = 256, BN = 256, NW = 4;
     constexpr int BN_OUT = MODE == MODE_SWIGLU ? BN / 2 : BN;
@@ -577,16 +581,19 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, lq = lane >> 4;
     const int total_tiles = p.tiles_m * p.tiles_n;
-    const int KT = p.K / BK;  // at least 2
-    const int last = KT - 1;
+    const int total_units = SPLIT ? total_tiles * p.splits : total_tiles;
+    const int KT_ALL = p.K / BK;  // at least 2
 
     const int rb = lane >> 3, slot = lane & 7;
     const int lchunk = slot ^ rb;
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     uint32_t x_off[XB], w_off[WB];
     __amdgpu_buffer_rsrc_t x_rsrc, w_rsrc, w2_rsrc;
-    auto set_load_tile = [&](int tile_id) {
+    int kbase = 0;  // first K tile of the unit the loads are fetching
+    auto set_load_tile = [&](int unit) {
         int tile_m, tile_n;
+        const int tile_id = SPLIT ? unit % total_tiles : unit;
+        if constexpr (SPLIT) kbase = (unit / total_tiles) * p.kt_per_split;
         tile_of_block(tile_id, total_tiles, p.tiles_m, p.tiles_n, tile_m, tile_n);
         const int m0 = tile_m * BM, n0 = tile_n * BN_OUT;
         const char *x_base = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
@@ -622,13 +629,13 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
     auto gx = [&](auto ic, int kt, int stage) {
         constexpr int i = decltype(ic)::value;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (lds_void *)(smem + stage * STAGE + (wave_s * XB + (i & ~3)) * BLK), 16,
-                                                 static_cast<int>(x_off[i]), kt * (BK * 2), (i & 3) * BLK, 0);
+                                                 static_cast<int>(x_off[i]), (kbase + kt) * (BK * 2), (i & 3) * BLK, 0);
     };
     auto gw = [&](auto ic, int kt, int stage) {
         constexpr int i = decltype(ic)::value;
         const bool up = MODE == MODE_SWIGLU && wave_s >= NW / 2;  // wavefronts 2 and 3 fetch the up rows
         __builtin_amdgcn_raw_ptr_buffer_load_lds(up ? w2_rsrc : w_rsrc, (lds_void *)(smem + stage * STAGE + XREG + (wave_s * WB + (i & ~3)) * BLK), 16,
-                                                 static_cast<int>(w_off[i]), kt * (BK * 2), (i & 3) * BLK, 0);
+                                                 static_cast<int>(w_off[i]), (kbase + kt) * (BK * 2), (i & 3) * BLK, 0);
     };
 #define IC(n) std::integral_constant<int, n>{}
 
@@ -727,20 +734,47 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         xq[0][0] = lds_read16<0>(xa); xq[0][1] = lds_read16<1 * T16>(xa); xq[0][2] = lds_read16<2 * T16>(xa); xq[0][3] = lds_read16<3 * T16>(xa);
         xq[0][4] = lds_read16<4 * T16>(xa); xq[0][5] = lds_read16<5 * T16>(xa); xq[0][6] = lds_read16<6 * T16>(xa); xq[0][7] = lds_read16<7 * T16>(xa);
     }
-    for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    for (int unit = blockIdx.x; unit < total_units; unit += SPLIT ? total_units : static_cast<int>(gridDim.x)) {
         int tile_m, tile_n;
+        const int tile = SPLIT ? unit % total_tiles : unit;
+        const int split = SPLIT ? unit / total_tiles : 0;
+        const int KT = SPLIT ? min(p.kt_per_split, KT_ALL - split * p.kt_per_split) : KT_ALL;
+        const int last = KT - 1;
         tile_of_block(tile, total_tiles, p.tiles_m, p.tiles_n, tile_m, tile_n);
 #pragma unroll
         for (int a = 0; a < 8; ++a)
 #pragma unroll
             for (int b = 0; b < 8; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int kt = 0; kt + 2 < KT; ++kt) T4_KTILE(kt + 2);
-        const bool more = tile + static_cast<int>(gridDim.x) < total_tiles;
-        if (more) set_load_tile(tile + gridDim.x);
+        const bool more = !SPLIT && unit + static_cast<int>(gridDim.x) < total_units;  // split: one unit per block
+        if (more) set_load_tile(unit + gridDim.x);
         // without a next tile the last K tile is fetched again, into stages nobody reads any more
         const int k0 = more ? 0 : last, k1 = more ? 1 : last;
         T4_KTILE(k0);
         T4_KTILE(k1);
+        if constexpr (SPLIT) {
+            // the wavefront's sums are tile (2 tile_m + wm, 2 tile_n + wn) of the 128 x 128 tiling; partial tile
+            // [w row][x row]: a lane's 4 values are 4 w rows of one x row, 16 lanes cover 16 consecutive x rows
+            const int tm128 = (p.M + 127) / 128, tn128 = (p.N + BN_OUT / 2 - 1) / (BN_OUT / 2);
+            int split_now = split;
+            asm volatile("" : "+s"(split_now));  // keeps the address arithmetic below out of the K loop's registers
+            const int m128 = tile_m * 2 + wm, n128 = tile_n * 2 + wn;
+            if (m128 < tm128 && n128 < tn128) {
+                float *ws = p.ws + (static_cast<int64_t>(split_now) * tm128 * tn128 + m128 * tn128 + n128) * (128 * 128) + lq * 4 * 128 + l16;
+#pragma unroll
+                for (int b = 0; b < 8; ++b) {
+                    typedef __attribute__((address_space(1))) float global_float;
+                    global_float *wsb = (global_float *)(ws + b * 16 * 128);
+                    asm volatile("" : "+v"(wsb));  // one address per w tile, the rest are store offsets
+#pragma unroll
+                    for (int a = 0; a < 8; ++a)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)  // stored from the accumulator registers, no copies
+                            asm volatile("global_store_dword %0, %1, off offset:%2" ::"v"(wsb), "a"(acc[a][b][i]), "n"((i * 128 + a * 16) * 4) : "memory");
+                }
+            }
+            continue;
+        }
         // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up
         const int m_wave = tile_m * BM + wm * 128;
         const int n_wave = tile_n * BN_OUT + (MODE == MODE_SWIGLU ? wn * 64 : wn * 128);
@@ -1098,37 +1132,6 @@ int launch_gemm(GemmParams p, hipStream_t s) {
     return TPAMD_OK;
 }
 
-template <int DT, int MODE>
-int launch_direct(GemmParams p, int cus, hipStream_t s) {
-    constexpr int LDS = 2 * 64 * 1152;
-    const char *w4 = getenv("TPAMD_GEMM_W4");
-#ifndef TPAMD_W4_DEFAULT
-#define TPAMD_W4_DEFAULT 1
-#endif
-    const bool four = (w4 != nullptr ? atoi(w4) != 0 : TPAMD_W4_DEFAULT != 0) && p.K >= 128;
-    auto kern = four ? gemm_direct4_kernel<DT, MODE> : gemm_direct_kernel<DT, MODE>;
-    static thread_local int configured_dev = -1;
-    int dev = 0;
-    TPAMD_HIP(hipGetDevice(&dev));
-    if (configured_dev != dev) {
-        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct_kernel<DT, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct4_kernel<DT, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-        configured_dev = dev;
-    }
-    p.tiles_m = (p.M + 255) / 256;
-    constexpr int BN_OUT = MODE == MODE_SWIGLU ? 128 : 256;
-    p.tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
-    const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-    TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
-    // one block per CU at most (a block needs most of a CU's LDS anyway); a multiple of 8 when blocks take several
-    // tiles, so that a block's tiles all belong to one XCD's share
-    int64_t blocks = tiles;
-    if (tiles > cus) blocks = cus >= 8 ? (cus / 8) * 8 : cus;
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(four ? 256 : 512), LDS, s, p);
-    TPAMD_HIP(hipGetLastError());
-    return TPAMD_OK;
-}
-
 }  // namespace
 
 // Split-K scratch: one buffer per device, allocated at first use with room for any split this file chooses, kept
@@ -1159,6 +1162,69 @@ int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, voi
     *out = ptr;
     return TPAMD_OK;
 }
+
+namespace {
+
+template <int DT, int MODE>
+int launch_direct(GemmParams p, int cus, int splits, hipStream_t s) {
+    constexpr int LDS = 2 * 64 * 1152;
+    const char *w4 = getenv("TPAMD_GEMM_W4");
+#ifndef TPAMD_W4_DEFAULT
+#define TPAMD_W4_DEFAULT 1
+#endif
+    const bool four = (w4 != nullptr ? atoi(w4) != 0 : TPAMD_W4_DEFAULT != 0) && p.K >= 128;
+    auto kern = four ? gemm_direct4_kernel<DT, MODE, false> : gemm_direct_kernel<DT, MODE>;
+    static thread_local int configured_dev = -1;
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct_kernel<DT, MODE>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct4_kernel<DT, MODE, false>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct4_kernel<DT, MODE, true>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        configured_dev = dev;
+    }
+    p.tiles_m = (p.M + 255) / 256;
+    constexpr int BN_OUT = MODE == MODE_SWIGLU ? 128 : 256;
+    p.tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+    const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
+    // one block per CU at most (a block needs most of a CU's LDS anyway); a multiple of 8 when blocks take several
+    // tiles, so that a block's tiles all belong to one XCD's share
+    int64_t blocks = tiles;
+    if (tiles > cus) blocks = cus >= 8 ? (cus / 8) * 8 : cus;
+    // K split over `splits` units per tile (all units in one round): every split gets at least 2 K tiles
+    const int KT = p.K / 64;
+    if (four && splits > 1 && KT >= 4) {
+        p.kt_per_split = (KT + splits - 1) / splits;
+        if (p.kt_per_split < 2) p.kt_per_split = 2;
+        while (KT % p.kt_per_split == 1) ++p.kt_per_split;  // the last split would be a single K tile
+        p.splits = (KT + p.kt_per_split - 1) / p.kt_per_split;
+        if (p.splits > 1 && tiles * p.splits <= cus) {
+            GemmParams f = p;  // the finishing pass sees the 128 x 128 tiling
+            f.tiles_m = (p.M + 127) / 128;
+            f.tiles_n = (p.N + BN_OUT / 2 - 1) / (BN_OUT / 2);
+            const int64_t tiles128 = static_cast<int64_t>(f.tiles_m) * f.tiles_n;
+            const size_t ws_bytes = static_cast<size_t>(p.splits) * tiles128 * 128 * 128 * sizeof(float);
+            std::lock_guard<std::mutex> hold(splitk_mutex());
+            void *ws = nullptr;
+            const int rc = splitk_scratch(dev, s, ws_bytes, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
+            if (rc != TPAMD_OK) return rc;
+            if (ws != nullptr) {
+                p.ws = f.ws = static_cast<float *>(ws);
+                hipLaunchKernelGGL((gemm_direct4_kernel<DT, MODE, true>), dim3(static_cast<unsigned>(tiles * p.splits)), dim3(256), LDS, s, p);
+                TPAMD_HIP(hipGetLastError());
+                hipLaunchKernelGGL((splitk_finish_kernel<DT, MODE>), dim3(MODE == MODE_SWIGLU ? 8 : 16, static_cast<unsigned>(tiles128)), dim3(256), 0, s, f, p.splits);
+                TPAMD_HIP(hipGetLastError());
+                return TPAMD_OK;
+            }
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(four ? 256 : 512), LDS, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+}  // namespace
 
 template <int DT, int MODE, int NS, bool SPLIT>
 int configure128(int dev) {
@@ -1251,13 +1317,24 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     const int64_t small_tiles = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128));
     const int KT = static_cast<int>(p.K / 64);
     const int64_t full_rounds = big_tiles / cus, last_round = big_tiles % cus;
-    const double t256 = 8.0 + KT * (full_rounds * 1.45 + (last_round == 0 ? 0.0 : last_round * 4 <= 3ll * cus ? 1.3 : 1.45));
+    double t256 = 8.0 + KT * (full_rounds * 1.45 + (last_round == 0 ? 0.0 : last_round * 4 <= 3ll * cus ? 1.3 : 1.45));
+    // ... or split over K while all units still fit one round; the partial tiles cost 3 us + 0.3 us per MB (more than
+    // with the small tiles: all blocks finish together, so nothing overlaps the writes and the finishing pass)
+    int splits256 = 1;
+    for (int sp = 2; sp <= 8 && big_tiles * sp <= cus; ++sp) {
+        const int kt = (KT + sp - 1) / sp;
+        if (kt < 4) break;
+        const int64_t units = big_tiles * sp;
+        const double t = 8.0 + kt * (units * 4 <= 3ll * cus ? 1.3 : 1.45) + 3.0 + units * 0.262144 * 0.3;
+        if (t < t256) { t256 = t; splits256 = sp; }
+    }
+    if (const char *e = getenv("TPAMD_GEMM_SPLITK256")) splits256 = atoi(e);
     int unused_splits = 1;
     const double t128 = estimate128(small_tiles, KT, cus, &unused_splits);
     const char *force = getenv("TPAMD_GEMM_TILE");
     const bool big = force ? atoi(force) == 256 : (t256 < t128 || small_tiles >= 65536);
     if (direct_ok) {
-        if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, s) : launch_direct<DT, MODE_LINEAR>(p, cus, s);
+        if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, splits256, s) : launch_direct<DT, MODE_LINEAR>(p, cus, splits256, s);
         return swiglu ? launch_direct128<DT, MODE_SWIGLU>(p, cus, s) : launch_direct128<DT, MODE_LINEAR>(p, cus, s);
     }
     if (big) return swiglu ? launch_gemm<DT, MODE_SWIGLU, 256, 256, 2, 4>(p, s) : launch_gemm<DT, MODE_LINEAR, 256, 256, 2, 4>(p, s);

@@ -209,8 +209,8 @@ def test_mid_sized_linear_inside_a_hip_graph():
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (513, 260, 192), (700, 1028, 320), (256, 256, 64), (1030, 772, 1088)])
 @pytest.mark.parametrize("waves", [4, 8])
 def test_256_tiles_on_ragged_shapes(dtype, M, N, K, waves, monkeypatch):
-    """The 256 x 256 tiling (forced through the library's debugging knobs; by default it is taken from about 200
-    tiles on) with 4 and with 8 wavefronts per block: two-tile K (the pipeline's minimum), tile rows past M, tile
+    """The 256 x 256 tiling (forced through the library's debugging knobs; by default it is taken when a cost model
+    predicts it to be faster) with 4 and with 8 wavefronts per block: two-tile K (the pipeline's minimum), tile rows past M, tile
     columns past N, bias and GELU, the gated pair, and a strided x. K = 64 is always served by the 8-wavefront
     kernel. Blocks that walk through several tiles are covered by the next test and by the full-shape tests."""
     monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
@@ -241,3 +241,34 @@ def test_both_256_tile_kernels_agree_bit_for_bit(monkeypatch):
     assert torch.equal(four, eight)
     check_half(four[:, :512], F.linear(x.float().cpu(), w[:512].float().cpu()), K)
     check_half(four[:, -512:], F.linear(x.float().cpu(), w[-512:].float().cpu()), K)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,splits", [(300, 520, 256, 2), (513, 260, 320, 2), (700, 1028, 448, 3), (256, 256, 576, 4), (1030, 772, 1088, 8), (130, 8, 704, 5)])
+def test_256_tiles_split_over_k(dtype, M, N, K, splits, monkeypatch):
+    """The 4-wavefront 256 x 256 kernel with K split over several blocks per tile (forced; by default the cost model
+    decides): splits of unequal length, the shortest allowed (2 K tiles), a last split that would be a single K tile
+    (K = 448 = 7 tiles in 3 splits: the library lengthens the splits instead), an odd number of 128 x 128 partial
+    tiles along M and N, bias and GELU applied by the finishing pass, and the gated pair."""
+    monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
+    monkeypatch.setenv("TPAMD_GEMM_SPLITK256", str(splits))
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
+    check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
+    w2 = rnd((N, K), 5, 0.02, dtype)
+    h = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    # the unsplit launch adds the same products in another order
+    monkeypatch.setenv("TPAMD_GEMM_SPLITK256", "1")
+    unsplit = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
+    torch.testing.assert_close(got.float(), unsplit.float(), rtol=RTOL_HALF, atol=RTOL_HALF * 0.02 * math.sqrt(K))
+
+
+def test_mid_sized_shapes_choose_a_correct_path():
+    """Shapes on which the dispatch takes the 256 x 256 tiling with K split (few tiles, long K) and without."""
+    for M, N, K in [(1024, 4608, 8192), (768, 8192, 8192), (1024, 5504, 4096)]:
+        x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
+        got = _native.linear(x, w)
+        check_half(got[:, :256], F.linear(x.float().cpu(), w[:256].float().cpu()), K)
+        check_half(got[-300:, -300:], F.linear(x[-300:].float().cpu(), w[-300:].float().cpu()), K)
