@@ -655,6 +655,10 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
     f32x4 acc[8][8];
     u32x4 xq[2][8], wq[2][8];
     const uint32_t smem_base = lds_addr_of(smem);
+    // epilogue staging behind the two stages: 16 rows x 64 packed outputs per wavefront, rows 144 bytes apart
+    constexpr int EP_PITCH = 144;
+    char *ep_slab = smem + 2 * STAGE + wave * (16 * EP_PITCH);
+    const bool wide_stores = (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && p.ldy % 8 == 0;
 
 #define T4_SB __builtin_amdgcn_sched_barrier(0)
 #define T4_MFMA(buf, a, b) acc[a][b] = mfma16<DT>(wq[buf][b], xq[buf][a], acc[a][b])
@@ -775,27 +779,85 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
             }
             continue;
         }
-        // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up
+        // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up. A lane holds 4 consecutive columns of
+        // one row per accumulator tile; stored like that an instruction would write 32-byte pieces of 16 rows. The
+        // packed results of 16 rows x 64 columns go through the wavefront's staging slab instead and leave as whole
+        // 128-byte lines, 8 rows per store instruction.
         const int m_wave = tile_m * BM + wm * 128;
         const int n_wave = tile_n * BN_OUT + (MODE == MODE_SWIGLU ? wn * 64 : wn * 128);
+        auto epilogue = [&](auto gelu_c) {
+            constexpr bool GELU = decltype(gelu_c)::value;
+            constexpr int GROUPS = MODE == MODE_SWIGLU ? 1 : 2;  // 64-column groups per wavefront
+            uint2 braw[GROUPS * 4];
+            if constexpr (MODE == MODE_LINEAR) {
 #pragma unroll
-        for (int a = 0; a < 8; ++a) {
-            const int m = m_wave + a * 16 + l16;
-            if (m >= p.M) continue;
-            char *yrow = p.y + static_cast<int64_t>(m) * p.ldy * 2;
-#pragma unroll
-            for (int b = 0; b < (MODE == MODE_SWIGLU ? 4 : 8); ++b) {
-                const int n = n_wave + b * 16 + lq * 4;
-                if (n >= p.N) continue;
-                float gsum[4], usum[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    gsum[j] = acc[a][b][j];
-                    usum[j] = MODE == MODE_SWIGLU ? acc[a][(b + 4) & 7][j] : 0.f;
+                for (int b = 0; b < 8; ++b) {
+                    const int n = n_wave + b * 16 + lq * 4;
+                    braw[b] = p.bias != nullptr && n < p.N ? *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2) : make_uint2(0, 0);
                 }
-                *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = finish4<DT, MODE>(p, gsum, usum, n);
             }
-        }
+            const int rd_row = lane >> 3, rd_col = lane & 7;
+#pragma unroll
+            for (int a = 0; a < 8; ++a) {
+#pragma unroll
+                for (int gq = 0; gq < GROUPS; ++gq) {
+#pragma unroll
+                    for (int bb = 0; bb < 4; ++bb) {
+                        const int b = gq * 4 + bb;
+                        uint2 o;
+                        if constexpr (MODE == MODE_SWIGLU) {
+                            float gsum[4], usum[4];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                gsum[j] = acc[a][b][j];
+                                usum[j] = acc[a][b + 4][j];
+                            }
+                            o = finish4<DT, MODE>(p, gsum, usum, 0);
+                        } else {
+                            float v[4];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) v[j] = acc[a][b][j];
+                            v[0] += lo_half_to_f32<DT>(braw[b].x); v[1] += hi_half_to_f32<DT>(braw[b].x);
+                            v[2] += lo_half_to_f32<DT>(braw[b].y); v[3] += hi_half_to_f32<DT>(braw[b].y);
+                            if constexpr (GELU) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
+                            }
+                            o.x = pack2_half<DT>(v[0], v[1]);
+                            o.y = pack2_half<DT>(v[2], v[3]);
+                        }
+                        *reinterpret_cast<uint2 *>(ep_slab + l16 * EP_PITCH + bb * 32 + lq * 8) = o;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int row = h * 8 + rd_row;
+                        const uint4 v = *reinterpret_cast<const uint4 *>(ep_slab + row * EP_PITCH + rd_col * 16);
+                        const int m = m_wave + a * 16 + row;
+                        const int n = n_wave + gq * 64 + rd_col * 8;
+#ifdef T4_ABL_NOSTORE
+                        if (p.act != 12345) continue;
+#endif
+                        if (m >= p.M || n >= p.N) continue;
+                        char *dst = p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2;
+                        if (n + 8 <= p.N) {
+                            if (wide_stores) *reinterpret_cast<uint4 *>(dst) = v;
+                            else {
+                                *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
+                                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(v.z, v.w);
+                            }
+                        } else {
+                            *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);  // N is a multiple of 4
+                        }
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                    asm volatile("" ::: "memory");
+                }
+            }
+        };
+        if (MODE == MODE_LINEAR && p.act == TPAMD_ACT_GELU) epilogue(std::true_type{});
+        else epilogue(std::false_type{});
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no global->LDS load in flight when the wavefront leaves
 #undef T4_SB
@@ -1167,7 +1229,7 @@ namespace {
 
 template <int DT, int MODE>
 int launch_direct(GemmParams p, int cus, int splits, hipStream_t s) {
-    constexpr int LDS = 2 * 64 * 1152;
+    constexpr int LDS = 2 * 64 * 1152 + 4 * 16 * 144;  // two stages + the 4-wavefront kernel's epilogue slabs
     const char *w4 = getenv("TPAMD_GEMM_W4");
 #ifndef TPAMD_W4_DEFAULT
 #define TPAMD_W4_DEFAULT 1
