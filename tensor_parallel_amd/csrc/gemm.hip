@@ -354,6 +354,89 @@ __device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[TMX
     }
 }
 
+// Epilogue of the 4-wavefront kernels. A lane holds 4 consecutive columns of one row per accumulator tile; stored like
+// that, an instruction would write 32-byte pieces of 16 rows. Instead the packed results of 16 rows x (16 * GB)
+// columns go through a wavefront-private LDS slab (16 rows, EP_PITCH bytes apart) and leave as 16 bytes per lane:
+// whole 128-byte lines, 8 rows per store instruction, when GB = 4.
+// acc[a][b]: a = 16-row tile of x, b = 16-row tile of w. The wavefront's columns are GROUPS runs of 16 * GB; gated pair:
+// tile b holds gate sums and tile b + UP the up sums of the same columns. wide: 16-byte stores are aligned.
+constexpr int EP_PITCH = 144;
+template <int DT, int MODE, bool GELU, int TMX, int NBT, int GROUPS, int GB, int UP>
+__device__ __forceinline__ void staged_epilogue(const GemmParams &p, f32x4 (&acc)[TMX][NBT], char *slab, int m_wave, int n_wave,
+                                                int lane, bool wide) {
+    static_assert(GB == 4 || GB == 2, "64 or 32 columns per slab");
+    const int l16 = lane & 15, lq = lane >> 4;
+    uint2 braw[GROUPS * GB];
+    if constexpr (MODE == MODE_LINEAR) {
+#pragma unroll
+        for (int b = 0; b < GROUPS * GB; ++b) {
+            const int n = n_wave + b * 16 + lq * 4;
+            braw[b] = p.bias != nullptr && n < p.N ? *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2) : make_uint2(0, 0);
+        }
+    }
+    constexpr int LANES_PER_ROW = GB * 2;            // 16 bytes per lane
+    constexpr int ROWS_PER_READ = 64 / LANES_PER_ROW;
+    const int rd_row = lane / LANES_PER_ROW, rd_col = lane % LANES_PER_ROW;
+#pragma unroll
+    for (int a = 0; a < TMX; ++a) {
+#pragma unroll
+        for (int gq = 0; gq < GROUPS; ++gq) {
+#pragma unroll
+            for (int bb = 0; bb < GB; ++bb) {
+                const int b = gq * GB + bb;
+                uint2 o;
+                if constexpr (MODE == MODE_SWIGLU) {
+                    float gsum[4], usum[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        gsum[j] = acc[a][b][j];
+                        usum[j] = acc[a][b + UP][j];
+                    }
+                    o = finish4<DT, MODE>(p, gsum, usum, 0);
+                } else {
+                    float v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = acc[a][b][j];
+                    v[0] += lo_half_to_f32<DT>(braw[b].x); v[1] += hi_half_to_f32<DT>(braw[b].x);
+                    v[2] += lo_half_to_f32<DT>(braw[b].y); v[3] += hi_half_to_f32<DT>(braw[b].y);
+                    if constexpr (GELU) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
+                    }
+                    o.x = pack2_half<DT>(v[0], v[1]);
+                    o.y = pack2_half<DT>(v[2], v[3]);
+                }
+                *reinterpret_cast<uint2 *>(slab + l16 * EP_PITCH + bb * 32 + lq * 8) = o;
+            }
+            __builtin_amdgcn_wave_barrier();
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int h = 0; h < 16 / ROWS_PER_READ; ++h) {
+                const int row = h * ROWS_PER_READ + rd_row;
+                const uint4 v = *reinterpret_cast<const uint4 *>(slab + row * EP_PITCH + rd_col * 16);
+                const int m = m_wave + a * 16 + row;
+                const int n = n_wave + gq * (16 * GB) + rd_col * 8;
+#ifdef T4_ABL_NOSTORE
+                if (p.act != 12345) continue;
+#endif
+                if (m >= p.M || n >= p.N) continue;
+                char *dst = p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2;
+                if (n + 8 <= p.N) {
+                    if (wide) *reinterpret_cast<uint4 *>(dst) = v;
+                    else {
+                        *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
+                        *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(v.z, v.w);
+                    }
+                } else {
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);  // N is a multiple of 4
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            asm volatile("" ::: "memory");
+        }
+    }
+}
+
 // gemm_direct_kernel: 256 x 256 x 64 tiles, 8 wavefronts (2 x 4, 128 x-rows by 64 w-rows each), 2 LDS stages.
 //
 // MFMA shape: v_mfma_f32_16x16x32. Under the chip's power limit it sustains about 14% more flops than the
@@ -655,8 +738,7 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
     f32x4 acc[8][8];
     u32x4 xq[2][8], wq[2][8];
     const uint32_t smem_base = lds_addr_of(smem);
-    // epilogue staging behind the two stages: 16 rows x 64 packed outputs per wavefront, rows 144 bytes apart
-    constexpr int EP_PITCH = 144;
+    // epilogue staging behind the two stages: 16 rows x 64 packed outputs per wavefront
     char *ep_slab = smem + 2 * STAGE + wave * (16 * EP_PITCH);
     const bool wide_stores = (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && p.ldy % 8 == 0;
 
@@ -726,9 +808,10 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
     gx(IC(5), kt, stage); gx(IC(6), kt, stage); gx(IC(7), kt, stage); gw(IC(0), kt, stage); gw(IC(1), kt, stage);   \
     gw(IC(2), kt, stage); gw(IC(3), kt, stage); gw(IC(4), kt, stage); gw(IC(5), kt, stage); gw(IC(6), kt, stage);   \
     gw(IC(7), kt, stage)
+    // both K tiles are requested at once; loads return in order, so the first 16 being back means K tile 0 is there
     T4_ALL_LOADS(0, 0);
-    drain_and_barrier();
     T4_ALL_LOADS(1, 1);
+    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
 #undef T4_ALL_LOADS
     {
         const uint32_t xa = smem_base + x_rd0 + kk_off[0];
@@ -779,85 +862,15 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
             }
             continue;
         }
-        // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up. A lane holds 4 consecutive columns of
-        // one row per accumulator tile; stored like that an instruction would write 32-byte pieces of 16 rows. The
-        // packed results of 16 rows x 64 columns go through the wavefront's staging slab instead and leave as whole
-        // 128-byte lines, 8 rows per store instruction.
+        // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up
         const int m_wave = tile_m * BM + wm * 128;
         const int n_wave = tile_n * BN_OUT + (MODE == MODE_SWIGLU ? wn * 64 : wn * 128);
-        auto epilogue = [&](auto gelu_c) {
-            constexpr bool GELU = decltype(gelu_c)::value;
-            constexpr int GROUPS = MODE == MODE_SWIGLU ? 1 : 2;  // 64-column groups per wavefront
-            uint2 braw[GROUPS * 4];
-            if constexpr (MODE == MODE_LINEAR) {
-#pragma unroll
-                for (int b = 0; b < 8; ++b) {
-                    const int n = n_wave + b * 16 + lq * 4;
-                    braw[b] = p.bias != nullptr && n < p.N ? *reinterpret_cast<const uint2 *>(p.bias + static_cast<int64_t>(n) * 2) : make_uint2(0, 0);
-                }
-            }
-            const int rd_row = lane >> 3, rd_col = lane & 7;
-#pragma unroll
-            for (int a = 0; a < 8; ++a) {
-#pragma unroll
-                for (int gq = 0; gq < GROUPS; ++gq) {
-#pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) {
-                        const int b = gq * 4 + bb;
-                        uint2 o;
-                        if constexpr (MODE == MODE_SWIGLU) {
-                            float gsum[4], usum[4];
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                gsum[j] = acc[a][b][j];
-                                usum[j] = acc[a][b + 4][j];
-                            }
-                            o = finish4<DT, MODE>(p, gsum, usum, 0);
-                        } else {
-                            float v[4];
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) v[j] = acc[a][b][j];
-                            v[0] += lo_half_to_f32<DT>(braw[b].x); v[1] += hi_half_to_f32<DT>(braw[b].x);
-                            v[2] += lo_half_to_f32<DT>(braw[b].y); v[3] += hi_half_to_f32<DT>(braw[b].y);
-                            if constexpr (GELU) {
-#pragma unroll
-                                for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
-                            }
-                            o.x = pack2_half<DT>(v[0], v[1]);
-                            o.y = pack2_half<DT>(v[2], v[3]);
-                        }
-                        *reinterpret_cast<uint2 *>(ep_slab + l16 * EP_PITCH + bb * 32 + lq * 8) = o;
-                    }
-                    __builtin_amdgcn_wave_barrier();
-                    asm volatile("" ::: "memory");
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        const int row = h * 8 + rd_row;
-                        const uint4 v = *reinterpret_cast<const uint4 *>(ep_slab + row * EP_PITCH + rd_col * 16);
-                        const int m = m_wave + a * 16 + row;
-                        const int n = n_wave + gq * 64 + rd_col * 8;
-#ifdef T4_ABL_NOSTORE
-                        if (p.act != 12345) continue;
-#endif
-                        if (m >= p.M || n >= p.N) continue;
-                        char *dst = p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2;
-                        if (n + 8 <= p.N) {
-                            if (wide_stores) *reinterpret_cast<uint4 *>(dst) = v;
-                            else {
-                                *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
-                                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(v.z, v.w);
-                            }
-                        } else {
-                            *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);  // N is a multiple of 4
-                        }
-                    }
-                    __builtin_amdgcn_wave_barrier();
-                    asm volatile("" ::: "memory");
-                }
-            }
-        };
-        if (MODE == MODE_LINEAR && p.act == TPAMD_ACT_GELU) epilogue(std::true_type{});
-        else epilogue(std::false_type{});
+        if constexpr (MODE == MODE_SWIGLU) {
+            staged_epilogue<DT, MODE, false, 8, 8, 1, 4, 4>(p, acc, ep_slab, m_wave, n_wave, lane, wide_stores);
+        } else {
+            if (p.act == TPAMD_ACT_GELU) staged_epilogue<DT, MODE, true, 8, 8, 2, 4, 0>(p, acc, ep_slab, m_wave, n_wave, lane, wide_stores);
+            else staged_epilogue<DT, MODE, false, 8, 8, 2, 4, 0>(p, acc, ep_slab, m_wave, n_wave, lane, wide_stores);
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no global->LDS load in flight when the wavefront leaves
 #undef T4_SB
@@ -1064,7 +1077,17 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
                 for (int i = 0; i < 4; ++i) ws[(wr + i) * BM + xr] = acc[a][b][i];
             }
     } else {
-        epilogue16<DT, MODE, 4>(p, acc, m0 + wm * 64, n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64), l16, lq);
+        // the stages are free once every wavefront has read its last fragments: a slab per wavefront at their start
+        __syncthreads();
+        char *slab = smem + wave * (16 * EP_PITCH);
+        const bool wide = (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && p.ldy % 8 == 0;
+        const int m_wave = m0 + wm * 64, n_wave = n0 + (MODE == MODE_SWIGLU ? wn * 32 : wn * 64);
+        if constexpr (MODE == MODE_SWIGLU) {
+            staged_epilogue<DT, MODE, false, 4, 4, 1, 2, 2>(p, acc, slab, m_wave, n_wave, lane, wide);
+        } else {
+            if (p.act == TPAMD_ACT_GELU) staged_epilogue<DT, MODE, true, 4, 4, 1, 4, 0>(p, acc, slab, m_wave, n_wave, lane, wide);
+            else staged_epilogue<DT, MODE, false, 4, 4, 1, 4, 0>(p, acc, slab, m_wave, n_wave, lane, wide);
+        }
     }
 }
 
