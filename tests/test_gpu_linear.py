@@ -272,3 +272,33 @@ def test_mid_sized_shapes_choose_a_correct_path():
         got = _native.linear(x, w)
         check_half(got[:, :256], F.linear(x.float().cpu(), w[:256].float().cpu()), K)
         check_half(got[-300:, -300:], F.linear(x[-300:].float().cpu(), w[-300:].float().cpu()), K)
+
+
+@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("N,ldy,shift", [(260, 264, 0), (260, 264, 4), (256, 260, 0), (520, 528, 8), (132, 136, 4)])
+def test_strided_and_8_byte_aligned_outputs_through_the_c_abi(tile, N, ldy, shift, monkeypatch):
+    """y with a row pitch above N and a base that is 8- but not 16-byte aligned (shift = 4 elements): the epilogues
+    choose between 16- and 8-byte stores by the alignment of y and its pitch, and a row's last 4 columns (N % 8 == 4)
+    are always an 8-byte store. The columns between N and the pitch must stay untouched."""
+    import ctypes
+
+    monkeypatch.setenv("TPAMD_GEMM_TILE", tile)
+    M, K = 300, 256
+    x, w, b = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N,), 2, 0.1).to(DEV)
+    w2 = rnd((N, K), 5, 0.02).to(DEV)
+    buf = torch.full((M * ldy + 16,), 7.0, dtype=torch.bfloat16, device=DEV)
+    y = buf[shift: shift + M * ldy].view(M, ldy)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(DEV).cuda_stream)
+    rc = _native.lib().tpamd_linear(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), M, N, K, K, K, ldy,
+                                    _native.dtype_code(torch.bfloat16), _native.ACT_NONE, stream)
+    assert rc == 0
+    check_half(y[:, :N], F.linear(x.float().cpu(), w.float().cpu(), b.float().cpu()), K)
+    assert bool((y[:, N:] == 7.0).all()) and bool((buf[:shift] == 7.0).all()) and bool((buf[shift + M * ldy:] == 7.0).all())
+    buf.fill_(7.0)
+    rc = _native.lib().tpamd_swiglu_up(x.data_ptr(), w.data_ptr(), w2.data_ptr(), y.data_ptr(), M, N, K, K, K, ldy,
+                                       _native.dtype_code(torch.bfloat16), stream)
+    assert rc == 0
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    want = ofw.gated_mlp_hidden(x.float().cpu(), w.float().cpu(), w2.float().cpu())
+    torch.testing.assert_close(y[:, :N].float().cpu(), want, rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    assert bool((y[:, N:] == 7.0).all())
