@@ -1326,9 +1326,10 @@ int configure128(int dev) {
 }
 
 // Predicted time (microseconds) of the 128 x 128 tiling and the K split that gives it, from a small cost model
-// fitted on this part: a block that has its CU to itself takes 0.8 per K tile, two blocks sharing a CU 1.0 each
-// (the pace of the CU's global->LDS path), blocks beyond two per CU wait for the next round; the partial tiles cost
-// 3 + 0.18 per MB (written, read back and finished by a second launch).
+// fitted (least squares over 290 timings of 48 mid-sized shapes) on this part: a block that has its CU to itself takes
+// 0.82 per K tile, two blocks sharing a CU 0.98 each (the pace of the CU's global->LDS path), 0.92 when blocks queue
+// for several rounds of two per CU; the partial tiles cost 4.6 + 0.39 per MB (written, read back and finished by a
+// second launch).
 inline double estimate128(int64_t tiles, int KT, int cus, int *splits) {
     double best = 1e30;
     *splits = 1;
@@ -1337,7 +1338,8 @@ inline double estimate128(int64_t tiles, int KT, int cus, int *splits) {
         if (sp > 1 && (kt < 4 || tiles * sp > 4ll * cus)) break;  // too little K per split / more than the scratch buffer holds
         const double units = static_cast<double>(tiles) * sp;
         const double rounds = units <= cus ? 1.0 : static_cast<double>((static_cast<int64_t>(units) + 2 * cus - 1) / (2 * cus));
-        const double t = rounds * kt * (units <= cus ? 0.8 : 1.0) + (sp > 1 ? 3.0 + units * 0.065536 * 0.18 : 0.0);
+        const double per_kt = units <= cus ? 0.82 : units <= 2.0 * cus ? 0.98 : 0.92;
+        const double t = rounds * kt * per_kt + (sp > 1 ? 4.6 + units * 0.065536 * 0.39 : 0.0);
         if (t < best) { best = t; *splits = sp; }
     }
     return best;
@@ -1399,21 +1401,24 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     // the direct kernels address a tile with 32-bit byte offsets from the tile origin and step K in tiles of 64
     const bool direct_ok = p.K % 64 == 0 && p.K >= 64 && p.ldx < (1ll << 22) && p.ldw < (1ll << 22);
     // 256 x 256 tiles or 128 x 128 tiles (with K split): whichever the cost models predict to be faster. The 256 tiles
-    // run in rounds of one per CU; a K tile takes about 1.45 us in a full round (the part is power-limited then) and
-    // 1.3 us in a round that fills at most three quarters of the CUs; fill and epilogue add about 8 us.
+    // run in rounds of one per CU; fitted on the same timings, a K tile takes 1.47 us in a full round (the part is
+    // power-limited then), 1.2 us in a round that fills at most three quarters of the CUs and 1.3 us in between.
     const int64_t big_tiles = static_cast<int64_t>((p.M + 255) / 256) * ((p.N + (swiglu ? 127 : 255)) / (swiglu ? 128 : 256));
     const int64_t small_tiles = static_cast<int64_t>((p.M + 127) / 128) * ((p.N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128));
     const int KT = static_cast<int>(p.K / 64);
-    const int64_t full_rounds = big_tiles / cus, last_round = big_tiles % cus;
-    double t256 = 8.0 + KT * (full_rounds * 1.45 + (last_round == 0 ? 0.0 : last_round * 4 <= 3ll * cus ? 1.3 : 1.45));
-    // ... or split over K while all units still fit one round; the partial tiles cost 3 us + 0.3 us per MB (more than
+    auto rounds256 = [&](int64_t units, int kt) {
+        const int64_t full = units / cus, last = units % cus;
+        return kt * (full * 1.47 + (last == 0 ? 0.0 : last * 4 <= 3ll * cus ? 1.2 : 1.3));
+    };
+    double t256 = rounds256(big_tiles, KT);
+    // ... or split over K while all units still fit one round; the partial tiles cost 9 us + 0.33 us per MB (more than
     // with the small tiles: all blocks finish together, so nothing overlaps the writes and the finishing pass)
     int splits256 = 1;
     for (int sp = 2; sp <= 8 && big_tiles * sp <= cus; ++sp) {
         const int kt = (KT + sp - 1) / sp;
         if (kt < 4) break;
         const int64_t units = big_tiles * sp;
-        const double t = 8.0 + kt * (units * 4 <= 3ll * cus ? 1.3 : 1.45) + 3.0 + units * 0.262144 * 0.3;
+        const double t = rounds256(units, kt) + 9.0 + units * 0.262144 * 0.33;
         if (t < t256) { t256 = t; splits256 = sp; }
     }
     if (const char *e = getenv("TPAMD_GEMM_SPLITK256")) splits256 = atoi(e);
