@@ -40,7 +40,7 @@ struct GemmParams {
     int64_t ldx, ldw, ldy;  // elements
     int act;
     int tiles_m, tiles_n;
-    float *ws;          // split-K: partial tiles, [split][tile][128 w rows][128 x rows] fp32
+    float *ws;          // split-K: partial tiles, [split][tile][128 x rows][128 w rows] fp32
     int kt_per_split;   // split-K: K tiles (of 64) per split
     int splits;         // split-K of the 256 x 256 kernel: work units = tiles x splits
 };
@@ -841,23 +841,24 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         T4_KTILE(k1);
         if constexpr (SPLIT) {
             // the wavefront's sums are tile (2 tile_m + wm, 2 tile_n + wn) of the 128 x 128 tiling; partial tile
-            // [w row][x row]: a lane's 4 values are 4 w rows of one x row, 16 lanes cover 16 consecutive x rows
+            // [x row][w row]: a lane's 4 values are 4 consecutive w rows of one x row, one 16-byte store
             const int tm128 = (p.M + 127) / 128, tn128 = (p.N + BN_OUT / 2 - 1) / (BN_OUT / 2);
             int split_now = split;
             asm volatile("" : "+s"(split_now));  // keeps the address arithmetic below out of the K loop's registers
             const int m128 = tile_m * 2 + wm, n128 = tile_n * 2 + wn;
             if (m128 < tm128 && n128 < tn128) {
-                float *ws = p.ws + (static_cast<int64_t>(split_now) * tm128 * tn128 + m128 * tn128 + n128) * (128 * 128) + lq * 4 * 128 + l16;
+                float *ws = p.ws + (static_cast<int64_t>(split_now) * tm128 * tn128 + m128 * tn128 + n128) * (128 * 128) + l16 * 128 + lq * 4;
 #pragma unroll
-                for (int b = 0; b < 8; ++b) {
+                for (int a = 0; a < 8; ++a) {
                     typedef __attribute__((address_space(1))) float global_float;
-                    global_float *wsb = (global_float *)(ws + b * 16 * 128);
-                    asm volatile("" : "+v"(wsb));  // one address per w tile, the rest are store offsets
+                    global_float *wsa = (global_float *)(ws + a * 16 * 128);
+                    asm volatile("" : "+v"(wsa));  // one address per x tile, the rest are store offsets
 #pragma unroll
-                    for (int a = 0; a < 8; ++a)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)  // stored from the accumulator registers, no copies
-                            asm volatile("global_store_dword %0, %1, off offset:%2" ::"v"(wsb), "a"(acc[a][b][i]), "n"((i * 128 + a * 16) * 4) : "memory");
+                    for (int b = 0; b < 8; ++b)
+                        // Stored from accumulator registers. The no-ops are the wait states a store of more than 8
+                        // bytes needs before its data registers may be written again: the compiler does not see
+                        // into the asm statement and may reuse them in the very next instruction.
+                        asm volatile("global_store_dwordx4 %0, %1, off offset:%2\n\ts_nop 2" ::"v"(wsa), "a"(acc[a][b]), "n"(b * 64) : "memory");
                 }
             }
             continue;
@@ -1067,7 +1068,7 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
 #undef TPAMD_TILE_BARRIER
 
     if constexpr (SPLIT) {
-        // partial tile [w row][x row]: a lane's 4 values are 4 w rows of one x row; 16 lanes cover 16 consecutive x rows
+        // partial tile [x row][w row]: a lane's 4 values are 4 consecutive w rows of one x row, one 16-byte store
         const int tile = tile_m * p.tiles_n + tile_n;
         float *ws = p.ws + (static_cast<int64_t>(blockIdx.y) * p.tiles_m * p.tiles_n + tile) * (BM * BN);
 #pragma unroll
@@ -1076,8 +1077,7 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
             for (int b = 0; b < 4; ++b) {
                 const int wr = (MODE == MODE_SWIGLU ? (b >> 1) * 64 + wn * 32 + (b & 1) * 16 : wn * 64 + b * 16) + lq * 4;
                 const int xr = wm * 64 + a * 16 + l16;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) ws[(wr + i) * BM + xr] = acc[a][b][i];
+                *reinterpret_cast<f32x4 *>(ws + xr * BN + wr) = acc[a][b];
             }
     } else {
         // the stages are free once every wavefront has read its last fragments: a slab per wavefront at their start
@@ -1094,28 +1094,37 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
     }
 }
 
-// Sums the split-K partial tiles of gemm_direct128_kernel and applies the epilogue. One thread = one x row and 4
-// consecutive output columns; the 128 x rows of a tile are the contiguous axis of a partial tile, so a block of
-// 256 threads reads two runs of 512 contiguous bytes per w row and split. Grid: (column-group pairs, tiles).
+// Sums the split-K partial tiles of one tile of the 128 x 128 tiling in split order and applies the epilogue. A partial
+// tile is [128 x rows][128 w rows] fp32 (gated pair: w rows 0-63 are gate rows, 64-127 the up rows of the same 64
+// output columns): 32 (gated pair: 16) consecutive threads read one row as 16-byte pieces and write 8 bytes each of
+// one output row. Grid: (16 or 8 blocks of 256 threads per tile, tiles).
 template <int DT, int MODE>
 __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmParams p, int splits) {
+    constexpr int PER_ROW = MODE == MODE_SWIGLU ? 16 : 32;
     const int tile = blockIdx.y;
     const int tile_m = tile / p.tiles_n, tile_n = tile % p.tiles_n;
-    const int64_t ntiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-    const int xr = threadIdx.x & 127, grp = blockIdx.x * 2 + (threadIdx.x >> 7);
-    const int m = tile_m * 128 + xr;
-    const int n = tile_n * (MODE == MODE_SWIGLU ? 64 : 128) + grp * 4;
-    if (m >= p.M || n >= p.N) return;
-    float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < splits; ++sp) {
-        const float *ws = p.ws + (sp * ntiles + tile) * (128 * 128);
+    const int64_t split_stride = static_cast<int64_t>(p.tiles_m) * p.tiles_n * (128 * 128);
+    const float *tile0 = p.ws + static_cast<int64_t>(tile) * (128 * 128);
+    {
+        const int idx = blockIdx.x * 256 + threadIdx.x;
+        const int r = idx / PER_ROW, c4 = idx % PER_ROW;
+        const int m = tile_m * 128 + r;
+        const int n = tile_n * (MODE == MODE_SWIGLU ? 64 : 128) + c4 * 4;
+        if (m >= p.M || n >= p.N) return;
+        float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+        const float *src = tile0 + r * 128 + c4 * 4;
+        for (int sp = 0; sp < splits; ++sp) {
+            const f32x4 gv = *reinterpret_cast<const f32x4 *>(src + sp * split_stride);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            g[i] += ws[(grp * 4 + i) * 128 + xr];
-            if constexpr (MODE == MODE_SWIGLU) u[i] += ws[(64 + grp * 4 + i) * 128 + xr];
+            for (int i = 0; i < 4; ++i) g[i] += gv[i];
+            if constexpr (MODE == MODE_SWIGLU) {
+                const f32x4 uv = *reinterpret_cast<const f32x4 *>(src + sp * split_stride + 64);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) u[i] += uv[i];
+            }
         }
+        *reinterpret_cast<uint2 *>(p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2) = finish4<DT, MODE>(p, g, u, n);
     }
-    *reinterpret_cast<uint2 *>(p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2) = finish4<DT, MODE>(p, g, u, n);
 }
 
 // ---- any dtype, any alignment: LDS-tiled FMA kernel, 64x64 tile, 256 threads, 4x4 outputs per thread ---------
@@ -1355,7 +1364,6 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     constexpr int BN_OUT = MODE == MODE_SWIGLU ? 64 : 128;
     p.tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
     const int64_t tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-    TPAMD_REQUIRE(tiles < 65536 || tiles >= 2 * cus, "gemm: too many tiles");  // the finishing pass indexes tiles with blockIdx.y
     TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
     const int KT = p.K / 64;
     int splits = 1;
@@ -1425,7 +1433,7 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     int unused_splits = 1;
     const double t128 = estimate128(small_tiles, KT, cus, &unused_splits);
     const char *force = getenv("TPAMD_GEMM_TILE");
-    const bool big = force ? atoi(force) == 256 : (t256 < t128 || small_tiles >= 65536);
+    const bool big = force ? atoi(force) == 256 : t256 < t128;
     if (direct_ok) {
         if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, splits256, s) : launch_direct<DT, MODE_LINEAR>(p, cus, splits256, s);
         return swiglu ? launch_direct128<DT, MODE_SWIGLU>(p, cus, s) : launch_direct128<DT, MODE_LINEAR>(p, cus, s);
