@@ -222,7 +222,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     flops = 6.0 * 512 * D_MODEL * FFN_SHARD
     extra["prefill_m512"] = {"us_per_step": us, "tokens_per_s": 512 / us * 1e6, "TFLOPs": flops / us / 1e6,
                              "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS, "algorithmic_flops": flops,
-                             "step": "swiglu_up + down (128x128 tiles, K split)"}
+                             "step": "swiglu_up + down (tiling and K split chosen by the library: 256x256 / 2 and 128x128 / 4)"}
     for m in (1, 32):
         extra[f"w8_decode_m{m}"] = w8_decode(torch, _native, dev, m)
     extra["attention_falcon40b_shard"] = attention_extra(torch, _native, dev)
