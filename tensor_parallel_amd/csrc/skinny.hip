@@ -394,6 +394,141 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(SkinnyParams p) {
     }
 }
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): loop indices that stay compile-time constants
+template <int N, int J = 0, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (J < N) {
+        f(std::integral_constant<int, J>{});
+        static_for<N, J + 1>(f);
+    }
+}
+
+// ---- x-resident form of the weight-streaming kernel ------------------------------------------------------
+// When there are several 16-row weight tiles per CU, the block above re-reads its K slices of x for every tile, and
+// from 8 rows on those bytes weigh as much as the weights in what a CU can take in. Here a block stays on its CU and
+// walks a contiguous range of output columns (the N columns are split evenly over the blocks; the last tile of a
+// range is partly masked): wavefront w keeps the x fragments of its chunks w, w + 8, ... in registers for the whole
+// launch (NCH chunks: K <= NCH * 1024), and the weights of the next tile are requested chunk by chunk as soon as the
+// registers of the current tile's chunk are free, so a wavefront always has about NCH * 4 KiB of weights in flight.
+// Partial sums of the wavefronts meet in LDS once per tile (two buffers, one barrier per tile).
+// MODE SK_SWIGLU: the tile is 8 gate rows + the 8 up rows of the same 8 columns (16-bit weights only).
+template <int DT, int MODE, int NCH>
+__global__ __launch_bounds__(SK_THREADS) void skinny_resident_kernel(SkinnyParams p) {
+    constexpr int NW = SK_WAVES;
+    constexpr bool PAIR = MODE == SK_SWIGLU;
+    constexpr int COLS = PAIR ? 8 : 16;
+    constexpr int CHUNK_K = 128;                // K elements per chunk: 256 bytes of every row
+    constexpr int TROW = 272;                   // staged row pitch: 256 bytes + 16 pad
+    __shared__ float red[2][NW][4][64];
+    __shared__ __align__(16) char stage_all[NW][16 * TROW];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int crow = lane >> 3, cpiece = lane & 7;
+    char *stage = stage_all[wave];
+    const int st_wr = crow * TROW + cpiece * 16;   // + (i&1)*8*TROW + (i/2)*128
+    const int st_rd = lr * TROW + lg * 16;         // + v*64
+    const int nchunks = (p.K + CHUNK_K - 1) / CHUNK_K;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    const int col_begin = static_cast<int>(static_cast<int64_t>(blockIdx.x) * p.N / gridDim.x);
+    const int col_end = static_cast<int>(static_cast<int64_t>(blockIdx.x + 1) * p.N / gridDim.x);
+
+    // registers in fetch order (load i: rows lane/8 + 8*(i&1), bytes (i/2)*128 + (lane%8)*16 of the chunk's 256)
+    // -> registers in MFMA operand order, through this wavefront's LDS tile
+    auto transpose = [&](uint4 *r) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(stage + st_wr + (i & 1) * 8 * TROW + (i >> 1) * 128) = r[i];
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r[v] = *reinterpret_cast<const uint4 *>(stage + st_rd + v * 64);
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    // x: this wavefront's chunks, resident
+    uint4 xq[NCH][4];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int c = wave + j * NW;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = crow + 8 * (i & 1);
+            const int byte = (i >> 1) * 128 + cpiece * 16;
+            const bool ok = c < nchunks && m < p.M && c * CHUNK_K + byte / 2 < p.K;
+            xq[j][i] = ok ? *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte) : zero4;
+        }
+    }
+
+    uint4 wv[NCH][4];
+    // chunk j of the tile whose first column is n0 (columns from n_valid on do not belong to this block)
+    auto load_w = [&](auto jc, int n0, int n_valid) {
+        constexpr int j = decltype(jc)::value;
+        const int c = wave + j * NW;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int h = i & 1;
+            const int col = PAIR ? crow : crow + 8 * h;              // column of the tile this row belongs to
+            const char *base = (PAIR && h == 1 ? p.w2 : p.w) + static_cast<int64_t>(n0 + col) * p.ldw * 2;
+            const int byte = (i >> 1) * 128 + cpiece * 16;
+            const bool ok = c < nchunks && col < n_valid && c * CHUNK_K + byte / 2 < p.K;
+            wv[j][i] = ok ? nt_load_u4(base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte) : zero4;
+        }
+    };
+    auto for_each_chunk = [&](auto &&f) { static_for<NCH>(f); };
+
+    int n0 = col_begin;
+    if (n0 < col_end) for_each_chunk([&](auto jc) { load_w(jc, n0, col_end - n0); });
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) transpose(xq[j]);
+
+    for (int t = 0; n0 < col_end; ++t, n0 += COLS) {
+        const int n_valid = col_end - n0 < COLS ? col_end - n0 : COLS;
+        const int n_next = n0 + COLS;
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        for_each_chunk([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            if (wave + j * NW < nchunks) {
+                transpose(wv[j]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc = mfma16<DT>(wv[j][v], xq[j][v], acc);
+                if (n_next < col_end) load_w(jc, n_next, col_end - n_next);
+            }
+        });
+        float(*rd)[4][64] = red[t & 1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rd[wave][i][lane] = acc[i];
+        __syncthreads();
+        // thread e -> output (m = e / 16, n_local = e % 16)
+        if (tid < 256) {
+            const int m = tid >> 4, nl = tid & 15;
+            if (m < p.M && nl < n_valid) {  // pair: tile rows 8-15 are the up sums of columns 0-7, n_valid <= 8
+                const int n = n0 + nl;
+                const int src_lane = (nl >> 2) * 16 + m, i = nl & 3;
+                float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    s0 += rd[w][i][src_lane];
+                    if constexpr (PAIR) s1 += rd[w][i][src_lane + 32];  // row nl + 8: two lane groups further on
+                }
+                uint16_t out;
+                if constexpr (PAIR) {
+                    const float gv = half_to_f32<DT>(f32_to_half<DT>(s0));
+                    const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
+                    const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(gv)));
+                    out = f32_to_half<DT>(sl * u);
+                } else {
+                    float v = s0;
+                    if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
+                    if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+                    out = f32_to_half<DT>(v);
+                }
+                reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
+            }
+        }
+    }
+}
+
 // ---- M <= 4: row-streaming kernel --------------------------------------------------------------------
 // One wavefront owns one output column (linear: one row of w; gated pair: the gate row and the up row of that
 // column) over the whole of K. A load instruction covers 1 KiB of consecutive bytes of a row, K_BATCH of them
@@ -580,8 +715,38 @@ inline bool pick_pair(const SkinnyParams &p) {
     return p.M <= 32;
 }
 
+// The x-resident kernel pays when a CU would otherwise run several weight tiles and re-read x for each, and x is large
+// enough to matter. Measured on Llama-7B-sized shapes: from 9 rows and 1.25 tiles per CU on (gated pair 5504 x 4096 at
+// 16 rows: 31 -> 22 us, single matrix 11008 x 4096: 30 -> 24 us); below 9 rows the plain kernel is as fast or faster.
+// 16-bit weights, at most 16 rows, K up to 6144 (the x fragments have to fit the registers; above 4096 they leave
+// room for less, and it takes 3 tiles per CU to pay).
+template <int MODE>
+inline bool pick_resident(const SkinnyParams &p, int cus) {
+    if (p.M > 16 || p.K > 6144) return false;
+    if (const char *e = getenv("TPAMD_SKINNY_RESIDENT")) return atoi(e) != 0;
+    const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
+    if (p.M < 9) return false;
+    return p.K <= 4096 ? tiles * 4 >= 5ll * cus : tiles >= 3ll * cus;
+}
+
+template <int DT, int MODE>
+int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
+    const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
+    const unsigned grid = static_cast<unsigned>(tiles < cus ? tiles : cus);
+    if (p.K <= 4096) hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 4>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 6>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 template <int DT, bool W8, int MODE>
 int launch_skinny(const SkinnyParams &p, hipStream_t s) {
+    if constexpr (!W8) {
+        int dev = 0, cus = 256;
+        TPAMD_HIP(hipGetDevice(&dev));
+        TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        if (pick_resident<MODE>(p, cus)) return launch_resident<DT, MODE>(p, cus, s);
+    }
     if constexpr (MODE == SK_SWIGLU && !W8) {
         if (p.M <= 32 && pick_pair(p)) {
             const unsigned grid8 = static_cast<unsigned>((p.N + 7) / 8);

@@ -302,3 +302,24 @@ def test_strided_and_8_byte_aligned_outputs_through_the_c_abi(tile, N, ldy, shif
     want = ofw.gated_mlp_hidden(x.float().cpu(), w.float().cpu(), w2.float().cpu())
     torch.testing.assert_close(y[:, :N].float().cpu(), want, rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
     assert bool((y[:, N:] == 7.0).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [4, 9, 16])
+@pytest.mark.parametrize("N,K", [(64, 64), (132, 200), (1028, 1000), (2740, 4096), (520, 5504)])
+def test_x_resident_weight_streaming_kernel(dtype, M, N, K, monkeypatch):
+    """The weight-streaming kernel that keeps its x fragments in registers and walks a range of columns per block
+    (forced; by default it serves 9 to 16 rows when there are enough weight tiles per CU): fewer tiles than CUs,
+    several tiles per block with a masked last tile (2740 columns over 256 blocks), column ranges that do not start
+    on a multiple of 8, a ragged last K chunk, K above 4096 (6 chunks per wavefront), bias and GELU, the gated pair."""
+    monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "1")
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
+    check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
+    w2 = rnd((N, K), 5, 0.02, dtype)
+    h = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "0")
+    plain = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
+    torch.testing.assert_close(h.float(), plain.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
