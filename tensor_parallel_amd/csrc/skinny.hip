@@ -1,11 +1,13 @@
 // Rank-shard Linear for decode-sized M (M <= 64): weight streaming, HBM-bound.
 //
-// Two kernels:
+// Three kernels:
 //   skinny_kernel (4 <= M <= 32, int8 weights up to 64): a block owns 16 output columns (16 rows of w; for the
 //     SiLU-gated pair 16 gate rows + 16 up rows) and splits K over its wavefronts in chunks of 256 bytes of every
 //     w row. v_mfma_f32_16x16x32 does both the multiply and the reduction over K, so no cross-lane shuffles are
 //     needed. Partial sums of the wavefronts meet in LDS; the epilogue applies scale, outliers, bias, activation
 //     and stores 16 consecutive columns per row.
+//   skinny_resident_kernel (9 <= M <= 16, 16-bit weights, several weight tiles per CU): the same products, but a
+//     block stays on its CU, keeps its x fragments in registers and walks a range of output columns.
 //   gemv_kernel (M <= 3): one wavefront per output column, v_dot2 products, x in LDS.
 //
 // The weight is either the activation dtype (bf16/f16) or int8 (weight-only quantisation: converted to
