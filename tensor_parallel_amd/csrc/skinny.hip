@@ -410,13 +410,14 @@ __device__ __forceinline__ void static_for(F &&f) {
 // from 8 rows on those bytes weigh as much as the weights in what a CU can take in. Here a block stays on its CU and
 // walks a contiguous range of output columns (the N columns are split evenly over the blocks; the last tile of a
 // range is partly masked): wavefront w keeps the x fragments of its chunks w, w + 8, ... in registers for the whole
-// launch (NCH chunks: K <= NCH * 1024), and the weights of the next tile are requested chunk by chunk as soon as the
-// registers of the current tile's chunk are free, so a wavefront always has about NCH * 4 KiB of weights in flight.
+// launch (NCH chunks: K <= NCH * NW * 128). Weights go through DEPTH register slots per wavefront: as soon as a chunk
+// has been multiplied, the chunk DEPTH further on in the stream (of this or the next tile) is requested into its slot,
+// so a wavefront always has about DEPTH * 4 KiB of weights in flight.
 // Partial sums of the wavefronts meet in LDS once per tile (two buffers, one barrier per tile).
 // MODE SK_SWIGLU: the tile is 8 gate rows + the 8 up rows of the same 8 columns (16-bit weights only).
-template <int DT, int MODE, int NCH>
-__global__ __launch_bounds__(SK_THREADS) void skinny_resident_kernel(SkinnyParams p) {
-    constexpr int NW = SK_WAVES;
+template <int DT, int MODE, int NW, int NCH, int DEPTH>
+__global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p) {
+    static_assert(NCH % DEPTH == 0, "a chunk's slot must not depend on the tile");
     constexpr bool PAIR = MODE == SK_SWIGLU;
     constexpr int COLS = PAIR ? 8 : 16;
     constexpr int CHUNK_K = 128;                // K elements per chunk: 256 bytes of every row
@@ -462,7 +463,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_resident_kernel(SkinnyParam
         }
     }
 
-    uint4 wv[NCH][4];
+    uint4 wv[DEPTH][4];
     // chunk j of the tile whose first column is n0 (columns from n_valid on do not belong to this block)
     auto load_w = [&](auto jc, int n0, int n_valid) {
         constexpr int j = decltype(jc)::value;
@@ -474,13 +475,13 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_resident_kernel(SkinnyParam
             const char *base = (PAIR && h == 1 ? p.w2 : p.w) + static_cast<int64_t>(n0 + col) * p.ldw * 2;
             const int byte = (i >> 1) * 128 + cpiece * 16;
             const bool ok = c < nchunks && col < n_valid && c * CHUNK_K + byte / 2 < p.K;
-            wv[j][i] = ok ? nt_load_u4(base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte) : zero4;
+            wv[j % DEPTH][i] = ok ? nt_load_u4(base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte) : zero4;
         }
     };
     auto for_each_chunk = [&](auto &&f) { static_for<NCH>(f); };
 
     int n0 = col_begin;
-    if (n0 < col_end) for_each_chunk([&](auto jc) { load_w(jc, n0, col_end - n0); });
+    if (n0 < col_end) static_for<DEPTH>([&](auto jc) { load_w(jc, n0, col_end - n0); });
 #pragma unroll
     for (int j = 0; j < NCH; ++j) transpose(xq[j]);
 
@@ -490,12 +491,13 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_resident_kernel(SkinnyParam
         f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
         for_each_chunk([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            if (wave + j * NW < nchunks) {
-                transpose(wv[j]);
+            // (chunks past the end of K are zeros on both sides: multiplied anyway, so that every slot is refilled
+            // at the same place in every wavefront)
+            transpose(wv[j % DEPTH]);
 #pragma unroll
-                for (int v = 0; v < 4; ++v) acc = mfma16<DT>(wv[j][v], xq[j][v], acc);
-                if (n_next < col_end) load_w(jc, n_next, col_end - n_next);
-            }
+            for (int v = 0; v < 4; ++v) acc = mfma16<DT>(wv[j % DEPTH][v], xq[j][v], acc);
+            if constexpr (j + DEPTH < NCH) load_w(std::integral_constant<int, j + DEPTH>{}, n0, n_valid);
+            else if (n_next < col_end) load_w(std::integral_constant<int, j + DEPTH - NCH>{}, n_next, col_end - n_next);
         });
         float(*rd)[4][64] = red[t & 1];
 #pragma unroll
@@ -717,26 +719,30 @@ inline bool pick_pair(const SkinnyParams &p) {
     return p.M <= 32;
 }
 
-// The x-resident kernel pays when a CU would otherwise run several weight tiles and re-read x for each, and x is large
-// enough to matter. Measured on Llama-7B-sized shapes: from 9 rows and 1.25 tiles per CU on (gated pair 5504 x 4096 at
-// 16 rows: 31 -> 22 us, single matrix 11008 x 4096: 30 -> 24 us); below 9 rows the plain kernel is as fast or faster.
-// 16-bit weights, at most 16 rows, K up to 6144 (the x fragments have to fit the registers; above 4096 they leave
-// room for less, and it takes 3 tiles per CU to pay).
+// The x-resident kernel pays when x is large enough to matter and a CU would otherwise re-read it for several weight
+// tiles. Measured on Llama-7B-sized shapes (K = 4096): gated pair from 9 rows and 1.25 tiles per CU on (5504 columns at
+// 16 rows: 31 -> 22 us), single matrix from 12 rows and one tile per CU on (4096 columns at 16 rows: 14 -> 11.5 us:
+// all of x is requested up front instead of chunk by chunk); with fewer rows, or K = 2048, the plain kernel, with
+// more blocks per CU, is as fast or faster. 16-bit weights, at most 16 rows, K up to 6144 (the x fragments have to
+// fit the registers; above 4096 they leave room for little else, and it takes 3 tiles per CU to pay).
 template <int MODE>
 inline bool pick_resident(const SkinnyParams &p, int cus) {
     if (p.M > 16 || p.K > 6144) return false;
     if (const char *e = getenv("TPAMD_SKINNY_RESIDENT")) return atoi(e) != 0;
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
-    if (p.M < 9) return false;
-    return p.K <= 4096 ? tiles * 4 >= 5ll * cus : tiles >= 3ll * cus;
+    if (p.K < 3072) return false;
+    if (p.K > 4096) return p.M >= 9 && tiles >= 3ll * cus;
+    return MODE == SK_SWIGLU ? p.M >= 9 && tiles * 4 >= 5ll * cus : p.M >= 12 && tiles >= cus;
 }
 
 template <int DT, int MODE>
 int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     const unsigned grid = static_cast<unsigned>(tiles < cus ? tiles : cus);
-    if (p.K <= 4096) hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 4>), dim3(grid), dim3(SK_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 6>), dim3(grid), dim3(SK_THREADS), 0, s, p);
+    // (two blocks of 4 wavefronts per CU, 8 chunks each and 4 register slots, were measured too: the registers do
+    // not fit and the kernel takes twice as long)
+    if (p.K <= 4096) hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 4, 4>), dim3(grid), dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 6, 6>), dim3(grid), dim3(512), 0, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }
