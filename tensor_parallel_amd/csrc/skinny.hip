@@ -720,29 +720,30 @@ inline bool pick_pair(const SkinnyParams &p) {
 }
 
 // The x-resident kernel pays when x is large enough to matter and a CU would otherwise re-read it for several weight
-// tiles. Measured on Llama-7B-sized shapes (K = 4096): gated pair from 9 rows and 1.25 tiles per CU on (5504 columns at
-// 16 rows: 31 -> 22 us), single matrix from 12 rows and one tile per CU on (4096 columns at 16 rows: 14 -> 11.5 us:
-// all of x is requested up front instead of chunk by chunk); with fewer rows, or K = 2048, the plain kernel, with
-// more blocks per CU, is as fast or faster. 16-bit weights, at most 16 rows, K up to 6144 (the x fragments have to
-// fit the registers; above 4096 they leave room for little else, and it takes 3 tiles per CU to pay).
+// tiles. Measured on Llama-7B-sized shapes: gated pair from 9 rows and 1.25 tiles per CU on (5504 columns, K = 4096,
+// 16 rows: 31 -> 22 us; 11008 columns, K = 5504: 74 -> 49 us), single matrix from 12 rows and 1.5 tiles per CU or 14
+// rows and one tile per CU on (4096 columns at 16 rows: K = 4096 14 -> 11.5 us, K = 5504 17 -> 16 us: all of x is
+// requested up front instead of chunk by chunk); with fewer rows, or K = 2048, the plain kernel, with more blocks per
+// CU, is as fast or faster. 16-bit weights, at most 16 rows, K up to 6144 (the x fragments have to fit the registers).
 template <int MODE>
 inline bool pick_resident(const SkinnyParams &p, int cus) {
     if (p.M > 16 || p.K > 6144) return false;
     if (const char *e = getenv("TPAMD_SKINNY_RESIDENT")) return atoi(e) != 0;
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     if (p.K < 3072) return false;
-    if (p.K > 4096) return p.M >= 9 && tiles >= 3ll * cus;
-    return MODE == SK_SWIGLU ? p.M >= 9 && tiles * 4 >= 5ll * cus : p.M >= 12 && tiles >= cus;
+    if (MODE == SK_SWIGLU) return p.M >= 9 && tiles * 4 >= 5ll * cus;
+    return (p.M >= 12 && tiles * 2 >= 3ll * cus) || (p.M >= 14 && tiles >= cus);
 }
 
 template <int DT, int MODE>
 int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     const unsigned grid = static_cast<unsigned>(tiles < cus ? tiles : cus);
-    // (two blocks of 4 wavefronts per CU, 8 chunks each and 4 register slots, were measured too: the registers do
-    // not fit and the kernel takes twice as long)
+    // K <= 4096: 4 chunks per wavefront, a slot each; above: 6 chunks and 3 slots (6 slots do not fit the registers).
+    // (Two blocks of 4 wavefronts per CU, 8 chunks each and 4 slots, were measured too: the registers do not fit and
+    // the kernel takes twice as long.)
     if (p.K <= 4096) hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 4, 4>), dim3(grid), dim3(512), 0, s, p);
-    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 6, 6>), dim3(grid), dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 6, 3>), dim3(grid), dim3(512), 0, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }
