@@ -75,6 +75,25 @@ __device__ __forceinline__ void cvt_i8x4(uint32_t q, uint32_t &lo, uint32_t &hi)
     }
 }
 
+// One output element from its fp32 sums (s1 = the up sum of a gated pair): the reference's op chain with its
+// roundings to the tensor dtype (gate and up products, SiLU, product), or bias and activation.
+template <int DT, int MODE>
+__device__ __forceinline__ void skinny_store_output(const SkinnyParams &p, float s0, float s1, int m, int n) {
+    uint16_t out;
+    if constexpr (MODE == SK_SWIGLU) {
+        const float gv = half_to_f32<DT>(f32_to_half<DT>(s0));
+        const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
+        const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(gv)));
+        out = f32_to_half<DT>(sl * u);
+    } else {
+        float v = s0;
+        if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
+        if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+        out = f32_to_half<DT>(v);
+    }
+    reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
+}
+
 // W8 = weight is int8. MT = number of 16-row tiles of x (M <= 16*MT). MODE = SK_LINEAR / SK_SWIGLU.
 //
 // Fetching. The MFMA row operand wants lane l to hold 16 bytes of row l%16 at K slot l/16; loading it that way
@@ -379,19 +398,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(SkinnyParams p) {
                 if constexpr (NMAT == 2) s1 += red[w][1][t][i][src_lane];
                 if constexpr (PAIR) s1 += red[w][0][t][i][src_lane + 32];  // row nl + 8: two lane groups further on
             }
-            uint16_t out;
-            if constexpr (MODE == SK_SWIGLU) {
-                const float gv = half_to_f32<DT>(f32_to_half<DT>(s0));
-                const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
-                const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(gv)));
-                out = f32_to_half<DT>(sl * u);
-            } else {
-                float v = s0;
-                if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
-                if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
-                out = f32_to_half<DT>(v);
-            }
-            reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
+            skinny_store_output<DT, MODE>(p, s0, s1, m, n);
         }
     }
 }
@@ -515,19 +522,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
                     s0 += rd[w][i][src_lane];
                     if constexpr (PAIR) s1 += rd[w][i][src_lane + 32];  // row nl + 8: two lane groups further on
                 }
-                uint16_t out;
-                if constexpr (PAIR) {
-                    const float gv = half_to_f32<DT>(f32_to_half<DT>(s0));
-                    const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
-                    const float sl = half_to_f32<DT>(f32_to_half<DT>(silu_f32(gv)));
-                    out = f32_to_half<DT>(sl * u);
-                } else {
-                    float v = s0;
-                    if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
-                    if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
-                    out = f32_to_half<DT>(v);
-                }
-                reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
+                skinny_store_output<DT, MODE>(p, s0, s1, m, n);
             }
         }
     }
@@ -664,21 +659,7 @@ __global__ __launch_bounds__(GV_WAVES * 64) void gemv_kernel(SkinnyParams p) {
         float s1 = 0.f;
         if constexpr (NMAT == 2) s1 = wave_sum(acc[NMAT - 1][m]);
         if constexpr (W8) s0 = s0 * p.scale[row] + wave_sum(acc_o[m]);
-        if (lane == 0 && live) {
-            uint16_t out;
-            if constexpr (MODE == SK_SWIGLU) {
-                const float g = half_to_f32<DT>(f32_to_half<DT>(s0));
-                const float u = half_to_f32<DT>(f32_to_half<DT>(s1));
-                const float sg = half_to_f32<DT>(f32_to_half<DT>(silu_f32(g)));
-                out = f32_to_half<DT>(sg * u);
-            } else {
-                float v = s0;
-                if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
-                if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
-                out = f32_to_half<DT>(v);
-            }
-            reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
-        }
+        if (lane == 0 && live) skinny_store_output<DT, MODE>(p, s0, s1, m, n);
     }
 }
 
