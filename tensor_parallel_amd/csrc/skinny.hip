@@ -15,6 +15,7 @@
 #include "common.h"
 
 #include <stdlib.h>
+#include <mutex>
 #include <type_traits>
 
 namespace tpamd {
@@ -528,6 +529,189 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
     }
 }
 
+// ---- int8 weights, 12 <= M <= 64: K split over blocks, x resident -----------------------------------------
+// With int8 weights x weighs 2 * M bytes per K element against 16 for the 16 weight rows of a tile, and a block
+// that covers all of K has to pull all of x through its CU for every tile: at M = 32 that is as many bytes as the
+// weights themselves. Here the grid is (column ranges, K splits): wavefront w of a block owns NCH chunks of 256 K
+// elements (a split is NCH * 2048 elements), keeps their x fragments in registers (NCH x MT tiles of 16 rows x 8
+// registers: 128 registers for MT * NCH = 4) and walks the 16-row weight tiles of the block's column range, so per
+// CU x is read once per split while the weights of 256 or more columns stream past. A chunk's registers are refilled
+// with the same chunk of the next tile as soon as it has been handed to the MFMA operands. Partial sums of the 8
+// wavefronts meet in LDS once per tile (two buffers, one barrier per tile), are scaled per output row, get the
+// outlier product added (split 0 only) and go to a [split][M][N] fp32 array; skinny_w8_finish_kernel adds the
+// splits, bias and activation.
+template <int DT, int MT, int NCH>
+__global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParams p, float *part, int cols_per_block) {
+    constexpr int NW = SK_WAVES;
+    constexpr int CHUNK_K = 256;                // K elements per chunk: 256 bytes of a weight row, 512 of an x row
+    constexpr int TROW = 272;
+    __shared__ float red[2][NW][MT][4][64];
+    __shared__ __align__(16) char stage_all[NW][16 * TROW];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int crow = lane >> 3, cpiece = lane & 7;
+    char *stage = stage_all[wave];
+    const int st_wr = crow * TROW + cpiece * 16;   // + (i&1)*8*TROW + (i/2)*128
+    const int st_rd = lr * TROW + lg * 16;         // + v*64
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    const int split = blockIdx.y;
+    const int col_begin = blockIdx.x * cols_per_block;
+    const int col_end = col_begin + cols_per_block < p.N ? col_begin + cols_per_block : p.N;
+    // first K element of this wavefront's chunk j
+    auto chunk_k0 = [&](int j) { return (static_cast<int64_t>(split * NCH + j) * NW + wave) * CHUNK_K; };
+
+    auto stage_in = [&](const uint4 *r) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(stage + st_wr + (i & 1) * 8 * TROW + (i >> 1) * 128) = r[i];
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    };
+    auto stage_done = [&]() {
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    // x fragments of this wavefront's chunks, in the operand order that meets the int8 tile: lane slot lg holds
+    // k = v*64 + lg*16 + h*8 .. +8 in register 2*v + h
+    uint4 xq[NCH][MT][8];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int m = t * 16 + crow + 8 * (i & 1);
+                const int byte = (i >> 1) * 128 + cpiece * 16;
+                const int64_t k0 = chunk_k0(j);
+                const bool ok = m < p.M && k0 + byte / 2 < p.K;
+                xq[j][t][i] = ok ? *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + k0 * 2 + byte) : zero4;
+            }
+#pragma unroll
+    for (int j = 0; j < NCH; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                stage_in(&xq[j][t][half * 4]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    xq[j][t][half * 4 + v] = *reinterpret_cast<const uint4 *>(stage + lr * TROW + (v >> 1) * 128 + lg * 32 + (v & 1) * 16);
+                stage_done();
+            }
+
+    // outlier columns (split 0): wavefront w takes outliers 32w .. 32w + 31 (n_out <= 256); its x values once
+    const bool outl = split == 0 && wave * 32 < p.n_out;
+    uint4 xo[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        uint32_t q[4] = {0, 0, 0, 0};
+        if (outl) {
+            const uint16_t *xs = reinterpret_cast<const uint16_t *>(p.x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int o = wave * 32 + lg * 8 + j;
+                if (o < p.n_out && t * 16 + lr < p.M) {
+                    const uint32_t xval = xs[static_cast<int64_t>(t * 16 + lr) * p.ldx + p.outlier_idx[o]];
+                    q[j >> 1] |= xval << ((j & 1) * 16);
+                }
+            }
+        }
+        xo[t] = make_uint4(q[0], q[1], q[2], q[3]);
+    }
+
+    uint4 wv[NCH][4];
+    auto load_w = [&](auto jc, int n0) {
+        constexpr int j = decltype(jc)::value;
+        const int64_t k0 = chunk_k0(j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = n0 + crow + 8 * (i & 1);
+            const int byte = (i >> 1) * 128 + cpiece * 16;
+            const bool ok = row < col_end && k0 + byte < p.K;
+            wv[j][i] = ok ? nt_load_u4(p.w + static_cast<int64_t>(row) * p.ldw + k0 + byte) : zero4;
+        }
+    };
+    if (col_begin < col_end) static_for<NCH>([&](auto jc) { load_w(jc, col_begin); });
+
+    int t_index = 0;
+    for (int n0 = col_begin; n0 < col_end; n0 += 16, ++t_index) {
+        f32x4 acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        static_for<NCH>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            stage_in(wv[j]);
+            uint4 wt[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) wt[v] = *reinterpret_cast<const uint4 *>(stage + st_rd + v * 64);
+            stage_done();
+            if (n0 + 16 < col_end) load_w(jc, n0 + 16);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {  // 16 int8 -> two operands of 8
+                uint4 w0, w1;
+                cvt_i8x4<DT>(wt[v].x, w0.x, w0.y);
+                cvt_i8x4<DT>(wt[v].y, w0.z, w0.w);
+                cvt_i8x4<DT>(wt[v].z, w1.x, w1.y);
+                cvt_i8x4<DT>(wt[v].w, w1.z, w1.w);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    acc[t] = mfma16<DT>(w0, xq[j][t][2 * v], acc[t]);
+                    acc[t] = mfma16<DT>(w1, xq[j][t][2 * v + 1], acc[t]);
+                }
+            }
+        });
+        // per-row scale, then the outlier product. D[n_local][m_local]: lane -> m_local = lr, register i -> n_local = 4*lg + i
+        float sc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + lg * 4 + i;
+            sc[i] = p.scale[n < p.N ? n : p.N - 1];
+        }
+        uint4 wo4 = zero4;
+        if (outl) {
+            const uint16_t *wo = reinterpret_cast<const uint16_t *>(p.w_out);
+            const int wr = n0 + lr < p.N ? n0 + lr : p.N - 1;
+            uint32_t q[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int o = wave * 32 + lg * 8 + j;
+                if (o < p.n_out) q[j >> 1] |= static_cast<uint32_t>(wo[static_cast<int64_t>(wr) * p.ld_wout + o]) << ((j & 1) * 16);
+            }
+            wo4 = make_uint4(q[0], q[1], q[2], q[3]);
+        }
+        float(*rd)[MT][4][64] = red[t_index & 1];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            f32x4 v = f32x4{acc[t][0] * sc[0], acc[t][1] * sc[1], acc[t][2] * sc[2], acc[t][3] * sc[3]};
+            if (outl) v = mfma16<DT>(wo4, xo[t], v);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) rd[wave][t][i][lane] = v[i];
+        }
+        __syncthreads();
+        for (int e = tid; e < MT * 256; e += NW * 64) {
+            const int m = e >> 4, nl = e & 15, n = n0 + nl;
+            if (m >= p.M || n >= col_end) continue;
+            const int t = m >> 4, src_lane = (nl >> 2) * 16 + (m & 15), i = nl & 3;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += rd[w][t][i][src_lane];
+            part[(static_cast<int64_t>(split) * p.M + m) * p.N + n] = sum;
+        }
+    }
+}
+
+// y[m][n] = act(sum over splits of part[split][m][n] + bias[n])
+template <int DT>
+__global__ __launch_bounds__(256) void skinny_w8_finish_kernel(SkinnyParams p, const float *part, int splits) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= static_cast<int64_t>(p.M) * p.N) return;
+    const int m = static_cast<int>(e / p.N), n = static_cast<int>(e % p.N);
+    float v = 0.f;
+    for (int sp = 0; sp < splits; ++sp) v += part[static_cast<int64_t>(sp) * p.M * p.N + e];
+    skinny_store_output<DT, SK_LINEAR>(p, v, 0.f, m, n);
+}
+
 // ---- M <= 4: row-streaming kernel --------------------------------------------------------------------
 // One wavefront owns one output column (linear: one row of w; gated pair: the gate row and the up row of that
 // column) over the whole of K. A load instruction covers 1 KiB of consecutive bytes of a row, K_BATCH of them
@@ -729,8 +913,60 @@ int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
     return TPAMD_OK;
 }
 
+// int8 weights, K split over blocks: K at least 4096, at most 64 rows and 256 outlier columns.
+// Needs the per-device scratch buffer for the partial sums; without it (first use under stream capture) the
+// caller takes the unsplit kernel.
+template <int DT>
+int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
+    *done = false;
+    if (const char *e = getenv("TPAMD_W8_SPLIT")) {
+        if (atoi(e) == 0) return TPAMD_OK;
+    } else {
+        // Measured (Falcon-40B MLP shard, 16384 x 8192 and 8192 x 16384, and smaller matrices): from 25 rows on it
+        // always pays (32 rows: 57 -> 47 us and 79 -> 49 us, 64 rows: 114 -> 72 us and 156 -> 73 us), from 17 rows
+        // on for matrices of 32 M elements or more, from 12 rows on for 64 M elements or more; below that the
+        // unsplit kernel, with more blocks per CU and no second launch, is as fast or faster.
+        const int64_t elems = static_cast<int64_t>(p.N) * p.K;
+        const bool pays = p.M > 24 || (p.M > 16 && elems >= (1ll << 25)) || (p.M >= 12 && elems >= (1ll << 26));
+        if (!pays) return TPAMD_OK;
+    }
+    if (p.K < 4096 || p.n_out > 256 || p.M > 64) return TPAMD_OK;
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    // x fragments fill 128 registers: 4 chunks per wavefront (8192 K elements per split) for 16 rows, 2 for 32, 1 for 64
+    const int nch = p.M <= 16 ? 4 : p.M <= 32 ? 2 : 1;
+    const int splits = (p.K + nch * 2048 - 1) / (nch * 2048);
+    int col_blocks = cus / splits > 0 ? cus / splits : 1;
+    int cols_per_block = (p.N + col_blocks - 1) / col_blocks;
+    cols_per_block = (cols_per_block + 15) / 16 * 16;
+    col_blocks = (p.N + cols_per_block - 1) / cols_per_block;
+    const size_t need = static_cast<size_t>(splits) * p.M * p.N * sizeof(float);
+    std::lock_guard<std::mutex> hold(splitk_mutex());
+    void *ws = nullptr;
+    const int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
+    if (rc != TPAMD_OK) return rc;
+    if (ws == nullptr) return TPAMD_OK;
+    float *part = static_cast<float *>(ws);
+    const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(splits));
+    if (p.M <= 16) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 1, 4>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
+    else if (p.M <= 32) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 2, 2>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
+    else hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 4, 1>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
+    TPAMD_HIP(hipGetLastError());
+    const int64_t outputs = static_cast<int64_t>(p.M) * p.N;
+    hipLaunchKernelGGL((skinny_w8_finish_kernel<DT>), dim3(static_cast<unsigned>((outputs + 255) / 256)), dim3(256), 0, s, p, part, splits);
+    TPAMD_HIP(hipGetLastError());
+    *done = true;
+    return TPAMD_OK;
+}
+
 template <int DT, bool W8, int MODE>
 int launch_skinny(const SkinnyParams &p, hipStream_t s) {
+    if constexpr (W8) {
+        bool done = false;
+        const int rc = launch_w8_split<DT>(p, s, &done);
+        if (rc != TPAMD_OK || done) return rc;
+    }
     if constexpr (!W8) {
         int dev = 0, cus = 256;
         TPAMD_HIP(hipGetDevice(&dev));

@@ -117,3 +117,28 @@ def test_16bit_decode_kernels_column_groups(dtype, M, cg, column_groups):
     lin, sw = _native.linear(x, w1), _native.swiglu_up(x, w1, w2)  # the gated pair uses at most 2 groups
     assert torch.equal(lin, lin1) and torch.equal(sw, sw1)
     torch.testing.assert_close(lin.float(), torch.nn.functional.linear(x.float(), w1.float()), rtol=2e-2, atol=2e-2 * 0.05 * math.sqrt(K))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [9, 16, 17, 32, 33, 64, 70])
+@pytest.mark.parametrize("N,K,n_out", [(64, 4096, 0), (200, 4128, 5), (1000, 8192, 41), (528, 6144, 33), (48, 16384, 256)])
+def test_k_split_kernel(dtype, M, N, K, n_out, monkeypatch):
+    """The int8 kernel that splits K over blocks and keeps its x fragments in registers (forced; by default it
+    serves 12 or more rows on large matrices): 1, 2 and 4 row tiles, a single split and several, a last split that
+    is partly or wholly past the end of K, column ranges whose last tile is masked, outlier columns on wavefronts
+    0 to 7 of split 0, more than 64 rows (slabs), bias and GELU. Same products as the unsplit kernel in another
+    order: both are compared with the definition, and with each other."""
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, dtype, seed=4)
+    args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+            torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None,
+            torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(5)) * 0.1).to(dtype).to(DEV)
+    monkeypatch.setenv("TPAMD_W8_SPLIT", "1")
+    got = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
+    monkeypatch.setenv("TPAMD_W8_SPLIT", "0")
+    plain = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out) + bias.double().cpu().numpy()
+    want = 0.5 * want * (1.0 + np.vectorize(math.erf)(want / math.sqrt(2.0)))
+    sigma = 0.02 * math.sqrt(K + 400 * n_out)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
+    torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * sigma)
