@@ -14,7 +14,8 @@
  *     message for the calling thread;
  *   - every entry point may be called concurrently from several host threads. Besides the thread-local error
  *     message the library keeps one piece of state: tpamd_linear / tpamd_swiglu_up split K for shapes with few
- *     output tiles (M from 17 to a few thousand, decided by a cost model) and keep one fp32 scratch buffer per
+ *     output tiles (M from 17 to a few thousand, decided by a cost model), tpamd_linear_w8 does so from 12 rows on
+ *     large matrices, tpamd_attention splits long key ranges, and they keep one fp32 scratch buffer per
  *     device for that (64 MiB on a 256-CU part), allocated with hipMalloc at first use and kept until the process
  *     ends. Such calls are ordered by their stream; a caller that spreads them over several streams of one device
  *     must order those streams itself. If the first such call happens under stream capture, nothing is allocated
