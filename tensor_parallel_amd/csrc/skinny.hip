@@ -539,8 +539,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
 // with the same chunk of the next tile as soon as it has been handed to the MFMA operands. Partial sums of the 8
 // wavefronts meet in LDS once per tile (two buffers, one barrier per tile), are scaled per output row, get the
 // outlier product added (split 0 only) and go to a [split][M][N] fp32 array; skinny_w8_finish_kernel adds the
-// splits, bias and activation.
-template <int DT, int MT, int NCH>
+// splits, bias and activation. DIRECT (a single split): bias, activation and the store to y happen here.
+template <int DT, int MT, int NCH, bool DIRECT>
 __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParams p, float *part, int cols_per_block) {
     constexpr int NW = SK_WAVES;
     constexpr int CHUNK_K = 256;                // K elements per chunk: 256 bytes of a weight row, 512 of an x row
@@ -696,7 +696,8 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParam
             float sum = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) sum += rd[w][t][i][src_lane];
-            part[(static_cast<int64_t>(split) * p.M + m) * p.N + n] = sum;
+            if constexpr (DIRECT) skinny_store_output<DT, SK_LINEAR>(p, sum, 0.f, m, n);
+            else part[(static_cast<int64_t>(split) * p.M + m) * p.N + n] = sum;
         }
     }
 }
@@ -941,6 +942,15 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     int cols_per_block = (p.N + col_blocks - 1) / col_blocks;
     cols_per_block = (cols_per_block + 15) / 16 * 16;
     col_blocks = (p.N + cols_per_block - 1) / cols_per_block;
+    const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(splits));
+    if (splits == 1) {  // nothing to add up: no scratch buffer, no second launch
+        if (p.M <= 16) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 1, 4, true>), grid, dim3(SK_THREADS), 0, s, p, nullptr, cols_per_block);
+        else if (p.M <= 32) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 2, 2, true>), grid, dim3(SK_THREADS), 0, s, p, nullptr, cols_per_block);
+        else hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 4, 1, true>), grid, dim3(SK_THREADS), 0, s, p, nullptr, cols_per_block);
+        TPAMD_HIP(hipGetLastError());
+        *done = true;
+        return TPAMD_OK;
+    }
     const size_t need = static_cast<size_t>(splits) * p.M * p.N * sizeof(float);
     std::lock_guard<std::mutex> hold(splitk_mutex());
     void *ws = nullptr;
@@ -948,10 +958,9 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     if (rc != TPAMD_OK) return rc;
     if (ws == nullptr) return TPAMD_OK;
     float *part = static_cast<float *>(ws);
-    const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(splits));
-    if (p.M <= 16) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 1, 4>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
-    else if (p.M <= 32) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 2, 2>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
-    else hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 4, 1>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
+    if (p.M <= 16) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 1, 4, false>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
+    else if (p.M <= 32) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 2, 2, false>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
+    else hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 4, 1, false>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
     TPAMD_HIP(hipGetLastError());
     const int64_t outputs = static_cast<int64_t>(p.M) * p.N;
     hipLaunchKernelGGL((skinny_w8_finish_kernel<DT>), dim3(static_cast<unsigned>((outputs + 255) / 256)), dim3(256), 0, s, p, part, splits);
