@@ -890,13 +890,20 @@ inline bool pick_pair(const SkinnyParams &p) {
 // 16 rows: 31 -> 22 us; 11008 columns, K = 5504: 74 -> 49 us), single matrix from 12 rows and 1.5 tiles per CU or 14
 // rows and one tile per CU on (4096 columns at 16 rows: K = 4096 14 -> 11.5 us, K = 5504 17 -> 16 us: all of x is
 // requested up front instead of chunk by chunk); with fewer rows, or K = 2048, the plain kernel, with more blocks per
-// CU, is as fast or faster. 16-bit weights, at most 16 rows, K up to 6144 (the x fragments have to fit the registers).
+// CU, is as fast or faster. 16-bit weights, at most 16 rows, K up to 8192 (the x fragments have to fit the registers).
 template <int MODE>
 inline bool pick_resident(const SkinnyParams &p, int cus) {
-    if (p.M > 16 || p.K > 6144) return false;
+    if (p.M > 16 || p.K > 8192) return false;
     if (const char *e = getenv("TPAMD_SKINNY_RESIDENT")) return atoi(e) != 0;
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     if (p.K < 3072) return false;
+    if (p.K > 6144) {
+        // 8 chunks per wavefront leave 2 register slots for the weights: gated pair from 12 rows on (16384 columns,
+        // K = 8192, 16 rows: 144 -> 96 us), single matrix only where the plain kernel's blocks do not fill the CUs
+        // evenly (4608 columns = 1.125 tiles per CU, 16 rows: 38 -> 33 us; at 2 tiles per CU it loses)
+        if (MODE == SK_SWIGLU) return p.M >= 12 && tiles * 4 >= 5ll * cus;
+        return p.M >= 14 && tiles >= cus && tiles * 2 < 3ll * cus;
+    }
     if (MODE == SK_SWIGLU) return p.M >= 9 && tiles * 4 >= 5ll * cus;
     return (p.M >= 12 && tiles * 2 >= 3ll * cus) || (p.M >= 14 && tiles >= cus);
 }
@@ -905,11 +912,13 @@ template <int DT, int MODE>
 int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     const unsigned grid = static_cast<unsigned>(tiles < cus ? tiles : cus);
-    // K <= 4096: 4 chunks per wavefront, a slot each; above: 6 chunks and 3 slots (6 slots do not fit the registers).
+    // K <= 4096: 4 chunks per wavefront, a slot each; up to 6144: 6 chunks and 3 slots (6 slots do not fit the
+    // registers); up to 8192: 8 chunks and 2 slots.
     // (Two blocks of 4 wavefronts per CU, 8 chunks each and 4 slots, were measured too: the registers do not fit and
     // the kernel takes twice as long.)
     if (p.K <= 4096) hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 4, 4>), dim3(grid), dim3(512), 0, s, p);
-    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 6, 3>), dim3(grid), dim3(512), 0, s, p);
+    else if (p.K <= 6144) hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 6, 3>), dim3(grid), dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((skinny_resident_kernel<DT, MODE, 8, 8, 2>), dim3(grid), dim3(512), 0, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }

@@ -306,12 +306,13 @@ def test_strided_and_8_byte_aligned_outputs_through_the_c_abi(tile, N, ldy, shif
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [4, 9, 16])
-@pytest.mark.parametrize("N,K", [(64, 64), (132, 200), (1028, 1000), (2740, 4096), (520, 5504)])
+@pytest.mark.parametrize("N,K", [(64, 64), (132, 200), (1028, 1000), (2740, 4096), (520, 5504), (300, 8192), (260, 7000)])
 def test_x_resident_weight_streaming_kernel(dtype, M, N, K, monkeypatch):
     """The weight-streaming kernel that keeps its x fragments in registers and walks a range of columns per block
     (forced; by default it serves 9 to 16 rows when there are enough weight tiles per CU): fewer tiles than CUs,
     several tiles per block with a masked last tile (2740 columns over 256 blocks), column ranges that do not start
-    on a multiple of 8, a ragged last K chunk, K above 4096 (6 chunks per wavefront), bias and GELU, the gated pair."""
+    on a multiple of 8, a ragged last K chunk, K above 4096 and above 6144 (6 and 8 chunks per wavefront), bias and
+    GELU, the gated pair."""
     monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "1")
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
