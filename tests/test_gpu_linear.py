@@ -324,3 +324,33 @@ def test_x_resident_weight_streaming_kernel(dtype, M, N, K, monkeypatch):
     monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "0")
     plain = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
     torch.testing.assert_close(h.float(), plain.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+
+
+@pytest.mark.parametrize("case", ["tiles256_split", "resident_pair", "resident_single"])
+def test_other_dispatch_paths_inside_a_hip_graph(case, monkeypatch):
+    """The 256 x 256 tiling with K split over blocks (two launches sharing the scratch buffer) and the x-resident
+    weight-streaming kernel, recorded into a HIP graph after a warm-up call: every replay gives the eager result,
+    with eager work in between."""
+    if case == "tiles256_split":
+        monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
+        monkeypatch.setenv("TPAMD_GEMM_SPLITK256", "3")
+        M, N, K = 300, 520, 1088
+    else:
+        monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "1")
+        M, N, K = 16, 2740, 4096
+    x, w, w2 = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N, K), 5, 0.02).to(DEV)
+    fn = (lambda: _native.swiglu_up(x, w, w2)) if case == "resident_pair" else (lambda: _native.linear(x, w))
+    eager = fn()
+    torch.cuda.synchronize()
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out.copy_(fn())
+    for i in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        assert torch.equal(fn(), eager)  # eager work between replays

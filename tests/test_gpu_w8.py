@@ -142,3 +142,27 @@ def test_k_split_kernel(dtype, M, N, K, n_out, monkeypatch):
     sigma = 0.02 * math.sqrt(K + 400 * n_out)
     torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
     torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * sigma)
+
+
+def test_k_split_kernel_inside_a_hip_graph(monkeypatch):
+    """The K-split int8 kernel and its finishing pass (two launches sharing the library's scratch buffer) recorded
+    into a HIP graph after a warm-up call: every replay gives the eager result, with eager work in between."""
+    monkeypatch.setenv("TPAMD_W8_SPLIT", "1")
+    M, N, K, n_out = 32, 200, 8192, 41
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, torch.float16, seed=6)
+    args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+            torch.from_numpy(cols.astype(np.int32)).to(DEV), torch.from_numpy(w_out).half().to(DEV))
+    eager = _native.linear_w8(*args)
+    torch.cuda.synchronize()
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out.copy_(_native.linear_w8(*args))
+    for i in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        assert torch.equal(_native.linear_w8(*args), eager)  # eager work between replays
