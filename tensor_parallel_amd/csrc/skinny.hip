@@ -947,6 +947,7 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     // x fragments fill 128 registers: 4 chunks per wavefront (8192 K elements per split) for 16 rows, 2 for 32, 1 for 64
     const int nch = p.M <= 16 ? 4 : p.M <= 32 ? 2 : 1;
     const int splits = (p.K + nch * 2048 - 1) / (nch * 2048);
+    if (splits > cus) return TPAMD_OK;  // K in the millions: not what this kernel is laid out for
     int col_blocks = cus / splits > 0 ? cus / splits : 1;
     int cols_per_block = (p.N + col_blocks - 1) / col_blocks;
     cols_per_block = (cols_per_block + 15) / 16 * 16;
