@@ -854,6 +854,7 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
                     typedef __attribute__((address_space(1))) float global_float;
                     global_float *wsa = (global_float *)(ws + a * 16 * 128);
                     asm volatile("" : "+v"(wsa));  // one address per x tile, the rest are store offsets
+                    if (m128 * 128 + a * 16 + l16 >= p.M) continue;  // the finishing pass reads valid rows only
 #pragma unroll
                     for (int b = 0; b < 8; ++b)
                         // Stored from accumulator registers. The no-ops are the wait states a store of more than 8
@@ -1078,7 +1079,7 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
             for (int b = 0; b < 4; ++b) {
                 const int wr = (MODE == MODE_SWIGLU ? (b >> 1) * 64 + wn * 32 + (b & 1) * 16 : wn * 64 + b * 16) + lq * 4;
                 const int xr = wm * 64 + a * 16 + l16;
-                *reinterpret_cast<f32x4 *>(ws + xr * BN + wr) = acc[a][b];
+                if (m0 + xr < p.M) *reinterpret_cast<f32x4 *>(ws + xr * BN + wr) = acc[a][b];  // the finishing pass reads valid rows only
             }
     } else {
         // the stages are free once every wavefront has read its last fragments: a slab per wavefront at their start
