@@ -1340,8 +1340,8 @@ int configure128(int dev) {
 // fitted (least squares over 290 timings of 48 mid-sized shapes) on this part: a block that has its CU to itself takes
 // 0.82 per K tile, two blocks sharing a CU 0.98 each (the pace of the CU's global->LDS path), 0.92 when blocks queue
 // for several rounds of two per CU; the partial tiles cost 4.6 + 0.39 per MB (written, read back and finished by a
-// second launch).
-inline double estimate128(int64_t tiles, int KT, int cus, int *splits) {
+// second launch; valid_rows = the fraction of the tiles' rows that lie inside M: the others are not stored).
+inline double estimate128(int64_t tiles, int KT, int cus, double valid_rows, int *splits) {
     double best = 1e30;
     *splits = 1;
     for (int sp = 1; sp <= 8; ++sp) {
@@ -1350,7 +1350,7 @@ inline double estimate128(int64_t tiles, int KT, int cus, int *splits) {
         const double units = static_cast<double>(tiles) * sp;
         const double rounds = units <= cus ? 1.0 : static_cast<double>((static_cast<int64_t>(units) + 2 * cus - 1) / (2 * cus));
         const double per_kt = units <= cus ? 0.82 : units <= 2.0 * cus ? 0.98 : 0.92;
-        const double t = rounds * kt * per_kt + (sp > 1 ? 4.6 + units * 0.065536 * 0.39 : 0.0);
+        const double t = rounds * kt * per_kt + (sp > 1 ? 4.6 + units * 0.065536 * valid_rows * 0.39 : 0.0);
         if (t < best) { best = t; *splits = sp; }
     }
     return best;
@@ -1370,7 +1370,7 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     const int KT = p.K / 64;
     int splits = 1;
     if (const char *e = getenv("TPAMD_GEMM_SPLITK")) splits = atoi(e);
-    else estimate128(tiles, KT, cus, &splits);
+    else estimate128(tiles, KT, cus, static_cast<double>(p.M) / (p.tiles_m * 128.0), &splits);
     if (splits > 8) splits = 8;
     if (splits > KT) splits = KT;
     if (splits < 1) splits = 1;
@@ -1424,16 +1424,17 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     // ... or split over K while all units still fit one round; the partial tiles cost 9 us + 0.33 us per MB (more than
     // with the small tiles: all blocks finish together, so nothing overlaps the writes and the finishing pass)
     int splits256 = 1;
+    const double valid256 = static_cast<double>(p.M) / (((p.M + 255) / 256) * 256.0);
     for (int sp = 2; sp <= 8 && big_tiles * sp <= cus; ++sp) {
         const int kt = (KT + sp - 1) / sp;
         if (kt < 4) break;
         const int64_t units = big_tiles * sp;
-        const double t = rounds256(units, kt) + 9.0 + units * 0.262144 * 0.33;
+        const double t = rounds256(units, kt) + 9.0 + units * 0.262144 * valid256 * 0.33;
         if (t < t256) { t256 = t; splits256 = sp; }
     }
     if (const char *e = getenv("TPAMD_GEMM_SPLITK256")) splits256 = atoi(e);
     int unused_splits = 1;
-    const double t128 = estimate128(small_tiles, KT, cus, &unused_splits);
+    const double t128 = estimate128(small_tiles, KT, cus, static_cast<double>(p.M) / (((p.M + 127) / 128) * 128.0), &unused_splits);
     const char *force = getenv("TPAMD_GEMM_TILE");
     const bool big = force ? atoi(force) == 256 : t256 < t128;
     if (direct_ok) {
