@@ -104,6 +104,25 @@ def test_llama_mlp_block_with_llama_rules(world, tokens):
     torch.testing.assert_close(out.float().cpu(), ref, rtol=2e-2, atol=2e-2 * ref.std().item())
 
 
+@pytest.mark.parametrize("tokens", [6, 7])
+def test_llama_mlp_block_at_decode_batch_sizes_of_real_width(tokens):
+    """A Llama-7B-wide MLP (d = 4096, ffn 11008) at W = 2 with 12 and 14 tokens per forward: the sizes at which the
+    library serves the shards' gate/up pair and down projection with its x-resident weight-streaming kernel by
+    default. The two shards' partial sums recombine to the unsplit module."""
+    torch.manual_seed(0)
+    d, f, world = 4096, 11008, 2
+    block = Block(d, f).to(torch.bfloat16)
+    for p in block.parameters():
+        nn.init.normal_(p, std=0.02)
+    x = torch.randn(2, tokens, d).to(torch.bfloat16)
+    cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=d, num_attention_heads=32, num_key_value_heads=32), [DEV] * world)
+    model_tp = tp.TensorParallel(deepcopy(block), [DEV] * world, tensor_parallel_config=cfg, sharded=False)
+    with torch.no_grad():
+        ref = block.to(DEV).float()(x.to(DEV).float())
+        out = model_tp(x.to(DEV))
+    torch.testing.assert_close(out.float(), ref, rtol=2e-2, atol=2e-2 * ref.std().item())
+
+
 def test_opt_125m_tensor_parallel_logits():
     """BASELINE config 1: OPT-125m architecture, fp32, N(0, 0.02) weights from seed 0, W = 2 through
     tp.tensor_parallel, batch 2 x seq 64; final logits against the unsplit model."""
