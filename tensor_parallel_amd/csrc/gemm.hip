@@ -849,6 +849,9 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
             const int m128 = tile_m * 2 + wm, n128 = tile_n * 2 + wn;
             if (m128 < tm128 && n128 < tn128) {
                 float *ws = p.ws + (static_cast<int64_t>(split_now) * tm128 * tn128 + m128 * tn128 + n128) * (128 * 128) + l16 * 128 + lq * 4;
+                // the stores below are asm statements: the compiler does not count the wait states a memory
+                // instruction needs before it may read registers an MFMA has just written
+                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
 #pragma unroll
                 for (int a = 0; a < 8; ++a) {
                     typedef __attribute__((address_space(1))) float global_float;
