@@ -13,13 +13,17 @@
  *   - return value: 0 on success, a negative tpamd_status otherwise; tpamd_last_error() then returns a
  *     message for the calling thread;
  *   - every entry point may be called concurrently from several host threads. Besides the thread-local error
- *     message the library keeps one piece of state: tpamd_linear / tpamd_swiglu_up split K for shapes with few
- *     output tiles (M from 17 to a few thousand, decided by a cost model), tpamd_linear_w8 does so from 12 rows on
- *     large matrices, tpamd_attention splits long key ranges, and they keep one fp32 scratch buffer per
- *     device for that (64 MiB on a 256-CU part), allocated with hipMalloc at first use and kept until the process
- *     ends. Such calls are ordered by their stream; a caller that spreads them over several streams of one device
- *     must order those streams itself. If the first such call happens under stream capture, nothing is allocated
- *     and the call runs unsplit (slower, same result up to summation order).
+ *     message the library keeps one piece of state: tpamd_linear / tpamd_linear_add / tpamd_swiglu_up split K for
+ *     shapes with few output tiles (M from 17 to a few thousand, decided by a cost model), tpamd_linear_w8 does so
+ *     from 12 rows on large matrices, tpamd_attention splits long key ranges, and they keep fp32 scratch buffers for
+ *     the partial results: one per (device, stream), 64 MiB on a 256-CU part, allocated with hipMalloc at the
+ *     stream's first such call and kept until the process ends (at most 8 streams per device get one; calls on
+ *     further streams run unsplit). Streams never share a buffer, so such calls on different streams of a device
+ *     need no ordering among themselves. If a stream's first such call happens under stream capture, nothing is
+ *     allocated and the call runs unsplit (slower, same result up to summation order). A captured graph keeps
+ *     using the buffer of the stream it was captured on: replaying it on another stream while that stream runs
+ *     K-split work is for the caller to order.
+ *   - tuning knobs (environment variables TPAMD_*) are read once, when the library is loaded.
  */
 #ifndef TPAMD_H
 #define TPAMD_H
@@ -31,7 +35,7 @@
 extern "C" {
 #endif
 
-#define TPAMD_ABI_VERSION 1
+#define TPAMD_ABI_VERSION 2
 
 typedef enum tpamd_status {
     TPAMD_OK = 0,
@@ -65,6 +69,12 @@ typedef enum tpamd_act {
 
 int tpamd_abi_version(void);
 const char *tpamd_last_error(void);
+/* Reads the TPAMD_* environment variables again (they are read once at load time otherwise). For tests and
+ * experiments that force a kernel variant; no counterpart in the reference. */
+void tpamd_tuning_reload(void);
+/* The K-split scratch buffer that work on `stream` of the current device uses: *ptr_out = NULL and *bytes_out = 0
+ * while the stream has none. Diagnostic; no counterpart in the reference. */
+int tpamd_scratch_query(void *stream, void **ptr_out, uint64_t *bytes_out);
 
 /* ------------------------------------------------------------------------------------------------
  * Slicing engine.
@@ -143,6 +153,17 @@ int tpamd_reduce_partials(const void *const *parts_dev, int world_size, void *ou
  * ---------------------------------------------------------------------------------------------- */
 int tpamd_linear(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, void *stream);
+
+/* tpamd_linear followed by one step of the partial-sum reduction, in one launch:
+ *   y = round_dtype( round_dtype(act(x . w^T + bias)) + addend ),   addend [M,N] with leading dimension ldadd.
+ * With addend = the running sum of the partials of ranks 0..r-1 and (x, w) = rank r's row-parallel shard this is
+ * `sum([...])` over the rank partials (src/tensor_parallel/cross_device_ops.py:49, reached from AllReduce.__call__,
+ * src/tensor_parallel/communications.py:114-116) taken in rank order, bit for bit: torch adds two same-dtype tensors
+ * as the fp32 sum of the widened values, rounded once. F32: y = (x . w^T + bias) + addend in fp32.
+ * addend_dev may be y_dev (then ldadd must equal ldy): the partial is accumulated in place. */
+int tpamd_linear_add(const void *x_dev, const void *w_dev, const void *bias_dev, const void *addend_dev, void *y_dev,
+                     int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldadd, int64_t ldy, int dtype,
+                     int act, void *stream);
 
 /* h[M,N] = silu(x . wg^T) * (x . wu^T): the gate/up pair of a SiLU-gated MLP shard in one pass over x
  * (two column-parallel torch.nn.Linear calls, a SiLU and a product in the reference's wrapped module;

@@ -25,13 +25,16 @@ EXPORTS = (
     "tpamd_copy_jobs_run",
     "tpamd_scale",
     "tpamd_reduce_partials",
+    "tpamd_tuning_reload",
+    "tpamd_scratch_query",
     "tpamd_linear",
+    "tpamd_linear_add",
     "tpamd_swiglu_up",
     "tpamd_linear_w8",
     "tpamd_attention",
 )
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 BF16, F16, F32 = 0, 1, 2
 ACCUM_STEPWISE, ACCUM_F32 = 0, 1
@@ -82,6 +85,12 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_reduce_partials.argtypes = [c.POINTER(vp), ci, vp, u64, ci, ci, vp]
     lib.tpamd_linear.restype = ci
     lib.tpamd_linear.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
+    lib.tpamd_linear_add.restype = ci
+    lib.tpamd_linear_add.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, ci, ci, vp]
+    lib.tpamd_tuning_reload.restype = None
+    lib.tpamd_tuning_reload.argtypes = []
+    lib.tpamd_scratch_query.restype = ci
+    lib.tpamd_scratch_query.argtypes = [vp, c.POINTER(vp), c.POINTER(u64)]
     lib.tpamd_swiglu_up.restype = ci
     lib.tpamd_swiglu_up.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
     lib.tpamd_attention.restype = ci
@@ -254,30 +263,67 @@ def _ld(t: torch.Tensor) -> int:
     return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, act: int = ACT_NONE) -> torch.Tensor:
-    """y = act(x @ w.T + bias) with w of shape [N, K]; leading dimensions of x are kept."""
+def reload_tuning() -> None:
+    """Make the library read its TPAMD_* environment variables again (it reads them once, at load time)."""
+    lib().tpamd_tuning_reload()
+
+
+def scratch_of_stream(device: torch.device, stream_ptr: Optional[int] = None) -> tuple:
+    """(address, bytes) of the K-split scratch buffer that work on the stream uses, (None, 0) while it has none."""
+    ptr, nbytes = ctypes.c_void_p(), ctypes.c_uint64()
+    with torch.cuda.device(device):
+        if stream_ptr is None:
+            stream_ptr = current_stream_ptr(device)
+        _check(lib().tpamd_scratch_query(ctypes.c_void_p(stream_ptr), ctypes.byref(ptr), ctypes.byref(nbytes)), "tpamd_scratch_query")
+    return ptr.value, int(nbytes.value)
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, act: int = ACT_NONE,
+           addend: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = act(x @ w.T + bias) with w of shape [N, K]; leading dimensions of x are kept. With `addend` (same shape
+    and dtype as y): y = (that result, rounded to the dtype) + addend, one step of the sum over rank partials, in the
+    same launch. `out` (contiguous, may be `addend`) receives the result."""
     require_device(x, "linear")
     require_device(w, "linear")
     if x.dtype != w.dtype:
         raise TypeError(f"linear: x is {x.dtype} but w is {w.dtype}")
-    if x.shape[-1] != w.shape[1]:
-        raise ValueError(f"linear: x has {x.shape[-1]} input features, w expects {w.shape[1]}")
+    if w.dim() != 2 or x.shape[-1] != w.shape[1]:
+        raise ValueError(f"linear: x has {x.shape[-1]} input features, w is {tuple(w.shape)}")
+    if w.device != x.device:
+        raise ValueError(f"linear: x is on {x.device}, w on {w.device}")
     x2, w2 = _as_2d(x), _as_2d(w)
     M, K = x2.shape
     N = w2.shape[0]
-    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if out is None:
+        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    else:
+        if out.dtype != x.dtype or out.device != x.device or out.numel() != M * N or not out.is_contiguous():
+            raise ValueError("linear: out must be a contiguous tensor of the result's size, dtype and device")
+        y = out.view(M, N)
     b = None
     if bias is not None:
         b = bias.contiguous()
-        if b.shape != (N,) or b.dtype != x.dtype:
-            raise ValueError("linear: bias must have shape [N] and the dtype of x")
+        if b.shape != (N,) or b.dtype != x.dtype or b.device != x.device:
+            raise ValueError("linear: bias must have shape [N], the dtype of x and live on its device")
+    a2 = None
+    if addend is not None:
+        if addend.dtype != x.dtype or addend.device != x.device or addend.numel() != M * N or addend.shape[-1] != N:
+            raise ValueError("linear: addend must have the shape, dtype and device of the result")
+        a2 = _as_2d(addend)
     with torch.cuda.device(x.device):
-        _check(
-            lib().tpamd_linear(x2.data_ptr(), w2.data_ptr(), b.data_ptr() if b is not None else None, y.data_ptr(),
-                               M, N, K, _ld(x2), _ld(w2), N, dtype_code(x.dtype), act,
-                               ctypes.c_void_p(current_stream_ptr(x.device))),
-            "tpamd_linear",
-        )
+        stream = ctypes.c_void_p(current_stream_ptr(x.device))
+        if a2 is None:
+            _check(
+                lib().tpamd_linear(x2.data_ptr(), w2.data_ptr(), b.data_ptr() if b is not None else None, y.data_ptr(),
+                                   M, N, K, _ld(x2), _ld(w2), N, dtype_code(x.dtype), act, stream),
+                "tpamd_linear",
+            )
+        else:
+            _check(
+                lib().tpamd_linear_add(x2.data_ptr(), w2.data_ptr(), b.data_ptr() if b is not None else None, a2.data_ptr(),
+                                       y.data_ptr(), M, N, K, _ld(x2), _ld(w2), _ld(a2), N, dtype_code(x.dtype), act, stream),
+                "tpamd_linear_add",
+            )
     return y.view(*x.shape[:-1], N)
 
 
@@ -286,8 +332,10 @@ def swiglu_up(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor) -> torch.Tens
     require_device(x, "swiglu_up")
     if not (x.dtype == wg.dtype == wu.dtype):
         raise TypeError("swiglu_up: x, wg, wu must share one dtype")
-    if wg.shape != wu.shape or x.shape[-1] != wg.shape[1]:
+    if wg.dim() != 2 or wg.shape != wu.shape or x.shape[-1] != wg.shape[1]:
         raise ValueError("swiglu_up: shape mismatch")
+    if wg.device != x.device or wu.device != x.device:
+        raise ValueError(f"swiglu_up: x is on {x.device}, wg on {wg.device}, wu on {wu.device}")
     x2, g2, u2 = _as_2d(x), _as_2d(wg), _as_2d(wu)
     if _ld(g2) != _ld(u2):
         u2 = u2.contiguous()
@@ -313,6 +361,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional
         raise TypeError("attention: q, k, v must share bfloat16 or float16")
     if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
         raise ValueError(f"attention: shapes q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit")
+    if k.device != q.device or v.device != q.device:
+        raise ValueError(f"attention: q is on {q.device}, k on {k.device}, v on {v.device}")
     B, Hq, Sq, D = q.shape
     Hkv, Skv = k.shape[1], k.shape[2]
     q, k, v = (t if t.stride(3) == 1 else t.contiguous() for t in (q, k, v))
@@ -335,14 +385,27 @@ def linear_w8(x: torch.Tensor, wq: torch.Tensor, scale_: torch.Tensor, outlier_i
     require_device(x, "linear_w8")
     if wq.dtype != torch.int8 or scale_.dtype != torch.float32:
         raise TypeError("linear_w8: wq must be int8 and scale float32")
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"linear_w8: x must be bfloat16 or float16, got {x.dtype}")
     x2 = _as_2d(x)
-    wq = wq.contiguous()
     M, K = x2.shape
+    if wq.dim() != 2 or wq.shape[1] != K:
+        raise ValueError(f"linear_w8: x has {K} input features, wq is {tuple(wq.shape)}")
     N = wq.shape[0]
+    if scale_.shape != (N,):
+        raise ValueError(f"linear_w8: scale must have shape [{N}], got {tuple(scale_.shape)}")
+    for name, t in (("wq", wq), ("scale", scale_), ("outlier_idx", outlier_idx), ("w_out", w_out), ("bias", bias)):
+        if t is not None and t.device != x.device:
+            raise ValueError(f"linear_w8: x is on {x.device}, {name} on {t.device}")
+    if bias is not None and (bias.shape != (N,) or bias.dtype != x.dtype):
+        raise ValueError("linear_w8: bias must have shape [N] and the dtype of x")
+    wq = wq.contiguous()
     n_out = 0 if outlier_idx is None else int(outlier_idx.numel())
     if n_out:
         if outlier_idx.dtype != torch.int32 or w_out is None or w_out.shape != (N, n_out) or w_out.dtype != x.dtype:
             raise ValueError("linear_w8: outlier_idx must be int32 [n_out] and w_out [N, n_out] in the dtype of x")
+        if n_out > K:
+            raise ValueError(f"linear_w8: {n_out} outlier columns for K = {K}")
         w_out = w_out.contiguous()
         outlier_idx = outlier_idx.contiguous()
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)

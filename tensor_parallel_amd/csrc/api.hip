@@ -14,11 +14,12 @@ void set_error(const char *fmt, ...) {
     va_end(ap);
 }
 
-int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias, void *y, int64_t M, int64_t N,
-                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu, bool generic, hipStream_t s);
-int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *scale,
-                    const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N, int64_t K,
-                    int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
+int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *addend, int64_t ldadd, void *y,
+                  int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu,
+                  bool generic, hipStream_t s);
+int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *addend, int64_t ldadd,
+                    const void *scale, const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
                     hipStream_t s);
 
 int attention_dispatch(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq,
@@ -59,18 +60,36 @@ using namespace tpamd;
 extern "C" int tpamd_abi_version(void) { return TPAMD_ABI_VERSION; }
 extern "C" const char *tpamd_last_error(void) { return g_err; }
 
+// y = act(x . w^T + bias), then, with an addend, y = round(y + addend) in the tensor dtype.
+int tpamd::linear_entry(const char *who, const void *x_dev, const void *w_dev, const void *bias_dev, const void *addend_dev,
+                        int64_t ldadd, void *y_dev, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy,
+                        int dtype, int act, void *stream) {
+    int rc = check_common(who, x_dev, w_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype);
+    if (rc != TPAMD_OK) return rc;
+    TPAMD_REQUIRE(act == TPAMD_ACT_NONE || act == TPAMD_ACT_GELU, "%s: unknown activation %d", who, act);
+    if (M == 0 || N == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(addend_dev == nullptr || ldadd >= N, "%s: ldadd=%lld is smaller than N=%lld", who, (long long)ldadd, (long long)N);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, w_dev, nullptr, bias_dev, y_dev, N, K, ldx, ldw, ldy) &&
+                      (addend_dev == nullptr || (aligned(addend_dev, 8) && ldadd % 4 == 0));
+    if (fast && M <= SKINNY_MAX_M)
+        return skinny_dispatch(x_dev, w_dev, nullptr, bias_dev, addend_dev, ldadd, nullptr, nullptr, nullptr, 0, y_dev, M, N, K,
+                               ldx, ldw, ldy, 0, dtype, act, false, false, s);
+    return gemm_dispatch(x_dev, w_dev, nullptr, bias_dev, addend_dev, ldadd, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, false,
+                         !fast, s);
+}
+
 extern "C" int tpamd_linear(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
                             int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, void *stream) {
-    int rc = check_common("tpamd_linear", x_dev, w_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype);
-    if (rc != TPAMD_OK) return rc;
-    TPAMD_REQUIRE(act == TPAMD_ACT_NONE || act == TPAMD_ACT_GELU, "tpamd_linear: unknown activation %d", act);
-    if (M == 0 || N == 0) return TPAMD_OK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, w_dev, nullptr, bias_dev, y_dev, N, K, ldx, ldw, ldy);
-    if (fast && M <= SKINNY_MAX_M)
-        return skinny_dispatch(x_dev, w_dev, nullptr, bias_dev, nullptr, nullptr, nullptr, 0, y_dev, M, N, K, ldx, ldw, ldy, 0,
-                               dtype, act, false, false, s);
-    return gemm_dispatch(x_dev, w_dev, nullptr, bias_dev, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, false, !fast, s);
+    return linear_entry("tpamd_linear", x_dev, w_dev, bias_dev, nullptr, 0, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, stream);
+}
+
+extern "C" int tpamd_linear_add(const void *x_dev, const void *w_dev, const void *bias_dev, const void *addend_dev, void *y_dev,
+                                int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldadd, int64_t ldy, int dtype,
+                                int act, void *stream) {
+    TPAMD_REQUIRE(addend_dev != nullptr || M == 0 || N == 0, "tpamd_linear_add: addend is NULL");
+    return linear_entry("tpamd_linear_add", x_dev, w_dev, bias_dev, addend_dev, ldadd, y_dev, M, N, K, ldx, ldw, ldy, dtype, act,
+                        stream);
 }
 
 extern "C" int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void *wu_dev, void *h_dev, int64_t M, int64_t N,
@@ -82,9 +101,10 @@ extern "C" int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, wg_dev, wu_dev, nullptr, h_dev, N, K, ldx, ldw, ldh);
     if (fast && M <= SKINNY_MAX_M)
-        return skinny_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw, ldh, 0,
-                               dtype, TPAMD_ACT_NONE, true, false, s);
-    return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true, !fast, s);
+        return skinny_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw,
+                               ldh, 0, dtype, TPAMD_ACT_NONE, true, false, s);
+    return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true,
+                         !fast, s);
 }
 
 extern "C" int tpamd_attention(const void *q_dev, const void *k_dev, const void *v_dev, void *out_dev, int64_t B, int64_t Hq,
@@ -131,7 +151,7 @@ extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void
     const int esz = 2;
     for (int64_t m0 = 0; m0 < M; m0 += SKINNY_W8_SLAB) {  // weights are re-streamed once per slab of 64 rows
         const int64_t mm = M - m0 < SKINNY_W8_SLAB ? M - m0 : SKINNY_W8_SLAB;
-        int rc = skinny_dispatch(static_cast<const char *>(x_dev) + m0 * ldx * esz, wq_dev, nullptr, bias_dev, scale_dev,
+        int rc = skinny_dispatch(static_cast<const char *>(x_dev) + m0 * ldx * esz, wq_dev, nullptr, bias_dev, nullptr, 0, scale_dev,
                                  outlier_idx_dev, w_out_dev, n_out, static_cast<char *>(y_dev) + m0 * ldy * esz, mm, N, K, ldx,
                                  ldw, ldy, ld_wout, dtype, act, false, true, s);
         if (rc != TPAMD_OK) return rc;

@@ -322,7 +322,7 @@ int launch(AttnParams p, int cus, hipStream_t s) {
         if (nsplit > 64) nsplit = 64;
         if (nsplit < 1) nsplit = 1;
     }
-    if (const char *e = getenv("TPAMD_ATTN_SPLITS")) nsplit = atoi(e) > 0 ? atoi(e) : 1;
+    if (tuning().attn_splits != TUNE_UNSET) nsplit = tuning().attn_splits > 0 ? tuning().attn_splits : 1;
     p.keys_per_split = ((p.Skv + nsplit - 1) / nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
     nsplit = (p.Skv + p.keys_per_split - 1) / p.keys_per_split;
     p.nsplit = nsplit;
@@ -364,7 +364,7 @@ int attention_dispatch(const void *q, const void *k, const void *v, void *o, int
                        int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal, int dtype, hipStream_t s) {
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
-    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
     AttnParams p{};
     p.q = static_cast<const char *>(q);
     p.k = static_cast<const char *>(k);

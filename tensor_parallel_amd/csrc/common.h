@@ -33,11 +33,38 @@ void set_error(const char *fmt, ...);
         }                                                                                        \
     } while (0)
 
-// The per-device fp32 scratch buffer (split-K partial tiles, split-KV attention partials): defined in gemm.hip.
-// Callers hold splitk_mutex() from the lookup until their launches that use the buffer are enqueued and pass
-// reserve = 4 * CUs * 64 KiB, so that whoever comes first allocates the size everybody can live with.
+// ---- tuning knobs: environment variables, read once when the library is loaded (tpamd_tuning_reload() re-reads them).
+// TUNE_UNSET = the variable is not set and the library's own choice applies.
+constexpr int TUNE_UNSET = -2147483647 - 1;
+struct Tuning {
+    int gemm_w4;             // TPAMD_GEMM_W4: 0 = the 8-wavefront 256 x 256 kernel instead of the 4-wavefront one
+    int gemm_splitk;         // TPAMD_GEMM_SPLITK: K splits of the 128 x 128 tiling
+    int gemm_splitk256;      // TPAMD_GEMM_SPLITK256: K splits of the 256 x 256 tiling
+    int gemm_tile;           // TPAMD_GEMM_TILE: 256 or 128
+    int gemm_balance;        // TPAMD_GEMM_BALANCE: 0 = never split the tiles of a last, partly filled round over K
+    int skinny_cg;           // TPAMD_SKINNY_CG: column groups per block (1, 2, 4)
+    int skinny_pair;         // TPAMD_SKINNY_PAIR: 8-column form of the gated pair
+    int skinny_resident;     // TPAMD_SKINNY_RESIDENT: x-resident kernel on/off
+    int gemv_persistent;     // TPAMD_GEMV_PERSISTENT: 0 = one block per group of rows instead of the persistent grid
+    int w8_split;            // TPAMD_W8_SPLIT: int8 K-split kernel on/off
+    int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel
+    int copy_tile_units;     // TPAMD_COPY_TILE_UNITS: 16-byte units per copy tile
+    int copy_blocks_per_cu;  // TPAMD_COPY_BLOCKS_PER_CU
+};
+const Tuning &tuning();
+
+// Compute units of device `dev` (asked from the runtime once per device).
+int device_cus(int dev, int *cus_out);
+
+// fp32 scratch memory of the K-split kernels (split-K partial tiles, split-key attention partials): defined in
+// runtime.hip. Callers hold splitk_mutex() from the lookup until their launches that use the buffer are enqueued
+// and pass reserve = 4 * CUs * 64 KiB, so that a stream's buffer is allocated with the size every shape can live with.
 std::mutex &splitk_mutex();
 int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out);
+// Body of tpamd_linear / tpamd_linear_add (api.hip).
+int linear_entry(const char *who, const void *x_dev, const void *w_dev, const void *bias_dev, const void *addend_dev,
+                 int64_t ldadd, void *y_dev, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype,
+                 int act, void *stream);
 
 static inline bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
@@ -105,6 +132,14 @@ template <int DT>
 __device__ __forceinline__ float hi_half_to_f32(uint32_t p) {
     if constexpr (DT == TPAMD_BF16) return __uint_as_float(p & 0xffff0000u);
     else return half_to_f32<DT>(static_cast<uint16_t>(p >> 16));
+}
+
+// out = round(out + addend) per 16-bit element: the sum of two same-dtype tensors as torch computes it (fp32 add of the
+// widened values, one rounding), which is one step of the reference's `sum([...])` over rank partials
+// (src/tensor_parallel/cross_device_ops.py:49).
+template <int DT>
+__device__ __forceinline__ uint32_t add_packed2(uint32_t a, uint32_t b) {
+    return pack2_half<DT>(lo_half_to_f32<DT>(a) + lo_half_to_f32<DT>(b), hi_half_to_f32<DT>(a) + hi_half_to_f32<DT>(b));
 }
 
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }

@@ -35,9 +35,10 @@ struct GemmParams {
     const char *w;   // linear: weight; swiglu: gate weight
     const char *w2;  // swiglu: up weight
     const char *bias;
+    const char *addend;  // linear: added to the rounded result (another rank's partial sum), or NULL
     char *y;
     int M, N, K;
-    int64_t ldx, ldw, ldy;  // elements
+    int64_t ldx, ldw, ldy, ldadd;  // elements
     int act;
     int tiles_m, tiles_n;
     float *ws;          // split-K: partial tiles, [split][tile][128 x rows][128 w rows] fp32
@@ -126,6 +127,11 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, f32x16 (&acc)[TM][
                     uint2 o;
                     o.x = h[0] | (static_cast<uint32_t>(h[1]) << 16);
                     o.y = h[2] | (static_cast<uint32_t>(h[3]) << 16);
+                    if (p.addend != nullptr) {
+                        const uint2 araw = *reinterpret_cast<const uint2 *>(p.addend + (static_cast<int64_t>(m) * p.ldadd + n) * 2);
+                        o.x = add_packed2<DT>(o.x, araw.x);
+                        o.y = add_packed2<DT>(o.y, araw.y);
+                    }
                     *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = o;
                 }
             }
@@ -296,7 +302,7 @@ __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
 // Four consecutive output columns n..n+3 of one row, from fp32 sums to the packed 16-bit store value.
 // linear: v = bias/activation of g; swiglu: g = gate sums, u = up sums.
 template <int DT, int MODE>
-__device__ __forceinline__ uint2 finish4(const GemmParams &p, const float (&g)[4], const float (&u)[4], int n) {
+__device__ __forceinline__ uint2 finish4(const GemmParams &p, const float (&g)[4], const float (&u)[4], int n, const char *add_row = nullptr) {
     uint2 o;
     if constexpr (MODE == MODE_SWIGLU) {
         // gate and up products rounded to the tensor dtype, then silu and the product each rounded again
@@ -325,6 +331,11 @@ __device__ __forceinline__ uint2 finish4(const GemmParams &p, const float (&g)[4
         }
         o.x = pack2_half<DT>(v[0], v[1]);
         o.y = pack2_half<DT>(v[2], v[3]);
+        if (add_row != nullptr) {  // the row of p.addend this output row belongs to
+            const uint2 araw = *reinterpret_cast<const uint2 *>(add_row + static_cast<int64_t>(n) * 2);
+            o.x = add_packed2<DT>(o.x, araw.x);
+            o.y = add_packed2<DT>(o.y, araw.y);
+        }
     }
     return o;
 }
@@ -349,7 +360,8 @@ __device__ __forceinline__ void epilogue16(const GemmParams &p, f32x4 (&acc)[TMX
                 g[j] = acc[a][b][j];
                 u[j] = MODE == MODE_SWIGLU ? acc[a][(b + 2) & 3][j] : 0.f;
             }
-            *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = finish4<DT, MODE>(p, g, u, n);
+            const char *add_row = MODE == MODE_LINEAR && p.addend != nullptr ? p.addend + static_cast<int64_t>(m) * p.ldadd * 2 : nullptr;
+            *reinterpret_cast<uint2 *>(yrow + static_cast<int64_t>(n) * 2) = finish4<DT, MODE>(p, g, u, n, add_row);
         }
     }
 }
@@ -413,14 +425,21 @@ __device__ __forceinline__ void staged_epilogue(const GemmParams &p, f32x4 (&acc
 #pragma unroll
             for (int h = 0; h < 16 / ROWS_PER_READ; ++h) {
                 const int row = h * ROWS_PER_READ + rd_row;
-                const uint4 v = *reinterpret_cast<const uint4 *>(slab + row * EP_PITCH + rd_col * 16);
+                const uint4 vs = *reinterpret_cast<const uint4 *>(slab + row * EP_PITCH + rd_col * 16);
                 const int m = m_wave + a * 16 + row;
                 const int n = n_wave + gq * (16 * GB) + rd_col * 8;
-#ifdef T4_ABL_NOSTORE  // timing build only (wrong results): everything but the global stores
-                if (p.act != 12345) continue;
-#endif
                 if (m >= p.M || n >= p.N) continue;
                 char *dst = p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2;
+                uint4 v = vs;
+                if constexpr (MODE == MODE_LINEAR) {
+                    if (p.addend != nullptr) {  // the lane that stores 8 outputs adds the same 8 elements of the addend
+                        const char *ap = p.addend + (static_cast<int64_t>(m) * p.ldadd + n) * 2;
+                        const uint2 a0 = *reinterpret_cast<const uint2 *>(ap);
+                        const uint2 a1 = n + 8 <= p.N ? *reinterpret_cast<const uint2 *>(ap + 8) : make_uint2(0, 0);
+                        v.x = add_packed2<DT>(v.x, a0.x); v.y = add_packed2<DT>(v.y, a0.y);
+                        v.z = add_packed2<DT>(v.z, a1.x); v.w = add_packed2<DT>(v.w, a1.y);
+                    }
+                }
                 if (n + 8 <= p.N) {
                     if (wide) *reinterpret_cast<uint4 *>(dst) = v;
                     else {
@@ -779,16 +798,7 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         T4_PAIR(CUR, 7, 0); T4_PAIR(CUR, 7, 2); L14; T4_SB; T4_PAIR(CUR, 7, 4); T4_PAIR(CUR, 7, 6); L15; T4_SB;     \
     }
 #define T4_NOP (void)0
-    // T4_ABL_*: timing builds only (wrong results), to price the wait for the loads, the barrier, or both
-#if defined(T4_ABL_NOVM)
-#define T4_TILE_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
-#elif defined(T4_ABL_NOBAR)
-#define T4_TILE_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory")
-#elif defined(T4_ABL_NOSYNC)
-#define T4_TILE_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
-#else
 #define T4_TILE_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
-#endif
     // one K tile; kload = K tile (of the load context) fetched into the stage this one leaves
 #define T4_KTILE(kload)                                                                                             \
     {                                                                                                               \
@@ -871,9 +881,6 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
         // epilogue: acc[a][b], b = w tile; gated pair: tiles 0-3 gate, 4-7 up
         const int m_wave = tile_m * BM + wm * 128;
         const int n_wave = tile_n * BN_OUT + (MODE == MODE_SWIGLU ? wn * 64 : wn * 128);
-#ifdef T4_ABL_NOEPI  // timing build only (wrong results): no epilogue at all
-        if (p.act != 12345) continue;
-#endif
         if constexpr (MODE == MODE_SWIGLU) {
             staged_epilogue<DT, MODE, false, 8, 8, 1, 4, 4>(p, acc, ep_slab, m_wave, n_wave, lane, wide_stores);
         } else {
@@ -1128,7 +1135,8 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmParams p, int sp
                 for (int i = 0; i < 4; ++i) u[i] += uv[i];
             }
         }
-        *reinterpret_cast<uint2 *>(p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2) = finish4<DT, MODE>(p, g, u, n);
+        const char *add_row = MODE == MODE_LINEAR && p.addend != nullptr ? p.addend + static_cast<int64_t>(m) * p.ldadd * 2 : nullptr;
+        *reinterpret_cast<uint2 *>(p.y + (static_cast<int64_t>(m) * p.ldy + n) * 2) = finish4<DT, MODE>(p, g, u, n, add_row);
     }
 }
 
@@ -1206,6 +1214,10 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmParams p) {
             } else {
                 v = acc[0][i][j] + (p.bias ? load_elem<DT>(p.bias, n) : 0.f);
                 if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
+                if (p.addend != nullptr) {  // round to the tensor dtype first, as a separate sum of two tensors would
+                    if constexpr (DT != TPAMD_F32) v = half_to_f32<DT>(f32_to_half<DT>(v));
+                    v += load_elem<DT>(p.addend, static_cast<int64_t>(m) * p.ldadd + n);
+                }
             }
             store_elem<DT>(p.y, static_cast<int64_t>(m) * p.ldy + n, v);
         }
@@ -1236,45 +1248,12 @@ int launch_gemm(GemmParams p, hipStream_t s) {
 
 }  // namespace
 
-// Split-K scratch: one buffer per device, allocated at first use with room for any split this file chooses, kept
-// until the process ends. Work on one stream is ordered, so consecutive calls can share it (callers that spread
-// such GEMMs over several streams of one device have to order those streams themselves); the mutex keeps the two
-// launches of a call together when several host threads enqueue onto one stream. *out stays NULL when there is no
-// buffer yet and the stream is being captured (allocating is not allowed then): the caller runs unsplit.
-std::mutex &splitk_mutex() {
-    static std::mutex m;
-    return m;
-}
-int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
-    struct Entry { int dev; void *ptr; size_t bytes; };
-    static std::vector<Entry> cache;  // guarded by splitk_mutex(), held by the caller
-    *out = nullptr;
-    for (Entry &e : cache)
-        if (e.dev == dev) {
-            if (e.bytes >= need) *out = e.ptr;  // `reserve` covers every shape; a larger need runs unsplit
-            return TPAMD_OK;
-        }
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    TPAMD_HIP(hipStreamIsCapturing(stream, &capturing));
-    if (capturing != hipStreamCaptureStatusNone) return TPAMD_OK;
-    const size_t bytes = need > reserve ? need : reserve;
-    void *ptr = nullptr;
-    TPAMD_HIP(hipMalloc(&ptr, bytes));
-    cache.push_back(Entry{dev, ptr, bytes});
-    *out = ptr;
-    return TPAMD_OK;
-}
-
 namespace {
 
 template <int DT, int MODE>
 int launch_direct(GemmParams p, int cus, int splits, hipStream_t s) {
     constexpr int LDS = 2 * 64 * 1152 + 4 * 16 * 144;  // two stages + the 4-wavefront kernel's epilogue slabs
-    const char *w4 = getenv("TPAMD_GEMM_W4");
-#ifndef TPAMD_W4_DEFAULT
-#define TPAMD_W4_DEFAULT 1
-#endif
-    const bool four = (w4 != nullptr ? atoi(w4) != 0 : TPAMD_W4_DEFAULT != 0) && p.K >= 128;
+    const bool four = tuning().gemm_w4 != 0 && p.K >= 128;  // unset: the 4-wavefront kernel
     auto kern = four ? gemm_direct4_kernel<DT, MODE, false> : gemm_direct_kernel<DT, MODE>;
     static thread_local int configured_dev = -1;
     int dev = 0;
@@ -1372,7 +1351,7 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
     const int KT = p.K / 64;
     int splits = 1;
-    if (const char *e = getenv("TPAMD_GEMM_SPLITK")) splits = atoi(e);
+    if (tuning().gemm_splitk != TUNE_UNSET) splits = tuning().gemm_splitk;
     else estimate128(tiles, KT, cus, static_cast<double>(p.M) / (p.tiles_m * 128.0), &splits);
     if (splits > 8) splits = 8;
     if (splits > KT) splits = KT;
@@ -1410,7 +1389,7 @@ template <int DT>
 int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
-    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
     // the direct kernels address a tile with 32-bit byte offsets from the tile origin and step K in tiles of 64
     const bool direct_ok = p.K % 64 == 0 && p.K >= 64 && p.ldx < (1ll << 22) && p.ldw < (1ll << 22);
     // 256 x 256 tiles or 128 x 128 tiles (with K split): whichever the cost models predict to be faster. The 256 tiles
@@ -1435,11 +1414,10 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
         const double t = rounds256(units, kt) + 9.0 + units * 0.262144 * valid256 * 0.33;
         if (t < t256) { t256 = t; splits256 = sp; }
     }
-    if (const char *e = getenv("TPAMD_GEMM_SPLITK256")) splits256 = atoi(e);
+    if (tuning().gemm_splitk256 != TUNE_UNSET) splits256 = tuning().gemm_splitk256;
     int unused_splits = 1;
     const double t128 = estimate128(small_tiles, KT, cus, static_cast<double>(p.M) / (((p.M + 127) / 128) * 128.0), &unused_splits);
-    const char *force = getenv("TPAMD_GEMM_TILE");
-    const bool big = force ? atoi(force) == 256 : t256 < t128;
+    const bool big = tuning().gemm_tile != TUNE_UNSET ? tuning().gemm_tile == 256 : t256 < t128;
     if (direct_ok) {
         if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, splits256, s) : launch_direct<DT, MODE_LINEAR>(p, cus, splits256, s);
         return swiglu ? launch_direct128<DT, MODE_SWIGLU>(p, cus, s) : launch_direct128<DT, MODE_LINEAR>(p, cus, s);
@@ -1463,16 +1441,18 @@ int generic_dispatch(const GemmParams &p, int dtype, bool swiglu, hipStream_t s)
     return dtype == TPAMD_BF16 ? launch_generic<TPAMD_BF16>(p, swiglu, s) : launch_generic<TPAMD_F16>(p, swiglu, s);
 }
 
-int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias, void *y, int64_t M, int64_t N,
-                  int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu, bool generic, hipStream_t s) {
+int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *addend, int64_t ldadd, void *y,
+                  int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, bool swiglu,
+                  bool generic, hipStream_t s) {
     GemmParams p{};
     p.x = static_cast<const char *>(x);
     p.w = static_cast<const char *>(w);
     p.w2 = static_cast<const char *>(w2);
     p.bias = static_cast<const char *>(bias);
+    p.addend = static_cast<const char *>(addend);
     p.y = static_cast<char *>(y);
     p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
-    p.ldx = ldx; p.ldw = ldw; p.ldy = ldy;
+    p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ldadd = ldadd;
     p.act = act;
     if (dtype == TPAMD_F32 || generic) return generic_dispatch(p, dtype, swiglu, s);
     return dtype == TPAMD_BF16 ? gemm_large<TPAMD_BF16>(p, swiglu, s) : gemm_large<TPAMD_F16>(p, swiglu, s);

@@ -119,7 +119,7 @@ extern "C" int tpamd_reduce_partials(const void *const *parts_dev, int world_siz
     TPAMD_REQUIRE(aligned(out_dev, 16), "tpamd_reduce_partials: out not 16-byte aligned");
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
-    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // the tail handler needs at least (EPV - 1) threads in the grid: always true (grid >= 1 block of 256)
     if (dtype == TPAMD_F32) launch<TPAMD_F32, TPAMD_ACCUM_F32>(parts, world_size, out_dev, n_elems, s, cus);

@@ -1,0 +1,133 @@
+// Host-side state of the library: tuning knobs (read from the environment once), the number of compute units per
+// device, and the fp32 scratch memory that the K-split kernels (16-bit and int8 Linears, split-key attention) put their
+// partial results in: one buffer per (device, stream).
+#include "common.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+namespace tpamd {
+
+// ---- tuning knobs -----------------------------------------------------------------------------------
+namespace {
+
+int env_int(const char *name) {
+    const char *e = getenv(name);
+    return e != nullptr && *e != '\0' ? atoi(e) : TUNE_UNSET;
+}
+
+Tuning read_tuning() {
+    Tuning t;
+    t.gemm_w4 = env_int("TPAMD_GEMM_W4");
+    t.gemm_splitk = env_int("TPAMD_GEMM_SPLITK");
+    t.gemm_splitk256 = env_int("TPAMD_GEMM_SPLITK256");
+    t.gemm_tile = env_int("TPAMD_GEMM_TILE");
+    t.gemm_balance = env_int("TPAMD_GEMM_BALANCE");
+    t.skinny_cg = env_int("TPAMD_SKINNY_CG");
+    t.skinny_pair = env_int("TPAMD_SKINNY_PAIR");
+    t.skinny_resident = env_int("TPAMD_SKINNY_RESIDENT");
+    t.gemv_persistent = env_int("TPAMD_GEMV_PERSISTENT");
+    t.w8_split = env_int("TPAMD_W8_SPLIT");
+    t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
+    t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");
+    t.copy_blocks_per_cu = env_int("TPAMD_COPY_BLOCKS_PER_CU");
+    return t;
+}
+
+Tuning g_tuning = read_tuning();  // before any entry point can run: the library's load time
+
+}  // namespace
+
+const Tuning &tuning() { return g_tuning; }
+
+// ---- compute units per device -------------------------------------------------------------------------
+int device_cus(int dev, int *cus_out) {
+    constexpr int MAX_DEV = 64;
+    static int cached[MAX_DEV];  // 0 = not asked yet; written once per device with the same value by whoever asks first
+    if (dev >= 0 && dev < MAX_DEV && cached[dev] > 0) {
+        *cus_out = cached[dev];
+        return TPAMD_OK;
+    }
+    int cus = 0;
+    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (cus <= 0) cus = 1;
+    if (dev >= 0 && dev < MAX_DEV) cached[dev] = cus;
+    *cus_out = cus;
+    return TPAMD_OK;
+}
+
+// ---- scratch memory -------------------------------------------------------------------------------------
+namespace {
+
+struct Entry {
+    int dev;
+    hipStream_t stream;
+    void *ptr;
+    size_t bytes;
+};
+std::vector<Entry> g_cache;  // guarded by splitk_mutex()
+constexpr int MAX_BUFFERS_PER_DEVICE = 8;
+
+}  // namespace
+
+std::mutex &splitk_mutex() {
+    static std::mutex m;
+    return m;
+}
+
+// The caller holds splitk_mutex() from this call until its launches that use the buffer are enqueued.
+// *out = a buffer of at least `need` bytes for work on `stream` of device `dev` (the current device), or NULL: then the
+// caller runs its unsplit form. A stream's buffer is allocated at its first use with max(need, reserve) bytes and kept
+// until the process ends; streams of one device never share one, so K-split work on different streams cannot meet in
+// it. NULL comes back when the stream has no buffer yet and is being captured (allocating is not allowed then), when
+// `need` is larger than the stream's buffer, and for the ninth stream of a device.
+int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
+    *out = nullptr;
+    int on_device = 0;
+    for (Entry &e : g_cache) {
+        if (e.dev != dev) continue;
+        ++on_device;
+        if (e.stream == stream) {
+            if (e.bytes >= need) *out = e.ptr;
+            return TPAMD_OK;
+        }
+    }
+    if (on_device >= MAX_BUFFERS_PER_DEVICE) return TPAMD_OK;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    TPAMD_HIP(hipStreamIsCapturing(stream, &capturing));
+    if (capturing != hipStreamCaptureStatusNone) return TPAMD_OK;
+    const size_t bytes = need > reserve ? need : reserve;
+    void *ptr = nullptr;
+    const hipError_t e = hipMalloc(&ptr, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("hipMalloc of %zu bytes of K-split scratch memory failed: %s", bytes, hipGetErrorString(e));
+        return TPAMD_ERR_NOMEM;
+    }
+    g_cache.push_back(Entry{dev, stream, ptr, bytes});
+    *out = ptr;
+    return TPAMD_OK;
+}
+
+}  // namespace tpamd
+
+using namespace tpamd;
+
+extern "C" void tpamd_tuning_reload(void) { g_tuning = read_tuning(); }
+
+extern "C" int tpamd_scratch_query(void *stream, void **ptr_out, uint64_t *bytes_out) {
+    TPAMD_REQUIRE(ptr_out != nullptr && bytes_out != nullptr, "tpamd_scratch_query: null output pointer");
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    *ptr_out = nullptr;
+    *bytes_out = 0;
+    std::lock_guard<std::mutex> hold(splitk_mutex());
+    for (const Entry &e : g_cache)
+        if (e.dev == dev && e.stream == static_cast<hipStream_t>(stream)) {
+            *ptr_out = e.ptr;
+            *bytes_out = e.bytes;
+        }
+    return TPAMD_OK;
+}

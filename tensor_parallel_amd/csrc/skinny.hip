@@ -38,10 +38,11 @@ struct SkinnyParams {
     const float *scale;        // int8 path: per output row
     const int *outlier_idx;    // int8 path
     const char *w_out;         // int8 path: [N, n_out] in activation dtype
+    const char *addend;        // linear: added to the rounded result, or NULL
     char *y;
     int M, N, K;
     int n_out;
-    int64_t ldx, ldw, ldy, ld_wout;
+    int64_t ldx, ldw, ldy, ld_wout, ldadd;
     int act;
 };
 
@@ -91,6 +92,8 @@ __device__ __forceinline__ void skinny_store_output(const SkinnyParams &p, float
         if (p.bias) v += half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.bias)[n]);
         if (p.act == TPAMD_ACT_GELU) v = gelu_erf(v);
         out = f32_to_half<DT>(v);
+        if (p.addend != nullptr)  // one step of the sum over rank partials: both operands in the tensor dtype
+            out = f32_to_half<DT>(half_to_f32<DT>(out) + half_to_f32<DT>(reinterpret_cast<const uint16_t *>(p.addend)[static_cast<int64_t>(m) * p.ldadd + n]));
     }
     reinterpret_cast<uint16_t *>(p.y)[static_cast<int64_t>(m) * p.ldy + n] = out;
 }
@@ -871,7 +874,7 @@ int launch_gemv(const SkinnyParams &p, hipStream_t s) {
 
 // Column groups per block: as many as keep at least one block per CU and divide N; they pay once x outweighs w.
 inline int pick_cg(const SkinnyParams &p, bool w8, bool swiglu) {
-    if (const char *e = getenv("TPAMD_SKINNY_CG")) return atoi(e) == 4 ? 4 : atoi(e) == 2 ? 2 : 1;
+    if (const int v = tuning().skinny_cg; v != TUNE_UNSET) return v == 4 ? 4 : v == 2 ? 2 : 1;
     if (p.M < (w8 ? 4 : 12)) return 1;  // measured: below this the prefetching single-group kernel is faster
     if (!swiglu && p.N % 64 == 0 && p.N / 64 >= 256) return 4;
     if (p.N % 32 == 0 && p.N / 32 >= 256) return 2;
@@ -881,7 +884,7 @@ inline int pick_cg(const SkinnyParams &p, bool w8, bool swiglu) {
 // Gated pair with 16-bit weights and at most 32 rows: the 8-column form (measured 5-12 % faster than the
 // 16-column forms at every M from 4 to 32 on the Llama-7B shard shapes).
 inline bool pick_pair(const SkinnyParams &p) {
-    if (const char *e = getenv("TPAMD_SKINNY_PAIR")) return atoi(e) != 0;
+    if (tuning().skinny_pair != TUNE_UNSET) return tuning().skinny_pair != 0;
     return p.M <= 32;
 }
 
@@ -894,7 +897,7 @@ inline bool pick_pair(const SkinnyParams &p) {
 template <int MODE>
 inline bool pick_resident(const SkinnyParams &p, int cus) {
     if (p.M > 16 || p.K > 8192) return false;
-    if (const char *e = getenv("TPAMD_SKINNY_RESIDENT")) return atoi(e) != 0;
+    if (tuning().skinny_resident != TUNE_UNSET) return tuning().skinny_resident != 0;
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     if (p.K < 3072) return false;
     if (p.K > 6144) {
@@ -929,8 +932,8 @@ int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
 template <int DT>
 int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     *done = false;
-    if (const char *e = getenv("TPAMD_W8_SPLIT")) {
-        if (atoi(e) == 0) return TPAMD_OK;
+    if (tuning().w8_split != TUNE_UNSET) {
+        if (tuning().w8_split == 0) return TPAMD_OK;
     } else {
         // Measured (Falcon-40B MLP shard, 16384 x 8192 and 8192 x 16384, and smaller matrices): from 25 rows on it
         // always pays (32 rows: 57 -> 47 us and 79 -> 49 us, 64 rows: 114 -> 72 us and 156 -> 73 us), from 17 rows
@@ -943,7 +946,7 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     if (p.K < 4096 || p.n_out > 256 || p.M > 64) return TPAMD_OK;
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
-    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
     // x fragments fill 128 registers: 4 chunks per wavefront (8192 K elements per split) for 16 rows, 2 for 32, 1 for 64
     const int nch = p.M <= 16 ? 4 : p.M <= 32 ? 2 : 1;
     const int splits = (p.K + nch * 2048 - 1) / (nch * 2048);
@@ -989,7 +992,7 @@ int launch_skinny(const SkinnyParams &p, hipStream_t s) {
     if constexpr (!W8) {
         int dev = 0, cus = 256;
         TPAMD_HIP(hipGetDevice(&dev));
-        TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
         if (pick_resident<MODE>(p, cus)) return launch_resident<DT, MODE>(p, cus, s);
     }
     if constexpr (MODE == SK_SWIGLU && !W8) {
@@ -1011,6 +1014,7 @@ int launch_skinny(const SkinnyParams &p, hipStream_t s) {
             SkinnyParams q = p;
             q.x = p.x + static_cast<int64_t>(m0) * p.ldx * 2;
             q.y = p.y + static_cast<int64_t>(m0) * p.ldy * 2;
+            if (p.addend != nullptr) q.addend = p.addend + static_cast<int64_t>(m0) * p.ldadd * 2;
             q.M = p.M - m0 < 32 ? p.M - m0 : 32;
             const int rc = launch_skinny<DT, W8, MODE>(q, s);
             if (rc != TPAMD_OK) return rc;
@@ -1042,9 +1046,9 @@ int launch_skinny(const SkinnyParams &p, hipStream_t s) {
 }  // namespace
 
 // M <= 64. dtype is BF16 or F16. `w8` selects the int8 weight path (linear only).
-int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *scale,
-                    const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N, int64_t K,
-                    int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
+int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bias, const void *addend, int64_t ldadd,
+                    const void *scale, const void *outlier_idx, const void *w_out, int64_t n_out, void *y, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
                     hipStream_t s) {
     SkinnyParams p{};
     p.x = static_cast<const char *>(x);
@@ -1054,6 +1058,8 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     p.scale = static_cast<const float *>(scale);
     p.outlier_idx = static_cast<const int *>(outlier_idx);
     p.w_out = static_cast<const char *>(w_out);
+    p.addend = static_cast<const char *>(addend);
+    p.ldadd = ldadd;
     p.y = static_cast<char *>(y);
     p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
     p.n_out = static_cast<int>(n_out);

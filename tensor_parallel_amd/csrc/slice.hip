@@ -192,8 +192,8 @@ extern "C" int tpamd_copy_plan_create(const tpamd_copy_job *jobs, size_t n_jobs,
     std::vector<Tile> tiles;
     uint64_t bytes = 0;
     uint32_t TILE_UNITS = MAX_TILE_UNITS;
-    if (const char *e = getenv("TPAMD_COPY_TILE_UNITS")) {  // tuning knob
-        const int v = atoi(e);
+    {  // tuning knob
+        const int v = tuning().copy_tile_units;
         if (v >= 256 && v <= static_cast<int>(MAX_TILE_UNITS)) TILE_UNITS = static_cast<uint32_t>(v);
     }
     try {
@@ -268,8 +268,8 @@ extern "C" int tpamd_copy_plan_create(const tpamd_copy_job *jobs, size_t n_jobs,
     if (e == hipSuccess) e = hipGetDeviceProperties(&prop, plan->device);
     if (e == hipSuccess && plan->n_tiles) {
         int per_cu = 8;
-        if (const char *s = getenv("TPAMD_COPY_BLOCKS_PER_CU")) {
-            int v = atoi(s);
+        {
+            const int v = tuning().copy_blocks_per_cu;
             if (v >= 1 && v <= 64) per_cu = v;
         }
         const uint64_t cap = static_cast<uint64_t>(prop.multiProcessorCount) * per_cu;
@@ -343,7 +343,7 @@ extern "C" int tpamd_copy_jobs_run(const tpamd_copy_job *jobs, size_t n_jobs, vo
     b.n_tiles = static_cast<uint32_t>(tiles);
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
-    TPAMD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
     const uint64_t cap = static_cast<uint64_t>(cus) * 8;
     hipLaunchKernelGGL(copy_small_kernel, dim3(static_cast<unsigned>(tiles < cap ? tiles : cap)), dim3(COPY_THREADS), 0,
                        static_cast<hipStream_t>(stream), b);

@@ -53,3 +53,19 @@ def run_jobs_on_host(jobs, buffers):
             d0 = doff + r * (dp if rows > 1 else 0)
             assert s0 + row_bytes <= sbuf.size and d0 + row_bytes <= dbuf.size
             dbuf[d0 : d0 + row_bytes] = sbuf[s0 : s0 + row_bytes]
+
+
+@pytest.fixture
+def tune(monkeypatch):
+    """Sets a TPAMD_* tuning knob for one test: the library reads its environment once, so it is told to read it again,
+    and once more when the variable is gone."""
+    from tensor_parallel_amd import _native
+
+    def set_knob(name, value):
+        monkeypatch.setenv(name, str(value))
+        _native.reload_tuning()
+
+    yield set_knob
+    monkeypatch.undo()
+    if _native.available():
+        _native.reload_tuning()

@@ -168,12 +168,12 @@ def test_llama_mlp_shard_prefill_4096_sampled_rows():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(40, 136, 5504), (130, 260, 1536), (300, 64, 2048), (17, 512, 1024)])
 @pytest.mark.parametrize("splits", [1, 3, 8])
-def test_split_k_tiles(dtype, M, N, K, splits, monkeypatch):
+def test_split_k_tiles(dtype, M, N, K, splits, tune):
     """The 128 x 128 tiling with K split `splits` ways (forced through the library's debugging knob; by default
     the split is chosen from the tile count): ragged last split, tile rows past M, tile columns past N, bias and
     GELU applied by the finishing pass."""
-    monkeypatch.setenv("TPAMD_GEMM_SPLITK", str(splits))
-    monkeypatch.setenv("TPAMD_GEMM_TILE", "128")
+    tune("TPAMD_GEMM_SPLITK", str(splits))
+    tune("TPAMD_GEMM_TILE", "128")
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     want = F.gelu(F.linear(x.float(), w.float(), b.float()))
@@ -185,8 +185,8 @@ def test_split_k_tiles(dtype, M, N, K, splits, monkeypatch):
 
 
 def test_mid_sized_linear_inside_a_hip_graph():
-    """A split-K GEMM recorded into a HIP graph after a warm-up call (which allocates the library's scratch buffer)
-    replays to the eager result every time, with eager work in between."""
+    """A split-K GEMM recorded into a HIP graph after a warm-up call on the capture stream (which allocates that
+    stream's scratch buffer) replays to the eager result every time, with eager work in between."""
     M, N, K = 64, 512, 4096
     x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
     eager = _native.linear(x, w)
@@ -194,6 +194,9 @@ def test_mid_sized_linear_inside_a_hip_graph():
     out = torch.empty_like(eager)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert torch.equal(_native.linear(x, w), eager)
+    torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         out.copy_(_native.linear(x, w))
@@ -208,13 +211,13 @@ def test_mid_sized_linear_inside_a_hip_graph():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(300, 520, 128), (513, 260, 192), (700, 1028, 320), (256, 256, 64), (1030, 772, 1088)])
 @pytest.mark.parametrize("waves", [4, 8])
-def test_256_tiles_on_ragged_shapes(dtype, M, N, K, waves, monkeypatch):
+def test_256_tiles_on_ragged_shapes(dtype, M, N, K, waves, tune):
     """The 256 x 256 tiling (forced through the library's debugging knobs; by default it is taken when a cost model
     predicts it to be faster) with 4 and with 8 wavefronts per block: two-tile K (the pipeline's minimum), tile rows past M, tile
     columns past N, bias and GELU, the gated pair, and a strided x. K = 64 is always served by the 8-wavefront
     kernel. Blocks that walk through several tiles are covered by the next test and by the full-shape tests."""
-    monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
-    monkeypatch.setenv("TPAMD_GEMM_W4", "1" if waves == 4 else "0")
+    tune("TPAMD_GEMM_TILE", "256")
+    tune("TPAMD_GEMM_W4", "1" if waves == 4 else "0")
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
@@ -228,15 +231,15 @@ def test_256_tiles_on_ragged_shapes(dtype, M, N, K, waves, monkeypatch):
     check_half(got, F.linear(strided.float().cpu(), w.float()), K)
 
 
-def test_both_256_tile_kernels_agree_bit_for_bit(monkeypatch):
+def test_both_256_tile_kernels_agree_bit_for_bit(tune):
     """Same products added in the same order: the 4- and the 8-wavefront kernel must give identical results, also
     when a block walks through several tiles (3 x 96 = 288 tiles on at most 256 blocks)."""
     M, N, K = 700, 24500, 256
     x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
-    monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
-    monkeypatch.setenv("TPAMD_GEMM_W4", "1")
+    tune("TPAMD_GEMM_TILE", "256")
+    tune("TPAMD_GEMM_W4", "1")
     four = _native.linear(x, w)
-    monkeypatch.setenv("TPAMD_GEMM_W4", "0")
+    tune("TPAMD_GEMM_W4", "0")
     eight = _native.linear(x, w)
     assert torch.equal(four, eight)
     check_half(four[:, :512], F.linear(x.float().cpu(), w[:512].float().cpu()), K)
@@ -245,13 +248,13 @@ def test_both_256_tile_kernels_agree_bit_for_bit(monkeypatch):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,splits", [(300, 520, 256, 2), (513, 260, 320, 2), (700, 1028, 448, 3), (256, 256, 576, 4), (1030, 772, 1088, 8), (130, 8, 704, 5)])
-def test_256_tiles_split_over_k(dtype, M, N, K, splits, monkeypatch):
+def test_256_tiles_split_over_k(dtype, M, N, K, splits, tune):
     """The 4-wavefront 256 x 256 kernel with K split over several blocks per tile (forced; by default the cost model
     decides): splits of unequal length, the shortest allowed (2 K tiles), a last split that would be a single K tile
     (K = 448 = 7 tiles in 3 splits: the library lengthens the splits instead), an odd number of 128 x 128 partial
     tiles along M and N, bias and GELU applied by the finishing pass, and the gated pair."""
-    monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
-    monkeypatch.setenv("TPAMD_GEMM_SPLITK256", str(splits))
+    tune("TPAMD_GEMM_TILE", "256")
+    tune("TPAMD_GEMM_SPLITK256", str(splits))
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
@@ -260,7 +263,7 @@ def test_256_tiles_split_over_k(dtype, M, N, K, splits, monkeypatch):
     sigma = (0.02 * math.sqrt(K)) ** 2
     torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
     # the unsplit launch adds the same products in another order
-    monkeypatch.setenv("TPAMD_GEMM_SPLITK256", "1")
+    tune("TPAMD_GEMM_SPLITK256", "1")
     unsplit = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     torch.testing.assert_close(got.float(), unsplit.float(), rtol=RTOL_HALF, atol=RTOL_HALF * 0.02 * math.sqrt(K))
 
@@ -276,13 +279,13 @@ def test_mid_sized_shapes_choose_a_correct_path():
 
 @pytest.mark.parametrize("tile", ["128", "256"])
 @pytest.mark.parametrize("N,ldy,shift", [(260, 264, 0), (260, 264, 4), (256, 260, 0), (520, 528, 8), (132, 136, 4)])
-def test_strided_and_8_byte_aligned_outputs_through_the_c_abi(tile, N, ldy, shift, monkeypatch):
+def test_strided_and_8_byte_aligned_outputs_through_the_c_abi(tile, N, ldy, shift, tune):
     """y with a row pitch above N and a base that is 8- but not 16-byte aligned (shift = 4 elements): the epilogues
     choose between 16- and 8-byte stores by the alignment of y and its pitch, and a row's last 4 columns (N % 8 == 4)
     are always an 8-byte store. The columns between N and the pitch must stay untouched."""
     import ctypes
 
-    monkeypatch.setenv("TPAMD_GEMM_TILE", tile)
+    tune("TPAMD_GEMM_TILE", tile)
     M, K = 300, 256
     x, w, b = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N,), 2, 0.1).to(DEV)
     w2 = rnd((N, K), 5, 0.02).to(DEV)
@@ -307,13 +310,13 @@ def test_strided_and_8_byte_aligned_outputs_through_the_c_abi(tile, N, ldy, shif
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [4, 9, 16])
 @pytest.mark.parametrize("N,K", [(64, 64), (132, 200), (1028, 1000), (2740, 4096), (520, 5504), (300, 8192), (260, 7000)])
-def test_x_resident_weight_streaming_kernel(dtype, M, N, K, monkeypatch):
+def test_x_resident_weight_streaming_kernel(dtype, M, N, K, tune):
     """The weight-streaming kernel that keeps its x fragments in registers and walks a range of columns per block
     (forced; by default it serves 9 to 16 rows when there are enough weight tiles per CU): fewer tiles than CUs,
     several tiles per block with a masked last tile (2740 columns over 256 blocks), column ranges that do not start
     on a multiple of 8, a ragged last K chunk, K above 4096 and above 6144 (6 and 8 chunks per wavefront), bias and
     GELU, the gated pair."""
-    monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "1")
+    tune("TPAMD_SKINNY_RESIDENT", "1")
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
@@ -321,22 +324,22 @@ def test_x_resident_weight_streaming_kernel(dtype, M, N, K, monkeypatch):
     h = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
     sigma = (0.02 * math.sqrt(K)) ** 2
     torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
-    monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "0")
+    tune("TPAMD_SKINNY_RESIDENT", "0")
     plain = _native.swiglu_up(x.to(DEV), w.to(DEV), w2.to(DEV))
     torch.testing.assert_close(h.float(), plain.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
 
 
 @pytest.mark.parametrize("case", ["tiles256_split", "resident_pair", "resident_single"])
-def test_other_dispatch_paths_inside_a_hip_graph(case, monkeypatch):
+def test_other_dispatch_paths_inside_a_hip_graph(case, tune):
     """The 256 x 256 tiling with K split over blocks (two launches sharing the scratch buffer) and the x-resident
     weight-streaming kernel, recorded into a HIP graph after a warm-up call: every replay gives the eager result,
     with eager work in between."""
     if case == "tiles256_split":
-        monkeypatch.setenv("TPAMD_GEMM_TILE", "256")
-        monkeypatch.setenv("TPAMD_GEMM_SPLITK256", "3")
+        tune("TPAMD_GEMM_TILE", "256")
+        tune("TPAMD_GEMM_SPLITK256", "3")
         M, N, K = 300, 520, 1088
     else:
-        monkeypatch.setenv("TPAMD_SKINNY_RESIDENT", "1")
+        tune("TPAMD_SKINNY_RESIDENT", "1")
         M, N, K = 16, 2740, 4096
     x, w, w2 = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N, K), 5, 0.02).to(DEV)
     fn = (lambda: _native.swiglu_up(x, w, w2)) if case == "resident_pair" else (lambda: _native.linear(x, w))
@@ -345,6 +348,9 @@ def test_other_dispatch_paths_inside_a_hip_graph(case, monkeypatch):
     out = torch.empty_like(eager)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream: a stream's scratch buffer is allocated at its first use
+        assert torch.equal(fn(), eager)
+    torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         out.copy_(fn())

@@ -73,11 +73,11 @@ def test_falcon_mlp_shard_full_shape():
 
 
 @pytest.fixture
-def column_groups(monkeypatch):
+def column_groups(tune):
     """Forces the number of 16-column groups per block of the decode kernel (a debugging knob of the library;
     by default it is chosen from the shape and only large N gets more than one)."""
     def use(cg):
-        monkeypatch.setenv("TPAMD_SKINNY_CG", str(cg))
+        tune("TPAMD_SKINNY_CG", str(cg))
     return use
 
 
@@ -122,7 +122,7 @@ def test_16bit_decode_kernels_column_groups(dtype, M, cg, column_groups):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M", [9, 16, 17, 32, 33, 64, 70])
 @pytest.mark.parametrize("N,K,n_out", [(64, 4096, 0), (200, 4128, 5), (1000, 8192, 41), (528, 6144, 33), (48, 16384, 256)])
-def test_k_split_kernel(dtype, M, N, K, n_out, monkeypatch):
+def test_k_split_kernel(dtype, M, N, K, n_out, tune):
     """The int8 kernel that splits K over blocks and keeps its x fragments in registers (forced; by default it
     serves 12 or more rows on large matrices): 1, 2 and 4 row tiles, a single split and several, a last split that
     is partly or wholly past the end of K, column ranges whose last tile is masked, outlier columns on wavefronts
@@ -133,9 +133,9 @@ def test_k_split_kernel(dtype, M, N, K, n_out, monkeypatch):
             torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None,
             torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None)
     bias = (torch.randn(N, generator=torch.Generator().manual_seed(5)) * 0.1).to(dtype).to(DEV)
-    monkeypatch.setenv("TPAMD_W8_SPLIT", "1")
+    tune("TPAMD_W8_SPLIT", "1")
     got = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
-    monkeypatch.setenv("TPAMD_W8_SPLIT", "0")
+    tune("TPAMD_W8_SPLIT", "0")
     plain = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
     want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out) + bias.double().cpu().numpy()
     want = 0.5 * want * (1.0 + np.vectorize(math.erf)(want / math.sqrt(2.0)))
@@ -144,10 +144,10 @@ def test_k_split_kernel(dtype, M, N, K, n_out, monkeypatch):
     torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * sigma)
 
 
-def test_k_split_kernel_inside_a_hip_graph(monkeypatch):
+def test_k_split_kernel_inside_a_hip_graph(tune):
     """The K-split int8 kernel and its finishing pass (two launches sharing the library's scratch buffer) recorded
     into a HIP graph after a warm-up call: every replay gives the eager result, with eager work in between."""
-    monkeypatch.setenv("TPAMD_W8_SPLIT", "1")
+    tune("TPAMD_W8_SPLIT", "1")
     M, N, K, n_out = 32, 200, 8192, 41
     x, wq, scale, cols, w_out = make_case(M, N, K, n_out, torch.float16, seed=6)
     args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
@@ -157,6 +157,9 @@ def test_k_split_kernel_inside_a_hip_graph(monkeypatch):
     out = torch.empty_like(eager)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream: a stream's scratch buffer is allocated at its first use
+        assert torch.equal(_native.linear_w8(*args), eager)
+    torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         out.copy_(_native.linear_w8(*args))
