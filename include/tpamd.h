@@ -165,6 +165,19 @@ int tpamd_linear_add(const void *x_dev, const void *w_dev, const void *bias_dev,
                      int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldadd, int64_t ldy, int dtype,
                      int act, void *stream);
 
+/* tpamd_linear for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, same kernels and the same
+ * result, bit for bit, as tpamd_linear; the call allocates nothing (no hipMalloc, no hipFree), also at its first use
+ * and under stream capture. Where tpamd_linear would put the fp32 partial tiles of a K split into its stream's
+ * scratch buffer, this entry point puts them into a fixed array of tpamd_noalloc_scratch_bytes() = 32 MiB that every
+ * GPU the library is loaded on holds until the process ends. A shape whose K split needs more (the message names
+ * the size) is refused with TPAMD_ERR_UNSUPPORTED and nothing is launched; tpamd_linear takes such shapes.
+ * All calls on one GPU share that GPU's array: calls on the same stream are ordered by it, calls that overlap on
+ * different streams of one GPU race on the partial tiles and must be ordered by the caller. */
+int tpamd_linear_noalloc(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,
+                         int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype, int act, void *stream);
+uint64_t tpamd_noalloc_scratch_bytes(void);
+
 /* h[M,N] = silu(x . wg^T) * (x . wu^T): the gate/up pair of a SiLU-gated MLP shard in one pass over x
  * (two column-parallel torch.nn.Linear calls, a SiLU and a product in the reference's wrapped module;
  * weights sliced by `Split(world_size, dim=0)`, src/tensor_parallel/slicing_configs.py:376-378).

@@ -29,6 +29,8 @@ EXPORTS = (
     "tpamd_scratch_query",
     "tpamd_linear",
     "tpamd_linear_add",
+    "tpamd_linear_noalloc",
+    "tpamd_noalloc_scratch_bytes",
     "tpamd_swiglu_up",
     "tpamd_linear_w8",
     "tpamd_attention",
@@ -87,6 +89,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_linear.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
     lib.tpamd_linear_add.restype = ci
     lib.tpamd_linear_add.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, ci, ci, vp]
+    lib.tpamd_linear_noalloc.restype = ci
+    lib.tpamd_linear_noalloc.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, vp]
+    lib.tpamd_noalloc_scratch_bytes.restype = u64
+    lib.tpamd_noalloc_scratch_bytes.argtypes = []
     lib.tpamd_tuning_reload.restype = None
     lib.tpamd_tuning_reload.argtypes = []
     lib.tpamd_scratch_query.restype = ci

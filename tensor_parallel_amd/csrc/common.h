@@ -61,7 +61,19 @@ int device_cus(int dev, int *cus_out);
 // and pass reserve = 4 * CUs * 64 KiB, so that a stream's buffer is allocated with the size every shape can live with.
 std::mutex &splitk_mutex();
 int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out);
-// Body of tpamd_linear / tpamd_linear_add (api.hip).
+// While one of these lives on a host thread, splitk_scratch() on that thread hands out the library's fixed array and
+// allocates nothing.
+constexpr size_t TPAMD_NOALLOC_SCRATCH_BYTES = static_cast<size_t>(32) << 20;
+bool static_scratch_active();
+int static_scratch(int dev, size_t need, void **out);
+struct StaticScratchScope {
+    StaticScratchScope();
+    ~StaticScratchScope();
+    StaticScratchScope(const StaticScratchScope &) = delete;
+    StaticScratchScope &operator=(const StaticScratchScope &) = delete;
+};
+
+// Body of tpamd_linear / tpamd_linear_add / tpamd_linear_noalloc (api.hip).
 int linear_entry(const char *who, const void *x_dev, const void *w_dev, const void *bias_dev, const void *addend_dev,
                  int64_t ldadd, void *y_dev, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int dtype,
                  int act, void *stream);

@@ -83,8 +83,10 @@ std::mutex &splitk_mutex() {
 // until the process ends; streams of one device never share one, so K-split work on different streams cannot meet in
 // it. NULL comes back when the stream has no buffer yet and is being captured (allocating is not allowed then), when
 // `need` is larger than the stream's buffer, and for the ninth stream of a device.
+// Inside a StaticScratchScope (noalloc.hip) the library's fixed array is handed out instead.
 int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
     *out = nullptr;
+    if (static_scratch_active()) return static_scratch(dev, need, out);
     int on_device = 0;
     for (Entry &e : g_cache) {
         if (e.dev != dev) continue;
