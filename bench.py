@@ -1,8 +1,8 @@
 """Benchmark of the per-rank hot path on one MI355X.
 
 Workload (BASELINE.json configs[1]): the rank-0 shard at W = 2 of a Llama-7B MLP, d = 4096, shard width 5504,
-bf16, M = 4096 tokens. One step = fused gate/up GEMM + SiLU gate, down-projection GEMM (the row-parallel
-partial), and the on-device sum with the other rank's partial. Prints ONE JSON line.
+bf16, M = 4096 tokens. One step = fused gate/up GEMM + SiLU gate, then the down-projection GEMM (the row-parallel
+partial) whose epilogue adds the other rank's partial (the on-device 2-partial sum). Prints ONE JSON line.
 """
 from __future__ import annotations
 
@@ -66,7 +66,12 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--tokens", type=int, default=4096)
+    ap.add_argument("--settle", type=int, default=240, help="untimed steps before the counted warm-up (clock settling)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="instead of the benchmark, measure what this part sustains on the two bounding resources (MFMA-only "
+                         "loop, read / write / copy streams) and time hipBLASLt on the benchmark's GEMM shapes beside this "
+                         "library's kernels; prints a table and one JSON line")
     ap.add_argument("--no-extra", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -83,6 +88,8 @@ def main() -> int:
         return 1
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.ceilings:
+        return ceilings(torch, _native, dev)
     M = args.tokens
     g = torch.Generator(device=dev).manual_seed(0)
 
@@ -94,6 +101,8 @@ def main() -> int:
     x = torch.randn(M, D_MODEL, generator=torch.Generator(device=dev).manual_seed(1), device=dev).to(torch.bfloat16)
     other = torch.randn(M, D_MODEL, generator=g, device=dev).to(torch.bfloat16)  # the other rank's partial
 
+    out_buf = torch.empty(M, D_MODEL, device=dev, dtype=torch.bfloat16)
+
     def step(i, ev=None):
         wg, wu, wd = sets[i % n_sets]
         if ev is not None:
@@ -101,9 +110,15 @@ def main() -> int:
         h = _native.swiglu_up(x, wg, wu)
         if ev is not None:
             ev[1].record()
-        p = _native.linear(h, wd)
-        return _native.reduce_partials([p, other], out=p)
+        # the down projection adds the other rank's partial in its epilogue: product rounded to bf16, fp32 add, rounded
+        # again, i.e. the 2-partial `sum` of the reference in the same launch
+        return _native.linear(h, wd, addend=other, out=out_buf)
 
+    # Settling run, outside the counted warm-up: the part's power management needs about a hundred launches (50 ms) of
+    # this load before its clock stops moving (the first launches run at boost clock, the next ones over-correct), and
+    # every rotated weight set has to have been touched. Without it a short run times the transient, not the kernel.
+    for i in range(args.settle):
+        step(i)
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -150,13 +165,121 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"llama7b_mlp_rank0_shard_w2_m{M}_bf16", "d_model": D_MODEL, "ffn_shard": FFN_SHARD,
-                   "tokens": M, "step": "swiglu_up + down + 2-partial reduce", "weights": "N(0,0.02) seed 0", "weight_sets_rotated": n_sets},
+                   "tokens": M, "step": "swiglu_up + down projection with the 2-partial sum in its epilogue", "settle_steps": args.settle, "weights": "N(0,0.02) seed 0", "weight_sets_rotated": n_sets},
         "roofline": roofline,
     }
     if not args.no_extra:
         out["extra"] = extra_measurements(torch, _native, dev, sets, other)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def ceilings(torch, _native, dev) -> int:
+    """What bounds the kernels on this part, measured in one process. Every figure is taken after the part has run the
+    same load for a while (its clock settles over tens of milliseconds), as the average over the launches that follow."""
+    import ctypes
+
+    from tensor_parallel_amd.build import PROBES_LIB
+
+    probes = ctypes.CDLL(str(PROBES_LIB))
+    vp, ci, u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64
+    probes.tpamd_probe_mfma.argtypes = [ci, vp, vp, ci, ci, vp]
+    probes.tpamd_probe_mfma_flops.restype = ctypes.c_double
+    probes.tpamd_probe_mfma_flops.argtypes = [ci, ci, ci]
+    probes.tpamd_probe_stream.argtypes = [ci, vp, vp, u64, ci, vp, vp]
+    stream = lambda: vp(torch.cuda.current_stream(dev).cuda_stream)  # noqa: E731
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.zeros(256, device=dev)
+    out = {"device": torch.cuda.get_device_name(dev), "cus": cus}
+
+    def settled_us(fn, settle_s=0.25, iters=40):
+        """Average launch time of fn(i) after running it for settle_s seconds."""
+        t0, i = time.perf_counter(), 0
+        while time.perf_counter() - t0 < settle_s:
+            fn(i)
+            i += 1
+            if i % 16 == 0:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for j in range(iters):
+            fn(i + j)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters * 1e3
+
+    # ---- 1. nothing but MFMAs: constant operands against random ones, both instruction shapes
+    n_vec = cus * 256 * 8
+    ops = {"constant": torch.full((n_vec * 8,), 1.0, device=dev).to(torch.bfloat16),
+           "random": (torch.randn(n_vec * 8, device=dev, generator=torch.Generator(device=dev).manual_seed(0)) * 2).to(torch.bfloat16)}
+    mfma = {}
+    for shape, name in ((16, "v_mfma_f32_16x16x32_bf16"), (32, "v_mfma_f32_32x32x16_bf16")):
+        iters = 20000
+        flops = probes.tpamd_probe_mfma_flops(shape, cus, iters)
+        for kind, buf in ops.items():
+            us = settled_us(lambda i: probes.tpamd_probe_mfma(shape, vp(buf.data_ptr()), vp(sink.data_ptr()), cus, iters, stream()), 0.4, 10)
+            mfma[f"{name} {kind} operands"] = {"us_per_launch": us, "TFLOPs": flops / us / 1e6, "frac_of_2500": flops / us / 1e6 / PEAK_BF16_TFLOPS}
+    out["mfma_only_loop_4_wavefronts_per_cu"] = mfma
+
+    # ---- 2. streams at the byte counts of the HBM-bound kernels: down matrix, gate + up matrices, the whole state dict
+    streams = {}
+    sizes = (("llama7b_down_shard_45MB", FFN_SHARD * D_MODEL * 2, 6), ("llama7b_gate_up_shards_90MB", 2 * FFN_SHARD * D_MODEL * 2, 4),
+             ("llama2_7b_split_tensors_13.5GB", 13476298752, 1))
+    for label, nbytes, copies in sizes:
+        nbytes = nbytes // 16384 * 16384
+        srcs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
+        dsts = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(copies)]
+        row = {}
+        for mode, what, moved in ((0, "read_only", nbytes), (1, "write_only", nbytes), (2, "copy_read_plus_write", 2 * nbytes)):
+            best = None
+            for per_cu in (4, 8, 16):
+                us = settled_us(lambda i: probes.tpamd_probe_stream(mode, vp(srcs[i % copies].data_ptr()), vp(dsts[i % copies].data_ptr()),
+                                                                    nbytes, cus * per_cu, vp(sink.data_ptr()), stream()), 0.15, 20 if nbytes < 1e9 else 5)
+                if best is None or us < best[0]:
+                    best = (us, per_cu)
+            row[what] = {"us": best[0], "GBps": moved / best[0] / 1e3, "frac_of_8000": moved / best[0] / 1e3 / PEAK_HBM_GBS, "blocks_per_cu": best[1]}
+        us = settled_us(lambda i: dsts[i % copies].copy_(srcs[i % copies]), 0.15, 20 if nbytes < 1e9 else 5)
+        row["device_to_device_copy_of_the_runtime"] = {"us": us, "GBps": 2 * nbytes / us / 1e3, "frac_of_8000": 2 * nbytes / us / 1e3 / PEAK_HBM_GBS}
+        streams[label] = row
+        del srcs, dsts
+    out["streams"] = streams
+
+    # ---- 3. hipBLASLt (through torch.matmul) on the benchmark's GEMM shapes beside this library's kernels
+    M = 4096
+    g = torch.Generator(device=dev).manual_seed(0)
+    w = lambda shape: (torch.randn(shape, generator=g, device=dev) * 0.02).to(torch.bfloat16)  # noqa: E731
+    sets = [(w((FFN_SHARD, D_MODEL)), w((FFN_SHARD, D_MODEL)), w((D_MODEL, FFN_SHARD)), torch.cat([w((FFN_SHARD, D_MODEL)), w((FFN_SHARD, D_MODEL))]))
+            for _ in range(3)]
+    x = torch.randn(M, D_MODEL, generator=g, device=dev).to(torch.bfloat16)
+    h = torch.randn(M, FFN_SHARD, generator=g, device=dev).to(torch.bfloat16) * 0.1
+    other = torch.randn(M, D_MODEL, generator=g, device=dev).to(torch.bfloat16)
+    y = torch.empty(M, D_MODEL, device=dev, dtype=torch.bfloat16)
+    gu = torch.empty(M, 2 * FFN_SHARD, device=dev, dtype=torch.bfloat16)
+    f_up, f_down = 4.0 * M * D_MODEL * FFN_SHARD, 2.0 * M * D_MODEL * FFN_SHARD
+    side = {}
+
+    def row(label, fn, flops):
+        us = settled_us(fn, 0.3, 40)
+        side[label] = {"us": us, "TFLOPs": flops / us / 1e6, "frac_of_2500": flops / us / 1e6 / PEAK_BF16_TFLOPS}
+
+    row("gate_up: this library, tpamd_swiglu_up (GEMM + SiLU gate fused)", lambda i: _native.swiglu_up(x, sets[i % 3][0], sets[i % 3][1]), f_up)
+    row("gate_up: hipBLASLt, one GEMM on the stacked [11008 x 4096] weight, no SiLU gate", lambda i: torch.matmul(x, sets[i % 3][3].t(), out=gu), f_up)
+    row("down: this library, tpamd_linear", lambda i: _native.linear(h, sets[i % 3][2], out=y), f_down)
+    row("down: this library, tpamd_linear_add (2-partial sum in the epilogue)", lambda i: _native.linear(h, sets[i % 3][2], addend=other, out=y), f_down)
+    row("down: hipBLASLt", lambda i: torch.matmul(h, sets[i % 3][2].t(), out=y), f_down)
+    out["gemm_side_by_side_m4096"] = side
+
+    for section in ("mfma_only_loop_4_wavefronts_per_cu", "gemm_side_by_side_m4096"):
+        print(f"# {section}")
+        for k, v in out[section].items():
+            print(f"  {k:86s} {v['us']if 'us' in v else v['us_per_launch']:10.1f} us {v['TFLOPs']:8.1f} TFLOP/s  {v['frac_of_2500']:.3f} of 2500")
+    print("# streams")
+    for label, rowd in out["streams"].items():
+        for what, v in rowd.items():
+            print(f"  {label:34s} {what:38s} {v['us']:10.1f} us {v['GBps']:8.1f} GB/s  {v['frac_of_8000']:.3f} of 8000")
     print(json.dumps(out), flush=True)
     return 0
 
@@ -232,8 +355,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     from tensor_parallel_amd.slicing import BatchSlicer
     from tensor_parallel_amd.slicing_configs import get_llama_config
 
-    layers, world = 32, 2
-    cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=4096, num_attention_heads=32, num_key_value_heads=32), [dev] * world)
+    layers = 32
     state = {}
     for layer in range(layers):
         p = f"model.layers.{layer}."
@@ -243,18 +365,22 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
             state[p + name + ".weight"] = torch.empty(shape, device=dev, dtype=torch.bfloat16).normal_(0, 0.02)
     state["model.embed_tokens.weight"] = torch.empty((32000, 4096), device=dev, dtype=torch.bfloat16).normal_(0, 0.02)
     state["lm_head.weight"] = torch.empty((32000, 4096), device=dev, dtype=torch.bfloat16).normal_(0, 0.02)
-    batch = BatchSlicer(dev)
-    keep = []
-    for r in range(world):
-        for name, t in state.items():
-            action = next(a for p, a in cfg.state_rules.items() if p.search(name))
-            keep.append(batch.add(t, action.spec(tuple(t.shape), r)))
-    plan = batch.build()
-    us = _time_us(torch, lambda i: plan.run(), 2, 10)
-    moved = 2.0 * plan.nbytes
-    extra["slicing_w2"] = {"tensors": len(state), "bytes_read_plus_written": moved, "us_per_launch": us,
-                           "GBps": moved / us / 1e3, "hbm_frac": moved / us / 1e3 / PEAK_HBM_GBS}
-    batch.close()
+    for world in (2, 4, 8):
+        cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=4096, num_attention_heads=32, num_key_value_heads=32), [dev] * world)
+        batch = BatchSlicer(dev)
+        keep = []
+        for r in range(world):
+            for name, t in state.items():
+                action = next(a for p, a in cfg.state_rules.items() if p.search(name))
+                keep.append(batch.add(t, action.spec(tuple(t.shape), r)))
+        plan = batch.build()
+        us = _time_us(torch, lambda i: plan.run(), 2, 10)
+        moved = 2.0 * plan.nbytes
+        extra[f"slicing_w{world}"] = {"tensors": len(state), "shards": len(keep), "bytes_read_plus_written": moved, "us_per_launch": us,
+                                      "GBps": moved / us / 1e3, "hbm_frac": moved / us / 1e3 / PEAK_HBM_GBS}
+        torch.cuda.synchronize()
+        batch.close()
+        del keep, plan, batch
     return extra
 
 

@@ -297,25 +297,20 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
         raise ValueError(f"linear: x has {x.shape[-1]} input features, w is {tuple(w.shape)}")
     if w.device != x.device:
         raise ValueError(f"linear: x is on {x.device}, w on {w.device}")
+    N, K = w.shape
+    M = x.numel() // K if K else 0
+    if bias is not None and (bias.shape != (N,) or bias.dtype != x.dtype or bias.device != x.device):
+        raise ValueError("linear: bias must have shape [N], the dtype of x and live on its device")
+    if addend is not None and (addend.dtype != x.dtype or addend.device != x.device or addend.numel() != M * N
+                               or addend.shape[-1] != N):
+        raise ValueError("linear: addend must have the shape, dtype and device of the result")
+    if out is not None and (out.dtype != x.dtype or out.device != x.device or out.numel() != M * N or not out.is_contiguous()):
+        raise ValueError("linear: out must be a contiguous tensor of the result's size, dtype and device")
     x2, w2 = _as_2d(x), _as_2d(w)
-    M, K = x2.shape
-    N = w2.shape[0]
-    if out is None:
-        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
-    else:
-        if out.dtype != x.dtype or out.device != x.device or out.numel() != M * N or not out.is_contiguous():
-            raise ValueError("linear: out must be a contiguous tensor of the result's size, dtype and device")
-        y = out.view(M, N)
-    b = None
-    if bias is not None:
-        b = bias.contiguous()
-        if b.shape != (N,) or b.dtype != x.dtype or b.device != x.device:
-            raise ValueError("linear: bias must have shape [N], the dtype of x and live on its device")
-    a2 = None
-    if addend is not None:
-        if addend.dtype != x.dtype or addend.device != x.device or addend.numel() != M * N or addend.shape[-1] != N:
-            raise ValueError("linear: addend must have the shape, dtype and device of the result")
-        a2 = _as_2d(addend)
+    M = x2.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device) if out is None else out.view(M, N)
+    b = bias.contiguous() if bias is not None else None
+    a2 = _as_2d(addend) if addend is not None else None
     with torch.cuda.device(x.device):
         stream = ctypes.c_void_p(current_stream_ptr(x.device))
         if a2 is None:

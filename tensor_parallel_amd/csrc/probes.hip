@@ -1,0 +1,107 @@
+// Measurement probes, built into their own library (libtpamd_probes.so) and used only by `bench.py --ceilings`: what one
+// MI355X sustains on the two resources the hot path is bound by, measured with nothing else in the way.
+//   tpamd_probe_mfma    a loop of nothing but bf16 MFMAs (no loads, no LDS), operands constant or random
+//   tpamd_probe_stream  a read-only / write-only / copy stream over a buffer, 16 bytes per lane, non-temporal
+// The product library does not link this file.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+// One wavefront per SIMD (4 per block, one block per CU), 32 independent accumulator tiles: the issue pattern of the
+// GEMM kernels' inner loop without its loads and LDS reads. SHAPE 16: v_mfma_f32_16x16x32_bf16, 32: 32x32x16.
+template <int SHAPE>
+__global__ __launch_bounds__(256) void mfma_loop_kernel(const uint4 *operands, float *sink, int iters) {
+    const int tid = blockIdx.x * 256 + threadIdx.x;
+    uint4 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = operands[tid * 8 + i];
+        b[i] = operands[tid * 8 + 4 + i];
+    }
+    float s = 0.f;
+    if constexpr (SHAPE == 32) {
+        f32x16 acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[i & 3]), __builtin_bit_cast(bf16x8, b[(i >> 1) & 3]), acc[i], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += acc[i][0];
+    } else {
+        f32x4 acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[i & 3]), __builtin_bit_cast(bf16x8, b[(i >> 2) & 3]), acc[i], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s += acc[i][0];
+    }
+    if (s == 123.456f) sink[threadIdx.x] = s;  // keeps the loop alive; never true for these operands
+}
+
+// MODE 0: read src, 1: write dst, 2: copy src -> dst. A persistent grid; block b handles 16 KiB pieces b, b + grid, ...
+template <int MODE>
+__global__ __launch_bounds__(256) void stream_kernel(const char *src, char *dst, uint64_t pieces, float *sink) {
+    uint32_t keep = 0;
+    for (uint64_t p = blockIdx.x; p < pieces; p += gridDim.x) {
+        const uint64_t off = p * 16384 + threadIdx.x * 16;
+        v4u v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (MODE != 1) v[i] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(src + off + i * 4096));
+            else v[i] = v4u{static_cast<uint32_t>(p), 1u, 2u, 3u};
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (MODE != 0) __builtin_nontemporal_store(v[i], reinterpret_cast<v4u *>(dst + off + i * 4096));
+            else keep ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+        }
+    }
+    if (MODE == 0 && keep == 0x12345679u) sink[threadIdx.x] = 1.f;
+}
+
+}  // namespace
+
+// operands_dev: blocks * 256 * 8 * 16 bytes of bf16 values; sink_dev: 256 floats. shape: 16 or 32.
+extern "C" int tpamd_probe_mfma(int shape, const void *operands_dev, void *sink_dev, int blocks, int iters, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (shape == 32) hipLaunchKernelGGL((mfma_loop_kernel<32>), dim3(blocks), dim3(256), 0, s, static_cast<const uint4 *>(operands_dev), static_cast<float *>(sink_dev), iters);
+    else if (shape == 16) hipLaunchKernelGGL((mfma_loop_kernel<16>), dim3(blocks), dim3(256), 0, s, static_cast<const uint4 *>(operands_dev), static_cast<float *>(sink_dev), iters);
+    else return -1;
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+// Floating-point operations of one tpamd_probe_mfma launch (4 wavefronts per block; 2 * 16 * 16 * 32 = 2 * 32 * 32 * 16 / 2).
+extern "C" double tpamd_probe_mfma_flops(int shape, int blocks, int iters) {
+    const double per_wave_iter = shape == 32 ? 8 * 32768.0 : 16 * 16384.0;
+    return per_wave_iter * 4.0 * blocks * iters;
+}
+
+// mode 0 read, 1 write, 2 copy; bytes must be a multiple of 16384.
+extern "C" int tpamd_probe_stream(int mode, const void *src_dev, void *dst_dev, uint64_t bytes, int blocks, void *sink_dev, void *stream) {
+    if (bytes % 16384 != 0 || blocks <= 0) return -1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint64_t pieces = bytes / 16384;
+    const char *src = static_cast<const char *>(src_dev);
+    char *dst = static_cast<char *>(dst_dev);
+    float *sink = static_cast<float *>(sink_dev);
+    if (mode == 0) hipLaunchKernelGGL((stream_kernel<0>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink);
+    else if (mode == 1) hipLaunchKernelGGL((stream_kernel<1>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink);
+    else if (mode == 2) hipLaunchKernelGGL((stream_kernel<2>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink);
+    else return -1;
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}

@@ -29,6 +29,17 @@ from .utils import nested_flatten, nested_pack
 logger = logging.getLogger(__file__)
 
 
+# keyword names under which transformers modules take the legacy tuple-of-tensors key/value cache
+LEGACY_CACHE_KWARGS = ("past_key_values", "past_key_value", "layer_past")
+
+
+def _holds_tensors(value) -> bool:
+    """True for a (nested) tuple or list with a tensor somewhere inside."""
+    if isinstance(value, (tuple, list)):
+        return any(isinstance(v, torch.Tensor) or _holds_tensors(v) for v in value)
+    return False
+
+
 def canonicalize_device(device: Union[torch.device, str, int]) -> torch.device:
     device = torch.device(device)
     if device.type == "cuda" and device.index is None:
@@ -44,6 +55,10 @@ def check_device_ids(device_ids: Optional[Sequence[Union[torch.device, str]]]) -
 
 
 class TensorParallel(nn.Module):
+    """Public attributes, as in the reference (tensor_parallel.py:27-108): `module_shards`, `devices`, `device_ids`,
+    `output_device_index`, `all_cuda`, `tensor_parallel_config`, `modified_parameters_names`, `param_fractions`,
+    `sharding_manager`, `need_delayed_init`, `preserve_shards_when_saving`, `_sanity_check_params`."""
+
     def __init__(
         self,
         module: nn.Module,
@@ -57,86 +72,98 @@ class TensorParallel(nn.Module):
         sharded_param_names: Optional[Collection[str]] = None,
     ):
         super().__init__()
-        original_params = sum(p.numel() for p in module.parameters())
-        assert output_device is None or output_device_index is None, "please specify either device or index, not both"
-        device_ids = check_device_ids(device_ids)
-        if output_device is not None:
-            output_device = canonicalize_device(output_device)
-            assert output_device in device_ids, f"Output device {output_device} not in {device_ids}"
-            output_device_index = device_ids.index(output_device)
-        elif output_device_index is None:
-            output_device_index = 0
-
-        self.module_shards = nn.ModuleList()
-        self.devices = device_ids
-        self.output_device_index = output_device_index
-        self.all_cuda = all(d.type == "cuda" for d in self.devices)
+        self.devices = check_device_ids(device_ids)
+        self.output_device_index = self._pick_output_rank(output_device, output_device_index)
         self.device_ids = [d.index if d.type == "cuda" else None for d in self.devices]
-        self.need_delayed_init = delay_init
+        self.all_cuda = all(d.type == "cuda" for d in self.devices)
+        self.need_delayed_init = bool(delay_init)
         self.sharding_manager = None
-        world_size = len(self.devices)
+        self.module_shards = nn.ModuleList()
 
-        if world_size <= 1:
+        if len(self.devices) < 2:  # nothing to split: the module itself is the only shard
             self.module_shards.append(module)
-            if world_size == 1 and not delay_init:
-                self.module_shards[0].to(device_ids[0])
+            if self.devices and not delay_init:
+                module.to(self.devices[0])
             return
-        if delay_init:
-            raise NotImplementedError("delay_init builds shards on the host, which tensor_parallel_amd does not do")
 
+        params_before = sum(p.numel() for p in module.parameters())
         if tensor_parallel_config is None:
+            logger.info("No slicing config given: every Linear and Embedding gets the generic rules")
             tensor_parallel_config = get_default_config(module, self.devices)
-            logger.info("Using automatic config: sharding individual linear/emb layers")
-        tensor_parallel_config = add_lora_rules(module, tensor_parallel_config)
-        self.tensor_parallel_config = tensor_parallel_config
-        config_with_ops = tensor_parallel_config.create_collective_ops(self.devices, distributed)
+        self.tensor_parallel_config = add_lora_rules(module, tensor_parallel_config)
+        self._slice_into_shards(module, self.tensor_parallel_config.create_collective_ops(self.devices, distributed))
+        self._report_replication(params_before)
 
-        # all ranks' slicing is queued per device and launched once
-        batches = {}
-        self.modified_parameters_names = set()
-        for rank, device in enumerate(self.devices):
-            batch = batches.setdefault(device, BatchSlicer(device if device.type == "cuda" else None))
-            shard, modified = make_shard(module, device, config_with_ops, rank=rank, world_size=world_size, batch=batch)
-            self.module_shards.append(shard)
-            self.modified_parameters_names.update(modified)
-        self.sliced_bytes = 0
-        for batch in batches.values():
-            self.sliced_bytes += batch.run()
-        for device, batch in batches.items():
-            if device.type == "cuda" and batch.plan is not None:
-                torch.cuda.synchronize(device)  # sources uploaded for slicing are released below
-            batch.close()
-
-        params_per_shard = [sum(p.numel() for p in shard.parameters()) for shard in self.module_shards]
-        assert sum(params_per_shard) >= original_params, "Internal assert failed: lost some parameters during sharding"
-        self.param_fractions = tuple(n / original_params for n in params_per_shard) if original_params else ()
-        inefficiency_rate = (sum(self.param_fractions) - 1) / len(device_ids)
-        logger.log(
-            logging.DEBUG if inefficiency_rate < 0.1 else logging.WARNING,
-            f"Inefficiency warning: model has {original_params} params but shards have {params_per_shard} params. "
-            f"This means that each device uses {inefficiency_rate * 100:.3f}% extra memory for parameters",
-        )
-
-        # one empty parameter per rank, on the rank's device: shows whether someone moved the whole model
-        # (a model built on the meta device keeps them on meta until its weights are loaded)
-        all_meta = all(t.device.type == "meta" for t in module.state_dict().values())
-        self._sanity_check_params = nn.ParameterList(
-            [nn.Parameter(torch.empty(0, device="meta" if all_meta else d), requires_grad=False) for d in self.devices]
-        )
+        # An empty parameter per rank that sits where the rank's shard belongs: `model.cuda()` / `model.to(...)` on
+        # the whole wrapper moves it, which forward() then notices. A model built on the meta device keeps them on
+        # meta until its weights are loaded.
+        on_meta = all(t.device.type == "meta" for t in module.state_dict().values())
+        markers = [torch.empty(0, device="meta" if on_meta else d) for d in self.devices]
+        self._sanity_check_params = nn.ParameterList([nn.Parameter(m, requires_grad=False) for m in markers])
         self.preserve_shards_when_saving: bool = True
         if sharded:
             self.apply_sharding(sharded_param_names)
+        if delay_init:
+            # The slicing engine works on the device, so the shards were cut there; they wait in host memory until
+            # the first forward puts them back (the reference builds them on the host, tensor_parallel.py:80-81).
+            # Flat ZeRO-3 shards belong to the sharding manager and stay where they are.
+            for shard in self.module_shards:
+                shard.to("cpu")
+
+    def _pick_output_rank(self, output_device, output_device_index) -> int:
+        if output_device is not None and output_device_index is not None:
+            raise AssertionError("output_device and output_device_index name the same thing: give one of them")
+        if output_device is None:
+            return 0 if output_device_index is None else output_device_index
+        wanted = canonicalize_device(output_device)
+        if wanted not in self.devices:
+            raise AssertionError(f"output_device {wanted} is not one of device_ids {list(self.devices)}")
+        return self.devices.index(wanted)
+
+    def _slice_into_shards(self, module: nn.Module, config_with_ops: Config) -> None:
+        """Queues every rank's slicing in one BatchSlicer per device and launches each once."""
+        world_size = len(self.devices)
+        slicers = {d: BatchSlicer(d if d.type == "cuda" else None) for d in dict.fromkeys(self.devices)}
+        self.modified_parameters_names = set()
+        for rank, device in enumerate(self.devices):
+            shard, touched = make_shard(module, device, config_with_ops, rank=rank, world_size=world_size, batch=slicers[device])
+            self.module_shards.append(shard)
+            self.modified_parameters_names |= set(touched)
+        self.sliced_bytes = sum(slicer.run() for slicer in slicers.values())
+        for device, slicer in slicers.items():
+            if device.type == "cuda" and slicer.plan is not None:
+                torch.cuda.synchronize(device)  # host sources uploaded for the launch are released by close()
+            slicer.close()
+
+    def _report_replication(self, params_before: int) -> None:
+        """Parameters the rules leave whole exist once per rank; say how much memory that costs."""
+        per_shard = [sum(p.numel() for p in shard.parameters()) for shard in self.module_shards]
+        if sum(per_shard) < params_before:
+            raise AssertionError(f"slicing lost parameters: {params_before} before, {per_shard} in the shards")
+        self.param_fractions = tuple(n / params_before for n in per_shard) if params_before else ()
+        extra = (sum(self.param_fractions) - 1) / len(self.devices)
+        logger.log(
+            logging.WARNING if extra >= 0.1 else logging.DEBUG,
+            "%d parameters became shards of %s parameters: %.3f%% of the model is held again on every device",
+            params_before, per_shard, extra * 100,
+        )
 
     def apply_sharding(self, replicated_param_names: Optional[Collection[str]] = None):
         if self.sharding_manager is not None:
-            raise Exception(
-                "Trying to apply sharding for the second time. If you wish NOT to apply sharding during model initialization, pass `sharded=False`."
-            )
+            raise Exception("sharding was applied a second time; construct with `sharded=False` to apply it yourself later")
         self.sharding_manager = Sharded(self, len(self.devices), replicated_param_names)
 
     def prepare_args_kwargs_for_forward(self, *args, **kwargs):
         """One copy of (args, kwargs) per rank; every tensor is moved to that rank's device (tensor_parallel.py:121-137).
         An attention cache object becomes that rank's own cache (see kv_cache)."""
+        if len(self.devices) > 1:
+            for name in LEGACY_CACHE_KWARGS:
+                if _holds_tensors(kwargs.get(name)):
+                    raise NotImplementedError(
+                        f"`{name}` is a tuple/list of key and value tensors. Every rank attends over its own heads, so such "
+                        "a cache cannot be handed to all ranks; pass a transformers Cache object (for example DynamicCache), "
+                        "which gets one sibling per rank, or none."
+                    )
         structure = (args, kwargs)
         flat = list(nested_flatten(structure))
         caches = {i: rank_caches(x, len(self.devices)) for i, x in enumerate(flat) if is_kv_cache(x)}
@@ -150,14 +177,18 @@ class TensorParallel(nn.Module):
         return zip(*per_rank)
 
     def forward(self, *args, **kwargs):
+        if self.need_delayed_init:  # shards parked on the host by delay_init=True (tensor_parallel.py:140-143)
+            for shard, device in zip(self.module_shards, self.devices):
+                shard.to(device)
+            self.need_delayed_init = False
         if self.sharding_manager is not None:
             self.sharding_manager.synchronize_weights(self.all_cuda)
         if len(self.module_shards) <= 1:
             return [self.module_shards[0](*args, **kwargs)][self.output_device_index]
         if not all(p.device == d for p, d in zip(self._sanity_check_params, self.devices) if p.device.type != "meta"):
             raise ValueError(
-                "Model parameters were moved to incorrect devices, did call on model.cuda() or "
-                "model.to(device)? If so, please avoid doing that"
+                "the shards are no longer on their devices: the whole TensorParallel module was moved "
+                "(`.cuda()` / `.to(device)`), which puts every rank on one device. Build it again instead."
             )
         inputs, kwargs_tup = self.prepare_args_kwargs_for_forward(*args, **kwargs)
         return parallel_apply_simple(self.module_shards, inputs, kwargs_tup, self.devices)[self.output_device_index]

@@ -39,11 +39,13 @@ def llama_7b_state():
     return state
 
 
-@pytest.mark.parametrize("world", [2, 8])
+@pytest.mark.parametrize("world", [2, 4, 8])
 def test_convert_llama2_7b_state_dict(world):
-    """Configuration 3: every shard of the whole dict in one launch. Checked by size-independent properties on
-    all tensors (shapes, integer checksums adding up, split -> undo identity on a subset) and bit for bit
-    against the oracle on rows sampled from four tensors."""
+    """Configuration 3: every shard of the whole dict in one launch. Checked on ALL tensors by size-independent
+    properties (shapes, integer checksums adding up, split -> undo identity) and bit for bit against
+    `torch.tensor_split` on the device (what the reference's Split computes, state_actions.py:47-48; with 32 heads
+    and W in {2, 4, 8} the head-aligned splits of q/k/v/o are the same ranges), and bit for bit against the oracle on
+    rows sampled from four tensors."""
     state = llama_7b_state()
     assert len(state) == 291
     cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=4096, num_attention_heads=32, num_key_value_heads=32), [DEV] * world)
@@ -61,6 +63,10 @@ def test_convert_llama2_7b_state_dict(world):
             continue
         assert sum(s.numel() for s in shards) == full.numel()
         assert sum(checksum(s) for s in shards) == checksum(full), name
+        action = next(a for p, a in cfg.state_rules.items() if p.search(name))
+        for r, piece in enumerate(torch.tensor_split(full, world, dim=action.dim)):
+            assert shards[r].is_contiguous() and torch.equal(shards[r], piece), (name, r)
+        assert torch.equal(action.undo(shards), full), name
     for name in ("model.layers.0.self_attn.o_proj.weight", "model.layers.31.mlp.down_proj.weight", "model.embed_tokens.weight", "lm_head.weight"):
         full = state[name]
         action = next(a for p, a in cfg.state_rules.items() if p.search(name))

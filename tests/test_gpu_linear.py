@@ -165,6 +165,27 @@ def test_llama_mlp_shard_prefill_4096_sampled_rows():
     assert torch.equal(_native.linear(h[1024:1536].contiguous(), wd), sub)
 
 
+def test_llama_mlp_shard_prefill_4096_every_output():
+    """BASELINE config 2 at M = 4096: all 4096 x 5504 hidden values and all 4096 x 4096 outputs against fp32 products of
+    the same bf16 inputs on the host (rtol 2e-2, absolute floor 2e-2 output standard deviations), then the fused sum
+    with the other rank's partial against torch's host add, bit for bit."""
+    d, f, M = 4096, 5504, 4096
+    x, wg, wu, wd = rnd((M, d), 1), rnd((f, d), 0, 0.02), rnd((f, d), 3, 0.02), rnd((d, f), 4, 0.02)
+    h = _native.swiglu_up(x.to(DEV), wg.to(DEV), wu.to(DEV))
+    y = _native.linear(h, wd.to(DEV))
+    h_cpu, y_cpu = h.cpu(), y.cpu()
+    h_want = ofw.gated_mlp_hidden(x.float(), wg.float(), wu.float())
+    sig_h = (0.02 * math.sqrt(d)) ** 2
+    torch.testing.assert_close(h_cpu.float(), h_want, rtol=RTOL_HALF, atol=RTOL_HALF * sig_h)
+    del h_want
+    y_want = F.linear(h_cpu.float(), wd.float())  # the down projection of the hidden the device produced
+    sig_y = 0.5 * sig_h * 0.02 * math.sqrt(f)
+    torch.testing.assert_close(y_cpu.float(), y_want, rtol=RTOL_HALF, atol=RTOL_HALF * sig_y)
+    other = rnd((M, d), 9, 0.3)
+    fused = _native.linear(h, wd.to(DEV), addend=other.to(DEV))
+    assert torch.equal(fused.cpu(), y_cpu + other)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(40, 136, 5504), (130, 260, 1536), (300, 64, 2048), (17, 512, 1024)])
 @pytest.mark.parametrize("splits", [1, 3, 8])

@@ -149,3 +149,23 @@ def test_opt_125m_tensor_parallel_logits():
     assert out.shape == (2, 64, 50272)
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=3e-3)
     assert (out.cpu() - ref).abs().max().item() < 1e-3
+
+
+def test_delay_init_parks_shards_on_the_host_until_the_first_forward():
+    """`delay_init=True` (reference tensor_parallel.py:33,80-81,140-143): after construction the shards hold no device
+    memory, the first forward moves every rank's shard to its device, and the result equals the eager build's."""
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Embedding(50, 32), torch.nn.Linear(32, 64), torch.nn.ReLU(), torch.nn.Linear(64, 24))
+    ids = torch.randint(0, 50, (3, 7))
+    devices = ["cuda:0", "cuda:0"]
+    eager = tp.TensorParallel(model, devices, sharded=False)
+    lazy = tp.TensorParallel(model, devices, sharded=False, delay_init=True)
+    assert lazy.need_delayed_init
+    assert all(p.device.type == "cpu" for shard in lazy.module_shards for p in shard.parameters())
+    for a, b in zip(eager.module_shards.parameters(), lazy.module_shards.parameters()):
+        assert torch.equal(a.cpu(), b)
+    out = lazy(ids.to("cuda:0"))
+    assert not lazy.need_delayed_init
+    assert all(p.device == torch.device("cuda", 0) for shard in lazy.module_shards for p in shard.parameters())
+    assert torch.equal(out, eager(ids.to("cuda:0")))
+    torch.testing.assert_close(out.cpu(), model(ids), rtol=1e-5, atol=1e-5)

@@ -72,6 +72,24 @@ def test_falcon_mlp_shard_full_shape():
     torch.testing.assert_close(down.double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * scale_y)
 
 
+@pytest.mark.parametrize("M", [1, 16, 32, 64])
+def test_falcon_mlp_shard_full_shape_every_decode_batch(M):
+    """BASELINE config 5 at its real shape through the DEFAULT dispatch at batch 1, 16, 32 and 64 (the row-streaming
+    kernel at 1, the K-split kernel from 12 rows on at this size): both matrices against the closed-form definition in
+    float64. The down projection is fed the device's own hidden activations."""
+    d, f = 8192, 16384
+    x, wq1, s1, c1, o1 = make_case(M, f, d, 41, torch.float16, 0)
+    dev = lambda a, dt=None: (torch.from_numpy(a) if dt is None else torch.from_numpy(a).to(dt)).to(DEV)  # noqa: E731
+    up = _native.linear_w8(x.to(DEV), dev(wq1), dev(s1), dev(c1.astype(np.int32)), dev(o1, torch.float16), act=_native.ACT_GELU)
+    want_up = torch.nn.functional.gelu(torch.from_numpy(oq.linear_w8_f64(x.float().numpy(), wq1, s1, c1, o1)))
+    torch.testing.assert_close(up.double().cpu(), want_up, rtol=2e-2, atol=2e-2 * 0.02 * math.sqrt(d + 400 * 41))
+    del wq1, want_up
+    _, wq2, s2, c2, o2 = make_case(1, d, f, 82, torch.float16, 1)
+    down = _native.linear_w8(up, dev(wq2), dev(s2), dev(c2.astype(np.int32)), dev(o2, torch.float16))
+    want_down = oq.linear_w8_f64(up.cpu().float().numpy(), wq2, s2, c2, o2)
+    torch.testing.assert_close(down.double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * float(np.abs(want_down).std()))
+
+
 @pytest.fixture
 def column_groups(tune):
     """Forces the number of 16-column groups per block of the decode kernel (a debugging knob of the library;

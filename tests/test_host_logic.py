@@ -360,3 +360,174 @@ def test_rank_threads_take_turns_between_rendezvous():
     want = sum(sum(r + step for r in range(world)) for step in range(5))
     assert results == {r: want for r in range(world)}
     assert turn.acquire(blocking=False)
+
+
+# ---------------------------------------------------------------------------------------- wrapper protocol
+class _Recorder(torch.nn.Module):
+    def forward(self, *args, **kwargs):
+        self.seen = (args, kwargs)
+        return self.result
+
+
+def test_wrapper_routes_rules_by_position_and_name():
+    """Input rules address positions and keyword names, output rules positions / keys / 0 for a bare tensor; a keyword
+    the caller left out reaches its action as None (reference wrapper.py:31-48)."""
+    from tensor_parallel_amd.wrapper import TensorParallelWrapper, apply_action, process_input, process_output
+
+    calls = []
+
+    def tag(label):
+        def act(value, rank):
+            calls.append((label, value, rank))
+            return (label, value)
+        return act
+
+    args, kwargs = process_input({0: tag("a"), "mask": tag("m"), "absent": tag("n"), 5: tag("never")}, 1, 2, "x0", "x1", mask="M")
+    assert args == [("a", "x0"), "x1"] and kwargs == {"mask": ("m", "M"), "absent": ("n", None)}
+    assert ("never", None, 1) not in calls and all(rank == 1 for _, _, rank in calls)
+    # (split, undo) pairs act with their first half
+    assert apply_action("v", (tag("first"), tag("second")), rank=0, world_size=2) == ("first", "v")
+    with pytest.raises(Exception, match="unexpected action"):
+        apply_action(torch.zeros(2), "transpose 0", rank=0, world_size=2)
+
+    t = torch.zeros(1)
+    assert process_output(t, {0: tag("o")}, rank=0, world_size=2) == ("o", t)
+    assert process_output(t, {}, rank=0, world_size=2) is t
+    out = process_output((1, 2, 3), {1: tag("o")}, rank=0, world_size=2)
+    assert out == (1, ("o", 2), 3) and isinstance(out, tuple)
+    assert process_output([1, 2], {0: tag("o")}, rank=0, world_size=2) == [("o", 1), 2]
+    d = {"logits": 7, "other": 8}
+    assert process_output(d, {"logits": tag("o")}, rank=0, world_size=2) is d and d["logits"] == ("o", 7)
+
+    inner = _Recorder()
+    inner.result = (10, 20)
+    inner.hidden_size = 64
+    w = TensorParallelWrapper(inner, {0: tag("in")}, {0: tag("out")}, rank=1, world_size=2)
+    assert w("p", q="r") == (("out", 10), 20)
+    assert inner.seen == ((("in", "p"),), {"q": "r"})
+    # attributes of the wrapped module are reachable through the wrapper, its own come first
+    assert w.hidden_size == 64 and w.rank == 1 and w.tp_wrapped_module is inner
+    with pytest.raises(AttributeError):
+        w.no_such_attribute
+    assert [n for n, _ in w.named_modules()] == ["", "tp_wrapped_module"]
+
+
+def test_legacy_tuple_kv_cache_is_refused_for_several_ranks():
+    """A tuple of key/value tensors holds one rank's heads; handing it to every rank would be silently wrong."""
+    from tensor_parallel_amd.tensor_parallel import TensorParallel
+
+    tp_model = TensorParallel.__new__(TensorParallel)
+    torch.nn.Module.__init__(tp_model)
+    tp_model.devices = (torch.device("cuda", 0), torch.device("cuda", 0))
+    legacy = ((torch.zeros(1, 2, 3, 4), torch.zeros(1, 2, 3, 4)),)
+    for name in ("past_key_values", "past_key_value", "layer_past"):
+        with pytest.raises(NotImplementedError, match="Cache object"):
+            tp_model.prepare_args_kwargs_for_forward(torch.zeros(1), **{name: legacy})
+    tp_model.devices = (torch.device("cpu"),)
+    tp_model.prepare_args_kwargs_for_forward(torch.zeros(1), past_key_values=legacy)  # one rank: nothing to split
+
+
+def test_delay_init_and_output_device_arguments():
+    from tensor_parallel_amd.tensor_parallel import TensorParallel
+
+    lin = torch.nn.Linear(4, 4)
+    one = TensorParallel(lin, device_ids=["cpu"], delay_init=True)
+    assert one.need_delayed_init and one.module_shards[0] is lin and one.output_device_index == 0
+    with pytest.raises(AssertionError):
+        TensorParallel(lin, device_ids=["cpu"], output_device="cpu", output_device_index=0)
+    with pytest.raises(AssertionError):
+        TensorParallel(lin, device_ids=["cpu"], output_device="cuda:0")
+
+
+def test_native_wrappers_validate_operands_before_any_launch():
+    """Shapes, dtypes and devices the C ABI cannot see are checked in Python: a wrong operand raises instead of being
+    dereferenced by a kernel. Runs without a GPU: every check fires before the library is reached."""
+    meta = torch.device("meta")
+    x = torch.empty(4, 64, dtype=torch.float16, device=meta)
+
+    class OnGpu(torch.Tensor):
+        """A tensor that claims to live on cuda:0, for the device checks."""
+
+    def fake(shape, dtype, device="cuda:0"):
+        t = torch.empty(shape, dtype=dtype, device=meta)
+        t.__class__ = OnGpu
+        OnGpu.device = property(lambda self: self._dev)
+        t._dev = torch.device(device)
+        return t
+
+    xg = fake((4, 64), torch.float16)
+    wq = fake((32, 64), torch.int8)
+    sc = fake((32,), torch.float32)
+    with pytest.raises(_native.NativeLibraryError):
+        _native.linear_w8(x, wq, sc, None, None)  # x not on a HIP device
+    with pytest.raises(ValueError, match="input features"):
+        _native.linear_w8(xg, fake((32, 48), torch.int8), sc, None, None)
+    with pytest.raises(ValueError, match="scale must have shape"):
+        _native.linear_w8(xg, wq, fake((16,), torch.float32), None, None)
+    with pytest.raises(ValueError, match="wq on"):
+        _native.linear_w8(xg, fake((32, 64), torch.int8, "cuda:1"), sc, None, None)
+    with pytest.raises(ValueError, match="bias must have shape"):
+        _native.linear_w8(xg, wq, sc, None, None, bias=fake((31,), torch.float16))
+    with pytest.raises(ValueError, match="bias on"):
+        _native.linear_w8(xg, wq, sc, None, None, bias=fake((32,), torch.float16, "cuda:1"))
+    with pytest.raises(TypeError):
+        _native.linear_w8(fake((4, 64), torch.float32), wq, sc, None, None)
+    w = fake((32, 64), torch.float16)
+    with pytest.raises(ValueError, match="w on"):
+        _native.linear(xg, fake((32, 64), torch.float16, "cuda:1"))
+    with pytest.raises(ValueError, match="bias"):
+        _native.linear(xg, w, bias=fake((32,), torch.float16, "cuda:1"))
+    with pytest.raises(ValueError, match="wu on"):
+        _native.swiglu_up(xg, w, fake((32, 64), torch.float16, "cuda:1"))
+    q = fake((1, 2, 3, 64), torch.float16)
+    with pytest.raises(ValueError, match="k on"):
+        _native.attention(q, fake((1, 2, 3, 64), torch.float16, "cuda:1"), fake((1, 2, 3, 64), torch.float16))
+
+
+def test_infer_sharded_device_map_names_and_devices():
+    """Every parameter, buffer and tied alias of a tensor-parallel model maps to the device of the rank whose index its
+    name carries (reference dispatch.py:35-72)."""
+    from tensor_parallel_amd.dispatch import infer_sharded_data_device_id, infer_sharded_device_map
+
+    assert infer_sharded_data_device_id("wrapped_model.module_shards.3.model.layers.0.mlp.tp_wrapped_module.up_proj.weight") == 3
+    assert infer_sharded_data_device_id("_sanity_check_params.1") == 1
+    assert infer_sharded_data_device_id("wrapped_model.sharding_manager.flat_shards.2") == 2
+    assert infer_sharded_data_device_id("module_shards.10.bias") == 10
+    with pytest.raises(KeyError):
+        infer_sharded_data_device_id("model.layers.0.weight")
+
+    class Shard(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = torch.nn.Embedding(8, 4)
+            self.head = torch.nn.Linear(4, 8, bias=False)
+            self.head.weight = self.emb.weight  # tied
+            self.register_buffer("steps", torch.zeros(1))
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.module_shards = torch.nn.ModuleList([Shard(), Shard()])
+            self._sanity_check_params = torch.nn.ParameterList([torch.nn.Parameter(torch.empty(0)) for _ in range(2)])
+            self.devices = (torch.device("cuda", 0), torch.device("cuda", 1))
+
+    dm = infer_sharded_device_map(Model())
+    want = {}
+    for r in range(2):
+        dev = torch.device("cuda", r)
+        want.update({f"module_shards.{r}.emb.weight": dev, f"module_shards.{r}.head.weight": dev,
+                     f"module_shards.{r}.steps": dev, f"_sanity_check_params.{r}": dev})
+    assert dm == want
+
+
+def test_reference_import_name_serves_the_same_objects():
+    """`import tensor_parallel as tp`, the reference's import name, and its submodule paths."""
+    import tensor_parallel as ref_name
+    from tensor_parallel.slicing_configs import get_llama_config as by_ref_path
+    from tensor_parallel.state_actions import Split as split_by_ref_path
+
+    for name in ("Config", "TensorParallel", "tensor_parallel", "convert_state_dict", "infer_sharded_device_map",
+                 "save_tensor_parallel", "Sharded", "StateAction"):
+        assert getattr(ref_name, name) is getattr(tp, name)
+    assert by_ref_path is get_llama_config and split_by_ref_path is tp.Split
+    assert ref_name.tensor_parallel.__module__ == "tensor_parallel_amd.factory"
