@@ -188,7 +188,7 @@ def ceilings(torch, _native, dev) -> int:
     probes.tpamd_probe_mfma.argtypes = [ci, vp, vp, ci, ci, vp]
     probes.tpamd_probe_mfma_flops.restype = ctypes.c_double
     probes.tpamd_probe_mfma_flops.argtypes = [ci, ci, ci]
-    probes.tpamd_probe_stream.argtypes = [ci, vp, vp, u64, ci, vp, vp]
+    probes.tpamd_probe_stream.argtypes = [ci, ci, ci, vp, vp, u64, ci, vp, vp]
     stream = lambda: vp(torch.cuda.current_stream(dev).cuda_stream)  # noqa: E731
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     sink = torch.zeros(256, device=dev)
@@ -229,18 +229,21 @@ def ceilings(torch, _native, dev) -> int:
     sizes = (("llama7b_down_shard_45MB", FFN_SHARD * D_MODEL * 2, 6), ("llama7b_gate_up_shards_90MB", 2 * FFN_SHARD * D_MODEL * 2, 4),
              ("llama2_7b_split_tensors_13.5GB", 13476298752, 1))
     for label, nbytes, copies in sizes:
-        nbytes = nbytes // 16384 * 16384
+        nbytes = nbytes // 32768 * 32768
         srcs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
         dsts = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(copies)]
         row = {}
         for mode, what, moved in ((0, "read_only", nbytes), (1, "write_only", nbytes), (2, "copy_read_plus_write", 2 * nbytes)):
-            best = None
-            for per_cu in (4, 8, 16):
-                us = settled_us(lambda i: probes.tpamd_probe_stream(mode, vp(srcs[i % copies].data_ptr()), vp(dsts[i % copies].data_ptr()),
-                                                                    nbytes, cus * per_cu, vp(sink.data_ptr()), stream()), 0.15, 20 if nbytes < 1e9 else 5)
-                if best is None or us < best[0]:
-                    best = (us, per_cu)
-            row[what] = {"us": best[0], "GBps": moved / best[0] / 1e3, "frac_of_8000": moved / best[0] / 1e3 / PEAK_HBM_GBS, "blocks_per_cu": best[1]}
+            best = None  # best of: plain / non-temporal accesses, 4 / 16 / 32 KiB per block step, 4 / 8 / 16 blocks per CU
+            for nt in (1, 0):
+                for piece in (4096, 16384, 32768):
+                    for per_cu in (4, 8, 16):
+                        us = settled_us(lambda i: probes.tpamd_probe_stream(mode, nt, piece, vp(srcs[i % copies].data_ptr()), vp(dsts[i % copies].data_ptr()),
+                                                                            nbytes, cus * per_cu, vp(sink.data_ptr()), stream()), 0.05, 20 if nbytes < 1e9 else 4)
+                        if best is None or us < best[0]:
+                            best = (us, per_cu, nt, piece)
+            row[what] = {"us": best[0], "GBps": moved / best[0] / 1e3, "frac_of_8000": moved / best[0] / 1e3 / PEAK_HBM_GBS, "blocks_per_cu": best[1],
+                         "non_temporal": bool(best[2]), "piece_bytes": best[3]}
         us = settled_us(lambda i: dsts[i % copies].copy_(srcs[i % copies]), 0.15, 20 if nbytes < 1e9 else 5)
         row["device_to_device_copy_of_the_runtime"] = {"us": us, "GBps": 2 * nbytes / us / 1e3, "frac_of_8000": 2 * nbytes / us / 1e3 / PEAK_HBM_GBS}
         streams[label] = row

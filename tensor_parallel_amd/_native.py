@@ -163,8 +163,37 @@ def require_device(t: torch.Tensor, what: str) -> None:
         )
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream_ptr(device: torch.device) -> int:
+    """Handle of torch's current stream on `device` (the stream every kernel of a call is enqueued on)."""
+    if _raw_stream is not None:
+        index = device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """`with _on_device(dev):` makes `dev` the current HIP device for the call; costs nothing when it already is."""
+
+    __slots__ = ("index", "prev")
+
+    def __init__(self, device: torch.device):
+        self.index = device.index
+
+    def __enter__(self):
+        self.prev = None
+        if self.index is not None:
+            cur = torch.cuda.current_device()
+            if cur != self.index:
+                self.prev = cur
+                torch.cuda.set_device(self.index)
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 class CopyPlan:
@@ -177,7 +206,7 @@ class CopyPlan:
         arr = (CopyJob * max(len(jobs), 1))()
         for i, j in enumerate(jobs):
             arr[i] = CopyJob(*j)
-        with torch.cuda.device(device):
+        with _on_device(device):
             _check(lib().tpamd_copy_plan_create(arr, len(jobs), ctypes.byref(self._handle)), "tpamd_copy_plan_create")
         self.n_jobs = len(jobs)
 
@@ -186,7 +215,7 @@ class CopyPlan:
         return int(lib().tpamd_copy_plan_bytes(self._handle))
 
     def run(self, stream_ptr: Optional[int] = None) -> None:
-        with torch.cuda.device(self.device):
+        with _on_device(self.device):
             if stream_ptr is None:
                 stream_ptr = current_stream_ptr(self.device)
             _check(lib().tpamd_copy_plan_run(self._handle, ctypes.c_void_p(stream_ptr)), "tpamd_copy_plan_run")
@@ -212,7 +241,7 @@ def run_copy_jobs(jobs: Sequence[tuple], device: torch.device) -> None:
     through a plan, which is destroyed once its launch has finished."""
     if not jobs:
         return
-    with torch.cuda.device(device):
+    with _on_device(device):
         if len(jobs) <= SMALL_COPY_MAX_JOBS:
             arr = (CopyJob * len(jobs))(*[CopyJob(*j) for j in jobs])
             _check(lib().tpamd_copy_jobs_run(arr, len(jobs), ctypes.c_void_p(current_stream_ptr(device))), "tpamd_copy_jobs_run")
@@ -227,7 +256,7 @@ def scale(inp: torch.Tensor, world_size: int, multiply: bool = False) -> torch.T
     require_device(inp, "scale")
     src = inp.contiguous()
     out = torch.empty_like(src)
-    with torch.cuda.device(src.device):
+    with _on_device(src.device):
         _check(
             lib().tpamd_scale(src.data_ptr(), out.data_ptr(), src.numel(), dtype_code(src.dtype), world_size,
                               1 if multiply else 0, ctypes.c_void_p(current_stream_ptr(src.device))),
@@ -249,7 +278,7 @@ def reduce_partials(parts: Sequence[torch.Tensor], accum: int = ACCUM_STEPWISE, 
     if out is None:
         out = torch.empty_like(keep[0])
     ptrs = (ctypes.c_void_p * len(keep))(*[p.data_ptr() for p in keep])
-    with torch.cuda.device(first.device):
+    with _on_device(first.device):
         _check(
             lib().tpamd_reduce_partials(ptrs, len(keep), out.data_ptr(), first.numel(), dtype_code(first.dtype), accum,
                                         ctypes.c_void_p(current_stream_ptr(first.device))),
@@ -259,6 +288,8 @@ def reduce_partials(parts: Sequence[torch.Tensor], accum: int = ACCUM_STEPWISE, 
 
 
 def _as_2d(x: torch.Tensor) -> torch.Tensor:
+    if x.dim() == 2 and x.is_contiguous():
+        return x
     x2 = x.reshape(-1, x.shape[-1])
     if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
         x2 = x2.contiguous()
@@ -277,7 +308,7 @@ def reload_tuning() -> None:
 def scratch_of_stream(device: torch.device, stream_ptr: Optional[int] = None) -> tuple:
     """(address, bytes) of the K-split scratch buffer that work on the stream uses, (None, 0) while it has none."""
     ptr, nbytes = ctypes.c_void_p(), ctypes.c_uint64()
-    with torch.cuda.device(device):
+    with _on_device(device):
         if stream_ptr is None:
             stream_ptr = current_stream_ptr(device)
         _check(lib().tpamd_scratch_query(ctypes.c_void_p(stream_ptr), ctypes.byref(ptr), ctypes.byref(nbytes)), "tpamd_scratch_query")
@@ -311,7 +342,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
     y = torch.empty((M, N), dtype=x.dtype, device=x.device) if out is None else out.view(M, N)
     b = bias.contiguous() if bias is not None else None
     a2 = _as_2d(addend) if addend is not None else None
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         stream = ctypes.c_void_p(current_stream_ptr(x.device))
         if a2 is None:
             _check(
@@ -344,7 +375,7 @@ def swiglu_up(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor) -> torch.Tens
     M, K = x2.shape
     N = g2.shape[0]
     h = torch.empty((M, N), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _check(
             lib().tpamd_swiglu_up(x2.data_ptr(), g2.data_ptr(), u2.data_ptr(), h.data_ptr(), M, N, K, _ld(x2), _ld(g2), N,
                                   dtype_code(x.dtype), ctypes.c_void_p(current_stream_ptr(x.device))),
@@ -370,7 +401,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional
     out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
     strides = (ctypes.c_int64 * 12)(q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
                                     v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2))
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         _check(
             lib().tpamd_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, Hq, Hkv, Sq, Skv, D, strides,
                                   float(scale if scale is not None else D ** -0.5), 1 if causal else 0, dtype_code(q.dtype),
@@ -411,7 +442,7 @@ def linear_w8(x: torch.Tensor, wq: torch.Tensor, scale_: torch.Tensor, outlier_i
         outlier_idx = outlier_idx.contiguous()
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     b = bias.contiguous() if bias is not None else None
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _check(
             lib().tpamd_linear_w8(x2.data_ptr(), wq.data_ptr(), scale_.contiguous().data_ptr(),
                                   outlier_idx.data_ptr() if n_out else None, w_out.data_ptr() if n_out else None, n_out,

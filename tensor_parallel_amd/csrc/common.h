@@ -45,11 +45,11 @@ struct Tuning {
     int skinny_cg;           // TPAMD_SKINNY_CG: column groups per block (1, 2, 4)
     int skinny_pair;         // TPAMD_SKINNY_PAIR: 8-column form of the gated pair
     int skinny_resident;     // TPAMD_SKINNY_RESIDENT: x-resident kernel on/off
-    int gemv_persistent;     // TPAMD_GEMV_PERSISTENT: 0 = one block per group of rows instead of the persistent grid
     int w8_split;            // TPAMD_W8_SPLIT: int8 K-split kernel on/off
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel
     int copy_tile_units;     // TPAMD_COPY_TILE_UNITS: 16-byte units per copy tile
     int copy_blocks_per_cu;  // TPAMD_COPY_BLOCKS_PER_CU
+    int copy_nt;             // TPAMD_COPY_NT: bit 0 non-temporal loads, bit 1 non-temporal stores of the slicing kernel
 };
 const Tuning &tuning();
 

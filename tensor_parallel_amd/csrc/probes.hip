@@ -13,16 +13,19 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
-// One wavefront per SIMD (4 per block, one block per CU), 32 independent accumulator tiles: the issue pattern of the
-// GEMM kernels' inner loop without its loads and LDS reads. SHAPE 16: v_mfma_f32_16x16x32_bf16, 32: 32x32x16.
+// One wavefront per SIMD (4 per block, one block per CU), 16 or 8 independent accumulator tiles in AGPRs that are
+// accumulated in place: the issue pattern of the GEMM kernels' inner loop without its loads and LDS reads. The MFMAs are
+// written as asm so that nothing but them (and the loop counter) is in the loop.
+// SHAPE 16: v_mfma_f32_16x16x32_bf16 (16 tiles), 32: v_mfma_f32_32x32x16_bf16 (8 tiles).
 template <int SHAPE>
 __global__ __launch_bounds__(256) void mfma_loop_kernel(const uint4 *operands, float *sink, int iters) {
     const int tid = blockIdx.x * 256 + threadIdx.x;
-    uint4 a[4], b[4];
+    v4u a[4], b[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        a[i] = operands[tid * 8 + i];
-        b[i] = operands[tid * 8 + 4 + i];
+        const uint4 av = operands[tid * 8 + i], bv = operands[tid * 8 + 4 + i];
+        a[i] = v4u{av.x, av.y, av.z, av.w};
+        b[i] = v4u{bv.x, bv.y, bv.z, bv.w};
     }
     float s = 0.f;
     if constexpr (SHAPE == 32) {
@@ -34,7 +37,7 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(const uint4 *operands, f
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[i & 3]), __builtin_bit_cast(bf16x8, b[(i >> 1) & 3]), acc[i], 0, 0, 0);
+                asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a[i & 3]), "v"(b[(i >> 1) & 3]));
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) s += acc[i][0];
@@ -45,7 +48,7 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(const uint4 *operands, f
         for (int it = 0; it < iters; ++it) {
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[i & 3]), __builtin_bit_cast(bf16x8, b[(i >> 2) & 3]), acc[i], 0, 0, 0);
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a[i & 3]), "v"(b[(i >> 2) & 3]));
         }
 #pragma unroll
         for (int i = 0; i < 16; ++i) s += acc[i][0];
@@ -53,25 +56,40 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(const uint4 *operands, f
     if (s == 123.456f) sink[threadIdx.x] = s;  // keeps the loop alive; never true for these operands
 }
 
-// MODE 0: read src, 1: write dst, 2: copy src -> dst. A persistent grid; block b handles 16 KiB pieces b, b + grid, ...
-template <int MODE>
+// MODE 0: read src, 1: write dst, 2: copy src -> dst. A persistent grid; block b handles pieces b, b + grid, ... of
+// PIECE bytes (256 threads x 16 bytes x PIECE / 4096 accesses in flight per thread). NT: non-temporal accesses.
+template <int MODE, bool NT, int PIECE>
 __global__ __launch_bounds__(256) void stream_kernel(const char *src, char *dst, uint64_t pieces, float *sink) {
+    constexpr int U = PIECE / 4096;
     uint32_t keep = 0;
     for (uint64_t p = blockIdx.x; p < pieces; p += gridDim.x) {
-        const uint64_t off = p * 16384 + threadIdx.x * 16;
-        v4u v[4];
+        const uint64_t off = p * PIECE + threadIdx.x * 16;
+        v4u v[U];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if constexpr (MODE != 1) v[i] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(src + off + i * 4096));
-            else v[i] = v4u{static_cast<uint32_t>(p), 1u, 2u, 3u};
+        for (int i = 0; i < U; ++i) {
+            if constexpr (MODE == 1) v[i] = v4u{static_cast<uint32_t>(p), 1u, 2u, 3u};
+            else if constexpr (NT) v[i] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(src + off + i * 4096));
+            else v[i] = *reinterpret_cast<const v4u *>(src + off + i * 4096);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if constexpr (MODE != 0) __builtin_nontemporal_store(v[i], reinterpret_cast<v4u *>(dst + off + i * 4096));
-            else keep ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+        for (int i = 0; i < U; ++i) {
+            if constexpr (MODE == 0) keep ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+            else if constexpr (NT) __builtin_nontemporal_store(v[i], reinterpret_cast<v4u *>(dst + off + i * 4096));
+            else *reinterpret_cast<v4u *>(dst + off + i * 4096) = v[i];
         }
     }
     if (MODE == 0 && keep == 0x12345679u) sink[threadIdx.x] = 1.f;
+}
+
+template <int MODE>
+void launch_stream(bool nt, int piece, int blocks, hipStream_t s, const char *src, char *dst, uint64_t bytes, float *sink) {
+    const uint64_t pieces = bytes / piece;
+#define TPAMD_PROBE_CASE(NTV, P) \
+    if (nt == NTV && piece == P) hipLaunchKernelGGL((stream_kernel<MODE, NTV, P>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink)
+    TPAMD_PROBE_CASE(true, 16384); TPAMD_PROBE_CASE(false, 16384);
+    TPAMD_PROBE_CASE(true, 32768); TPAMD_PROBE_CASE(false, 32768);
+    TPAMD_PROBE_CASE(true, 4096); TPAMD_PROBE_CASE(false, 4096);
+#undef TPAMD_PROBE_CASE
 }
 
 }  // namespace
@@ -91,17 +109,18 @@ extern "C" double tpamd_probe_mfma_flops(int shape, int blocks, int iters) {
     return per_wave_iter * 4.0 * blocks * iters;
 }
 
-// mode 0 read, 1 write, 2 copy; bytes must be a multiple of 16384.
-extern "C" int tpamd_probe_stream(int mode, const void *src_dev, void *dst_dev, uint64_t bytes, int blocks, void *sink_dev, void *stream) {
-    if (bytes % 16384 != 0 || blocks <= 0) return -1;
+// mode 0 read, 1 write, 2 copy; nt != 0: non-temporal accesses; piece: 4096, 16384 or 32768 bytes per block step;
+// bytes must be a multiple of 32768.
+extern "C" int tpamd_probe_stream(int mode, int nt, int piece, const void *src_dev, void *dst_dev, uint64_t bytes, int blocks,
+                                  void *sink_dev, void *stream) {
+    if (bytes % 32768 != 0 || blocks <= 0 || (piece != 4096 && piece != 16384 && piece != 32768)) return -1;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const uint64_t pieces = bytes / 16384;
     const char *src = static_cast<const char *>(src_dev);
     char *dst = static_cast<char *>(dst_dev);
     float *sink = static_cast<float *>(sink_dev);
-    if (mode == 0) hipLaunchKernelGGL((stream_kernel<0>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink);
-    else if (mode == 1) hipLaunchKernelGGL((stream_kernel<1>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink);
-    else if (mode == 2) hipLaunchKernelGGL((stream_kernel<2>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink);
+    if (mode == 0) launch_stream<0>(nt != 0, piece, blocks, s, src, dst, bytes, sink);
+    else if (mode == 1) launch_stream<1>(nt != 0, piece, blocks, s, src, dst, bytes, sink);
+    else if (mode == 2) launch_stream<2>(nt != 0, piece, blocks, s, src, dst, bytes, sink);
     else return -1;
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }

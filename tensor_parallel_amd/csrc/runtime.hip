@@ -28,11 +28,11 @@ Tuning read_tuning() {
     t.skinny_cg = env_int("TPAMD_SKINNY_CG");
     t.skinny_pair = env_int("TPAMD_SKINNY_PAIR");
     t.skinny_resident = env_int("TPAMD_SKINNY_RESIDENT");
-    t.gemv_persistent = env_int("TPAMD_GEMV_PERSISTENT");
     t.w8_split = env_int("TPAMD_W8_SPLIT");
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
     t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");
     t.copy_blocks_per_cu = env_int("TPAMD_COPY_BLOCKS_PER_CU");
+    t.copy_nt = env_int("TPAMD_COPY_NT");
     return t;
 }
 

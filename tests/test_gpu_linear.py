@@ -381,3 +381,19 @@ def test_other_dispatch_paths_inside_a_hip_graph(case, tune):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         assert torch.equal(fn(), eager)  # eager work between replays
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 2, 3])
+@pytest.mark.parametrize("N,K", [(2048, 512), (2053, 520), (4100, 5504), (6000, 1032), (3000, 8192)])
+def test_row_streaming_kernel_on_wide_matrices(dtype, M, N, K):
+    """M <= 3 and thousands of output columns (ragged column count, ragged last K step): against the fp32 host
+    product, the gated pair against the oracle, the fused sum bit for bit."""
+    x, w, w2, b = rnd((M, K), 1, 1.0, dtype).to(DEV), rnd((N, K), 0, 0.02, dtype).to(DEV), rnd((N, K), 5, 0.02, dtype).to(DEV), rnd((N,), 2, 0.1, dtype).to(DEV)
+    lin = _native.linear(x, w, b)
+    check_half(lin, F.linear(x.float().cpu(), w.float().cpu(), b.float().cpu()), K)
+    sw = _native.swiglu_up(x, w, w2)
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(sw.float().cpu(), ofw.gated_mlp_hidden(x.float().cpu(), w.float().cpu(), w2.float().cpu()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    other = rnd((M, N), 7, 1.0, dtype).to(DEV)
+    assert torch.equal(_native.linear(x, w, b, addend=other).cpu(), lin.cpu() + other.cpu())

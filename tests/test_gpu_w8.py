@@ -187,3 +187,15 @@ def test_k_split_kernel_inside_a_hip_graph(tune):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         assert torch.equal(_native.linear_w8(*args), eager)  # eager work between replays
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 2, 3])
+@pytest.mark.parametrize("N,K,n_out", [(2048, 1024, 0), (2100, 2064, 7), (4096, 4096, 41)])
+def test_int8_row_streaming_kernel_on_wide_matrices(dtype, M, N, K, n_out):
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, dtype, seed=4)
+    args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+            torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None, torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None)
+    got = _native.linear_w8(*args)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * 0.02 * math.sqrt(K + 400 * n_out))
