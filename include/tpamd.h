@@ -19,10 +19,11 @@
  *     the partial results: one per (device, stream), 64 MiB on a 256-CU part, allocated with hipMalloc at the
  *     stream's first such call and kept until the process ends (at most 8 streams per device get one; calls on
  *     further streams run unsplit). Streams never share a buffer, so such calls on different streams of a device
- *     need no ordering among themselves. If a stream's first such call happens under stream capture, nothing is
- *     allocated and the call runs unsplit (slower, same result up to summation order). A captured graph keeps
- *     using the buffer of the stream it was captured on: replaying it on another stream while that stream runs
- *     K-split work is for the caller to order.
+ *     need no ordering among themselves. Nothing can be allocated while a stream is being captured: the first
+ *     allocation on a device therefore sets one spare buffer aside, which the first capturing stream without a
+ *     buffer of its own takes over; a capture that finds neither runs the call unsplit (slower, same result up to
+ *     summation order). A captured graph keeps using the buffer of the stream it was captured on: replaying it
+ *     on another stream while the capture stream runs K-split work is for the caller to order.
  *   - tuning knobs (environment variables TPAMD_*) are read once, when the library is loaded.
  */
 #ifndef TPAMD_H

@@ -64,6 +64,7 @@ namespace {
 struct Entry {
     int dev;
     hipStream_t stream;
+    bool spare;  // set aside for the first capturing stream that needs one; `stream` means nothing until then
     void *ptr;
     size_t bytes;
 };
@@ -81,26 +82,12 @@ std::mutex &splitk_mutex() {
 // *out = a buffer of at least `need` bytes for work on `stream` of device `dev` (the current device), or NULL: then the
 // caller runs its unsplit form. A stream's buffer is allocated at its first use with max(need, reserve) bytes and kept
 // until the process ends; streams of one device never share one, so K-split work on different streams cannot meet in
-// it. NULL comes back when the stream has no buffer yet and is being captured (allocating is not allowed then), when
-// `need` is larger than the stream's buffer, and for the ninth stream of a device.
+// it. Allocating is not allowed while a stream is being captured, so the first allocation on a device also sets one
+// spare buffer aside, and the first capturing stream that has no buffer of its own takes it over (frameworks capture
+// on a stream of their own that runs nothing else). NULL comes back when a capturing stream finds no spare, when `need`
+// is larger than the stream's buffer, and for the ninth buffer of a device.
 // Inside a StaticScratchScope (noalloc.hip) the library's fixed array is handed out instead.
-int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
-    *out = nullptr;
-    if (static_scratch_active()) return static_scratch(dev, need, out);
-    int on_device = 0;
-    for (Entry &e : g_cache) {
-        if (e.dev != dev) continue;
-        ++on_device;
-        if (e.stream == stream) {
-            if (e.bytes >= need) *out = e.ptr;
-            return TPAMD_OK;
-        }
-    }
-    if (on_device >= MAX_BUFFERS_PER_DEVICE) return TPAMD_OK;
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    TPAMD_HIP(hipStreamIsCapturing(stream, &capturing));
-    if (capturing != hipStreamCaptureStatusNone) return TPAMD_OK;
-    const size_t bytes = need > reserve ? need : reserve;
+static int allocate_entry(int dev, hipStream_t stream, bool spare, size_t bytes, void **out) {
     void *ptr = nullptr;
     const hipError_t e = hipMalloc(&ptr, bytes);
     if (e != hipSuccess) {
@@ -108,8 +95,45 @@ int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, voi
         set_error("hipMalloc of %zu bytes of K-split scratch memory failed: %s", bytes, hipGetErrorString(e));
         return TPAMD_ERR_NOMEM;
     }
-    g_cache.push_back(Entry{dev, stream, ptr, bytes});
-    *out = ptr;
+    g_cache.push_back(Entry{dev, stream, spare, ptr, bytes});
+    if (out != nullptr) *out = ptr;
+    return TPAMD_OK;
+}
+
+int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out) {
+    *out = nullptr;
+    if (static_scratch_active()) return static_scratch(dev, need, out);
+    int on_device = 0;
+    Entry *spare = nullptr;
+    for (Entry &e : g_cache) {
+        if (e.dev != dev) continue;
+        ++on_device;
+        if (e.spare) {
+            spare = &e;
+            continue;
+        }
+        if (e.stream == stream) {
+            if (e.bytes >= need) *out = e.ptr;
+            return TPAMD_OK;
+        }
+    }
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    TPAMD_HIP(hipStreamIsCapturing(stream, &capturing));
+    if (capturing != hipStreamCaptureStatusNone) {
+        if (spare != nullptr && spare->bytes >= need) {  // from now on this is the capturing stream's buffer
+            spare->spare = false;
+            spare->stream = stream;
+            *out = spare->ptr;
+        }
+        return TPAMD_OK;
+    }
+    if (on_device >= MAX_BUFFERS_PER_DEVICE) return TPAMD_OK;
+    const size_t bytes = need > reserve ? need : reserve;
+    const int rc = allocate_entry(dev, stream, false, bytes, out);
+    if (rc != TPAMD_OK) return rc;
+    if (spare == nullptr && on_device + 1 < MAX_BUFFERS_PER_DEVICE) {
+        if (allocate_entry(dev, nullptr, true, reserve, nullptr) != TPAMD_OK) set_error("%s", "");  // no spare: captures run unsplit
+    }
     return TPAMD_OK;
 }
 
@@ -127,7 +151,7 @@ extern "C" int tpamd_scratch_query(void *stream, void **ptr_out, uint64_t *bytes
     *bytes_out = 0;
     std::lock_guard<std::mutex> hold(splitk_mutex());
     for (const Entry &e : g_cache)
-        if (e.dev == dev && e.stream == static_cast<hipStream_t>(stream)) {
+        if (e.dev == dev && !e.spare && e.stream == static_cast<hipStream_t>(stream)) {
             *ptr_out = e.ptr;
             *bytes_out = e.bytes;
         }

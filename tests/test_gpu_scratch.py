@@ -45,22 +45,28 @@ def test_each_stream_gets_its_own_buffer(tune):
     assert _native.scratch_of_stream(DEV, a.cuda_stream) == (pa, na)
 
 
-def test_first_use_under_capture_runs_unsplit_and_allocates_nothing(tune):
+def test_a_capturing_stream_takes_the_spare_buffer(tune):
+    """Nothing is allocated under capture; a stream that captures K-split work without having run any gets the spare
+    buffer that the device's first allocation set aside, and the graph replays to the eager (split) result."""
     tune("TPAMD_GEMM_TILE", "128")
     tune("TPAMD_GEMM_SPLITK", "4")
     M, N, K = 256, 512, 4096
     x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
-    eager = _native.linear(x, w)
+    eager = _native.linear(x, w)  # allocates the default stream's buffer and, the first time on this device, the spare
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
+    assert _native.scratch_of_stream(DEV, side.cuda_stream) == (None, 0)
     graph = torch.cuda.CUDAGraph()
-    out = None
     with torch.cuda.graph(graph, stream=side):
         out = _native.linear(x, w)
-    assert _native.scratch_of_stream(DEV, side.cuda_stream) == (None, 0)
+    taken = _native.scratch_of_stream(DEV, side.cuda_stream)
     for _ in range(3):
         out.zero_()
         torch.cuda.synchronize()
         graph.replay()
+        assert torch.equal(_native.linear(x, w), eager)  # eager K-split work on another stream between the replays
         torch.cuda.synchronize()
-        torch.testing.assert_close(out.float(), eager.float(), rtol=2e-2, atol=2e-2)
+        if taken[0] is not None:
+            assert torch.equal(out, eager) and taken[0] != _native.scratch_of_stream(DEV)[0]
+        else:  # an earlier capture in this process took the spare: the call ran unsplit
+            torch.testing.assert_close(out.float(), eager.float(), rtol=2e-2, atol=2e-2)
