@@ -121,6 +121,25 @@ int tpamd_copy_plan_destroy(tpamd_copy_plan *plan);
  * one rule, one "gather d" of W column-parallel outputs. */
 int tpamd_copy_jobs_run(const tpamd_copy_job *jobs, size_t n_jobs, void *stream);
 
+/* Transposing mover: for every job, dst[c][r] = src[r][c] over a 2-D region of `rows` x `cols` elements of
+ * `elem_bytes` (1, 2 or 4) bytes, staged through LDS in tiles whose rows are whole 128-byte lines on both sides.
+ * Weights that the model code keeps as [in, out] and multiplies as x @ w (transformers' Conv1D: GPT-2 c_attn / c_proj /
+ * c_fc, sliced by src/tensor_parallel/slicing_configs.py:192-201 and multiplied inside the wrapped module called at
+ * src/tensor_parallel/wrapper.py:69-72) are brought into the [out, in] layout of tpamd_linear with it. A job names a
+ * region through its base pointer and pitch, so slicing a column or row range out of the unsplit weight and
+ * transposing it is one job (a grouped split: one job per group). Up to 16 jobs per call travel in the kernel
+ * arguments; nothing is allocated. Pointers and pitches must be multiples of the element size; 16-byte multiples on
+ * both sides take the vector path. Source and destination must not overlap. */
+typedef struct tpamd_transpose_job {
+    const void *src_dev;
+    void *dst_dev;
+    uint64_t rows;      /* extent of the source region in elements; the destination region is cols x rows */
+    uint64_t cols;
+    uint64_t src_pitch; /* bytes between consecutive source rows */
+    uint64_t dst_pitch; /* bytes between consecutive destination rows */
+} tpamd_transpose_job;
+int tpamd_transpose_jobs_run(const tpamd_transpose_job *jobs, size_t n_jobs, int elem_bytes, void *stream);
+
 /* Scale state action: out[i] = in[i] / world_size in the tensor's dtype
  * (Scale.__call__, src/tensor_parallel/state_actions.py:59-60). For bf16/f16 the quotient of the
  * fp32-widened value is rounded to nearest even, as torch does. `mul != 0` multiplies instead

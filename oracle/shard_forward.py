@@ -30,6 +30,15 @@ def row_parallel_linear(x_full, w_full, world_size: int, rank: int) -> torch.Ten
     return F.linear(x, w)
 
 
+def conv1d_shard(x: torch.Tensor, w_in_out: torch.Tensor, bias) -> torch.Tensor:
+    """transformers' Conv1D on one rank's sliced weight, the module the reference's GPT-2 shards run
+    (slicing_configs.py:192-201; called through wrapper.py:69-72): addmm(bias, x2d, w) with w of shape [in, out]."""
+    out = x.reshape(-1, x.shape[-1]) @ w_in_out
+    if bias is not None:
+        out = out + bias
+    return out.reshape(*x.shape[:-1], w_in_out.shape[1])
+
+
 def gated_mlp_shard(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor) -> torch.Tensor:
     """Llama MLP on one rank's weights: down(silu(gate(x)) * up(x)), every op in the tensors' dtype."""
     return F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)

@@ -70,6 +70,14 @@ def split_in_grouped_chunks_undo(parts: Sequence[np.ndarray], dim: int, num_grou
     return cat.reshape(out_shape)
 
 
+def in_axis_fastest(shard: np.ndarray) -> np.ndarray:
+    """Memory image of a 2-D shard stored with its first axis fastest: the row-major array of its transpose. A weight
+    that the model code keeps as [in, out] (transformers' Conv1D, sliced by slicing_configs.py:192-201) read this way
+    is the [out, in] matrix of the equivalent torch.nn.Linear. Pinned by numpy's own transpose."""
+    assert shard.ndim == 2, shard.shape
+    return np.ascontiguousarray(shard.T)
+
+
 def scale(a: np.ndarray, world_size: int) -> np.ndarray:
     """Scale.__call__ for float32 input (state_actions.py:59-60)."""
     return (a / np.float32(world_size)).astype(a.dtype)

@@ -23,6 +23,7 @@ EXPORTS = (
     "tpamd_copy_plan_bytes",
     "tpamd_copy_plan_destroy",
     "tpamd_copy_jobs_run",
+    "tpamd_transpose_jobs_run",
     "tpamd_scale",
     "tpamd_reduce_partials",
     "tpamd_tuning_reload",
@@ -60,6 +61,17 @@ class CopyJob(ctypes.Structure):
     ]
 
 
+class TransposeJob(ctypes.Structure):
+    _fields_ = [
+        ("src", ctypes.c_void_p),
+        ("dst", ctypes.c_void_p),
+        ("rows", ctypes.c_uint64),
+        ("cols", ctypes.c_uint64),
+        ("src_pitch", ctypes.c_uint64),
+        ("dst_pitch", ctypes.c_uint64),
+    ]
+
+
 _lib: Optional[ctypes.CDLL] = None
 _load_error: Optional[str] = None
 
@@ -81,6 +93,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_copy_plan_destroy.argtypes = [vp]
     lib.tpamd_copy_jobs_run.restype = ci
     lib.tpamd_copy_jobs_run.argtypes = [c.POINTER(CopyJob), c.c_size_t, vp]
+    lib.tpamd_transpose_jobs_run.restype = ci
+    lib.tpamd_transpose_jobs_run.argtypes = [c.POINTER(TransposeJob), c.c_size_t, ci, vp]
     lib.tpamd_scale.restype = ci
     lib.tpamd_scale.argtypes = [vp, vp, u64, ci, ci, ci, vp]
     lib.tpamd_reduce_partials.restype = ci
@@ -250,6 +264,46 @@ def run_copy_jobs(jobs: Sequence[tuple], device: torch.device) -> None:
     plan.run()
     torch.cuda.current_stream(device).synchronize()  # the plan's tile table must outlive the launch
     plan.close()
+
+
+TRANSPOSE_MAX_JOBS = 16
+
+
+def run_transpose_jobs(jobs: Sequence[tuple], elem_bytes: int, device: torch.device) -> None:
+    """Launch transposing region moves: jobs are (src_ptr, dst_ptr, rows, cols, src_pitch, dst_pitch) with the extent
+    in elements of the source region and the pitches in bytes; 16 jobs per launch."""
+    with _on_device(device):
+        for at in range(0, len(jobs), TRANSPOSE_MAX_JOBS):
+            part = jobs[at:at + TRANSPOSE_MAX_JOBS]
+            arr = (TransposeJob * len(part))(*[TransposeJob(*j) for j in part])
+            _check(lib().tpamd_transpose_jobs_run(arr, len(part), elem_bytes, ctypes.c_void_p(current_stream_ptr(device))),
+                   "tpamd_transpose_jobs_run")
+
+
+def transpose_regions(src: torch.Tensor, col_ranges: Sequence[tuple], row_range: Optional[tuple] = None,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`cat([src[r0:r1, a:b] for a, b in col_ranges], dim=1).t()` as a fresh contiguous tensor, in one launch: column
+    ranges (and one row range) are cut out of the row-major 2-D tensor `src` and land transposed, one below the other.
+    With the whole tensor as its only range this is `src.t().contiguous()`."""
+    require_device(src, "transpose_regions")
+    if src.dim() != 2 or src.stride(1) != 1 or src.element_size() not in (1, 2, 4):
+        raise ValueError(f"transpose_regions: a row-major 2-D tensor of 1-, 2- or 4-byte elements is needed, got shape {tuple(src.shape)} "
+                         f"strides {src.stride()} {src.dtype}")
+    r0, r1 = (0, src.shape[0]) if row_range is None else row_range
+    if not (0 <= r0 <= r1 <= src.shape[0]) or any(not (0 <= a <= b <= src.shape[1]) for a, b in col_ranges):
+        raise ValueError(f"transpose_regions: ranges {row_range} x {list(col_ranges)} outside shape {tuple(src.shape)}")
+    es, n_out = src.element_size(), sum(b - a for a, b in col_ranges)
+    if out is None:
+        out = torch.empty((n_out, r1 - r0), dtype=src.dtype, device=src.device)
+    elif out.shape != (n_out, r1 - r0) or out.dtype != src.dtype or out.device != src.device or not out.is_contiguous():
+        raise ValueError("transpose_regions: out must be a contiguous tensor of the result's shape, dtype and device")
+    pitch, jobs, at = src.stride(0) * es, [], 0
+    for a, b in col_ranges:
+        if b > a and r1 > r0:
+            jobs.append((src.data_ptr() + r0 * pitch + a * es, out.data_ptr() + at * out.stride(0) * es, r1 - r0, b - a, pitch, out.stride(0) * es))
+        at += b - a
+    run_transpose_jobs(jobs, es, src.device)
+    return out
 
 
 def scale(inp: torch.Tensor, world_size: int, multiply: bool = False) -> torch.Tensor:

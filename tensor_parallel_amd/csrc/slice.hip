@@ -156,6 +156,89 @@ __global__ __launch_bounds__(COPY_THREADS) void copy_small_kernel(SmallBatch b) 
     }
 }
 
+// ---- transposing mover: dst[c][r] = src[r][c] over 2-D element regions, staged through LDS ---------------------------
+// A tile is TS x TS elements with TS * sizeof(E) = 128 bytes, so both the source rows read and the destination rows
+// written are whole 128-byte lines. The block stages the tile in LDS row by row (16-byte loads, 8 lanes per source
+// row), then every lane gathers the 16 bytes of one destination row segment from a column of the staged tile and
+// stores them (8 lanes per destination row). Rows of the LDS tile are padded by 4 bytes: a lane's column reads walk
+// down 128 / TS-apart rows and would otherwise all meet in one bank. Regions whose base addresses or pitches are not
+// multiples of 16 bytes, and tiles cut by the region's edge, move element by element through the same staging.
+constexpr int TR_MAX_JOBS = 16;
+struct TransposeJob {
+    const char *src;
+    char *dst;
+    uint64_t rows, cols;  // extent of the source region in elements
+    uint64_t src_pitch, dst_pitch;
+    uint32_t tiles_c;     // tiles along the source columns
+    uint32_t tile_begin;  // first global tile index of this job
+    uint32_t vec_ok;      // both sides allow 16-byte accesses
+};
+struct TransposeBatch {
+    TransposeJob job[TR_MAX_JOBS];
+    uint32_t n_jobs, n_tiles;
+};
+
+template <typename E>
+__global__ __launch_bounds__(COPY_THREADS) void transpose_tiles_kernel(TransposeBatch b) {
+    constexpr int ES = sizeof(E);
+    constexpr int TS = 128 / ES;       // tile edge in elements
+    constexpr int PER = 16 / ES;       // elements per 16-byte chunk
+    constexpr int PITCH = TS + 4 / ES; // LDS row pitch in elements (128 bytes + 4)
+    constexpr int PASSES = TS / 32;    // 256 lanes cover 32 rows of 8 chunks per pass
+    __shared__ __attribute__((aligned(4))) E tile[TS * PITCH];
+    const int tid = threadIdx.x;
+    const int chunk = tid & 7, lrow = tid >> 3;
+    for (uint32_t ti = blockIdx.x; ti < b.n_tiles; ti += gridDim.x) {
+        uint32_t ji = 0;
+        while (ji + 1 < b.n_jobs && b.job[ji + 1].tile_begin <= ti) ++ji;  // block-uniform
+        const TransposeJob &j = b.job[ji];
+        const uint32_t local = ti - j.tile_begin;
+        const uint64_t r0 = static_cast<uint64_t>(local / j.tiles_c) * TS, c0 = static_cast<uint64_t>(local % j.tiles_c) * TS;
+        const uint32_t nr = static_cast<uint32_t>(j.rows - r0 < TS ? j.rows - r0 : TS);
+        const uint32_t nc = static_cast<uint32_t>(j.cols - c0 < TS ? j.cols - c0 : TS);
+        const bool whole = j.vec_ok && nr == TS && nc == TS;
+        // stage: lane (lrow, chunk) of a pass brings elements [chunk * PER, +PER) of source row lrow + 32 * pass
+        if (whole) {
+            v4u regs[PASSES];
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p)
+                regs[p] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(j.src + (r0 + lrow + 32 * p) * j.src_pitch + c0 * ES) + chunk);
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                uint32_t *row = reinterpret_cast<uint32_t *>(tile + (lrow + 32 * p) * PITCH) + chunk * 4;
+                row[0] = regs[p].x, row[1] = regs[p].y, row[2] = regs[p].z, row[3] = regs[p].w;
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const uint32_t r = lrow + 32 * p;
+                if (r >= nr) continue;
+                const E *s = reinterpret_cast<const E *>(j.src + (r0 + r) * j.src_pitch) + c0;
+                for (uint32_t c = chunk * PER; c < static_cast<uint32_t>(chunk + 1) * PER && c < nc; ++c) tile[r * PITCH + c] = s[c];
+            }
+        }
+        __syncthreads();
+        // write: lane (lrow, chunk) of a pass stores elements [chunk * PER, +PER) of destination row lrow + 32 * pass,
+        // which are source rows chunk * PER ... of source column lrow + 32 * pass
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const uint32_t c = lrow + 32 * p;  // source column = destination row
+            if (whole) {
+                E v[PER];
+#pragma unroll
+                for (int i = 0; i < PER; ++i) v[i] = tile[(chunk * PER + i) * PITCH + c];
+                v4u out;
+                __builtin_memcpy(&out, v, 16);
+                __builtin_nontemporal_store(out, reinterpret_cast<v4u *>(j.dst + (c0 + c) * j.dst_pitch + r0 * ES) + chunk);
+            } else if (c < nc) {
+                E *d = reinterpret_cast<E *>(j.dst + (c0 + c) * j.dst_pitch) + r0;
+                for (uint32_t r = chunk * PER; r < static_cast<uint32_t>(chunk + 1) * PER && r < nr; ++r) d[r] = tile[r * PITCH + c];
+            }
+        }
+        __syncthreads();  // the tile is reused by the next iteration
+    }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void scale_kernel(const void *__restrict__ in, void *__restrict__ out, uint64_t n,
                                                     float w, int mul) {
@@ -362,6 +445,54 @@ extern "C" int tpamd_copy_jobs_run(const tpamd_copy_job *jobs, size_t n_jobs, vo
     const uint64_t cap = static_cast<uint64_t>(cus) * 8;
     hipLaunchKernelGGL(copy_small_kernel, dim3(static_cast<unsigned>(tiles < cap ? tiles : cap)), dim3(COPY_THREADS), 0,
                        static_cast<hipStream_t>(stream), b);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+extern "C" int tpamd_transpose_jobs_run(const tpamd_transpose_job *jobs, size_t n_jobs, int elem_bytes, void *stream) {
+    TPAMD_REQUIRE(n_jobs <= static_cast<size_t>(TR_MAX_JOBS), "tpamd_transpose_jobs_run: at most %d jobs (got %zu)", TR_MAX_JOBS, n_jobs);
+    TPAMD_REQUIRE(jobs != nullptr || n_jobs == 0, "tpamd_transpose_jobs_run: jobs is NULL");
+    TPAMD_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4, "tpamd_transpose_jobs_run: elem_bytes %d (1, 2 or 4)", elem_bytes);
+    const uint64_t es = static_cast<uint64_t>(elem_bytes), ts = 128 / es;
+    TransposeBatch b{};
+    uint64_t tiles = 0;
+    for (size_t ji = 0; ji < n_jobs; ++ji) {
+        const tpamd_transpose_job &j = jobs[ji];
+        if (j.rows == 0 || j.cols == 0) continue;
+        TPAMD_REQUIRE(j.src_dev != nullptr && j.dst_dev != nullptr, "transpose job %zu: null pointer", ji);
+        TPAMD_REQUIRE(j.src_pitch >= j.cols * es && j.dst_pitch >= j.rows * es,
+                      "transpose job %zu: pitch (%llu src, %llu dst) smaller than a row (%llu, %llu bytes)", ji,
+                      (unsigned long long)j.src_pitch, (unsigned long long)j.dst_pitch, (unsigned long long)(j.cols * es),
+                      (unsigned long long)(j.rows * es));
+        TPAMD_REQUIRE(j.src_pitch % es == 0 && j.dst_pitch % es == 0 && aligned(j.src_dev, es) && aligned(j.dst_dev, es),
+                      "transpose job %zu: pointers and pitches must be multiples of the element size %d", ji, elem_bytes);
+        TransposeJob &d = b.job[b.n_jobs++];
+        d.src = static_cast<const char *>(j.src_dev);
+        d.dst = static_cast<char *>(j.dst_dev);
+        d.rows = j.rows;
+        d.cols = j.cols;
+        d.src_pitch = j.src_pitch;
+        d.dst_pitch = j.dst_pitch;
+        d.vec_ok = aligned(j.src_dev, 16) && aligned(j.dst_dev, 16) && j.src_pitch % 16 == 0 && j.dst_pitch % 16 == 0;
+        const uint64_t tr = (j.rows + ts - 1) / ts, tc = (j.cols + ts - 1) / ts;
+        TPAMD_REQUIRE(tc < 0x7fffffffull && tr < 0x7fffffffull && tiles + tr * tc < 0xffffff00ull, "tpamd_transpose_jobs_run: too many tiles");
+        d.tiles_c = static_cast<uint32_t>(tc);
+        d.tile_begin = static_cast<uint32_t>(tiles);
+        tiles += tr * tc;
+    }
+    if (tiles == 0) return TPAMD_OK;
+    b.n_tiles = static_cast<uint32_t>(tiles);
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+    const uint64_t cap = static_cast<uint64_t>(cus) * 8;
+    const dim3 grid(static_cast<unsigned>(tiles < cap ? tiles : cap)), block(COPY_THREADS);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (elem_bytes) {
+        case 1: hipLaunchKernelGGL(transpose_tiles_kernel<uint8_t>, grid, block, 0, s, b); break;
+        case 2: hipLaunchKernelGGL(transpose_tiles_kernel<uint16_t>, grid, block, 0, s, b); break;
+        default: hipLaunchKernelGGL(transpose_tiles_kernel<uint32_t>, grid, block, 0, s, b); break;
+    }
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }

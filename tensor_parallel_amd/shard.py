@@ -12,7 +12,7 @@ from torch import nn
 
 from . import _native
 from .config import Config, MappedActions, ModuleRules, get_parameter_name_mapping
-from .shard_modules import install_shard_kernels
+from .shard_modules import install_shard_kernels, is_conv1d
 from .slicing import BatchSlicer
 from .state_actions import SegmentedAction
 from .wrapper import TensorParallelWrapper
@@ -126,12 +126,14 @@ def process_state_(
     own_batch = batch is None
     if own_batch:
         batch = BatchSlicer()
+    # [in, out] weights that the shard's kernels want with the `in` axis fastest: sliced and transposed in one pass
+    in_out_weights = {f"{prefix}.weight" if prefix else "weight" for prefix, sub in sharded_module.named_modules() if is_conv1d(sub)}
     for name, state in chain(sharded_module.named_parameters(), sharded_module.named_buffers()):
         src = source_tensors[name]
         for pattern, action in config.state_rules.items():
             if pattern.search(name) is not None:
                 if isinstance(action, SegmentedAction) and src is not None:
-                    new = batch.add(src, action.spec(tuple(src.shape), rank))
+                    new = batch.add(src, action.spec(tuple(src.shape), rank), k_major=name in in_out_weights)
                 else:
                     new = action(src, rank=rank)
                     new = new.clone() if new.device == state.device else new

@@ -3,7 +3,11 @@
 In the reference a shard is a deep copy of the user's module whose `torch.nn.Linear`s hold sliced weights and
 run ATen GEMMs (src/tensor_parallel/shard.py:160,184-187; wrapper.py:69-72). Here every `nn.Linear` of a shard
 is re-classed to `ShardLinear` (same parameters, same attributes, still an `nn.Linear`), and SiLU-gated MLP
-blocks with `gate_proj` / `up_proj` / `down_proj` children get a fused gate/up forward.
+blocks with `gate_proj` / `up_proj` / `down_proj` children get a fused gate/up forward. transformers' `Conv1D`
+(GPT-2's c_attn / c_proj / c_fc: weight kept as [in, out] and multiplied as x @ w, sliced by
+src/tensor_parallel/slicing_configs.py:192-201) is re-classed to a subclass whose forward is the same `tpamd_linear`:
+its weight keeps the [in, out] shape every rule and state dict expects but is stored with the `in` axis fastest, which
+is the kernel's [out, in] layout; the transposing mover writes it that way while slicing, or once at the first forward.
 
 Inference only: the kernels have no backward; asking for one raises.
 """
@@ -15,6 +19,7 @@ import torch
 from torch import nn
 
 from . import _native
+from .slicing import is_k_major
 
 
 class _NoBackward(torch.autograd.Function):
@@ -41,6 +46,34 @@ class ShardLinear(nn.Linear):
     def forward(self, input: torch.Tensor) -> torch.Tensor:  # noqa: A002
         out = _native.linear(input.detach(), self.weight.detach(), None if self.bias is None else self.bias.detach())
         return _guard(out, input, self.weight, self.bias)
+
+
+def is_conv1d(module: nn.Module) -> bool:
+    """transformers.pytorch_utils.Conv1D (or a subclass): a Linear whose weight is [in, out]."""
+    return any(c.__name__ == "Conv1D" and c.__module__.split(".")[0] == "transformers" for c in type(module).__mro__) and \
+        isinstance(getattr(module, "weight", None), torch.Tensor)
+
+
+def _conv1d_forward(self, x: torch.Tensor) -> torch.Tensor:
+    w = self.weight
+    if not is_k_major(w):  # a weight assigned after the shard was built: lay it out for the kernel, once
+        with torch.no_grad():
+            w.data = _native.transpose_regions(w.data.contiguous(), [(0, w.shape[1])]).t()
+    bias = getattr(self, "bias", None)
+    out = _native.linear(x.detach(), w.detach().t(), None if bias is None else bias.detach())
+    return _guard(out, x, w, bias)
+
+
+_conv1d_classes: dict = {}
+
+
+def _shard_conv1d_class(base: type) -> type:
+    """Subclass of the module's own Conv1D class with the kernel forward (isinstance checks keep working)."""
+    cls = _conv1d_classes.get(base)
+    if cls is None:
+        cls = _conv1d_classes[base] = type("ShardConv1D", (base,), {"forward": _conv1d_forward, "__doc__": "Conv1D whose forward is `tpamd_linear` "
+                                                                   "on the shard's weight, stored with its input axis fastest."})
+    return cls
 
 
 def _is_silu(fn) -> bool:
@@ -74,6 +107,8 @@ def install_shard_kernels(shard: nn.Module) -> None:
     for module in shard.modules():
         if type(module) is nn.Linear:
             module.__class__ = ShardLinear
+        elif is_conv1d(module) and type(module).__name__ == "Conv1D" and module.weight.dim() == 2 and module.weight.dtype in (torch.bfloat16, torch.float16, torch.float32):
+            module.__class__ = _shard_conv1d_class(type(module))
     for module in shard.modules():
         if is_gated_silu_mlp(module):
             module.forward = types.MethodType(_gated_mlp_forward, module)

@@ -88,9 +88,34 @@ def copy_jobs(spec: SliceSpec, itemsize: int, full_ptr: int, shard_ptr: int, sca
     return jobs
 
 
+def transpose_jobs(spec: SliceSpec, itemsize: int, full_ptr: int, out_ptr: int) -> List[tuple]:
+    """Transposing-mover jobs that cut `spec`'s segments out of a row-major 2-D tensor at `full_ptr` and write the
+    shard with its axes swapped: the shard of logical shape (R, C) is stored at `out_ptr` as C rows of R elements."""
+    if len(spec.shape) != 2:
+        raise ValueError(f"transposed slicing needs a 2-D tensor, got shape {spec.shape}")
+    rows, cols = spec.shape
+    out_rows = spec.out_shape[0]
+    jobs, done = [], 0
+    for start, length in spec.segments:
+        if length and rows and cols:
+            if spec.dim == 1:  # columns [start, start + length) become stored rows done ... done + length
+                jobs.append((full_ptr + start * itemsize, out_ptr + done * out_rows * itemsize, rows, length, cols * itemsize, out_rows * itemsize))
+            else:  # rows [start, start + length) become stored columns done ... done + length
+                jobs.append((full_ptr + start * cols * itemsize, out_ptr + done * itemsize, length, cols, cols * itemsize, out_rows * itemsize))
+        done += length
+    return jobs
+
+
+def is_k_major(t: torch.Tensor) -> bool:
+    """True for a 2-D tensor stored with its first axis fastest: `t.t()` is row-major contiguous."""
+    return t.dim() == 2 and t.stride(0) == 1 and t.stride(1) == t.shape[0]
+
+
 def _device_source(t: torch.Tensor, device: Optional[torch.device]) -> torch.Tensor:
     """The tensor, contiguous, on the HIP device the kernels will run on (uploaded if it lives on the host)."""
     if t.device.type == "cuda":
+        if is_k_major(t) and not t.is_contiguous() and t.element_size() in (1, 2, 4):
+            return _native.transpose_regions(t.t(), [(0, t.shape[0])])
         return t.contiguous()
     if t.device.type != "cpu":
         raise _native.NativeLibraryError(f"cannot slice a tensor on {t.device}")
@@ -160,13 +185,18 @@ class BatchSlicer:
         self._sources: Dict[int, torch.Tensor] = {}  # id(original) -> device-resident contiguous source
         self._keep: List[torch.Tensor] = []
         self._jobs: List[tuple] = []
+        self._transposing: Dict[int, List[tuple]] = {}  # element size -> jobs of the transposing mover
         self.plan: Optional[_native.CopyPlan] = None
 
-    def add(self, t: torch.Tensor, spec: SliceSpec) -> torch.Tensor:
+    def add(self, t: torch.Tensor, spec: SliceSpec, k_major: bool = False) -> torch.Tensor:
+        """Queue one shard of `t`. With `k_major` (2-D tensors) the shard is written with its first axis fastest: it has
+        the shape `spec.out_shape` and the memory of its transpose, which is how `tpamd_linear` wants a weight that the
+        model code keeps as [in, out]; slicing and transposing are one pass of the transposing mover."""
         if tuple(t.shape) != spec.shape:
             raise ValueError(f"spec was made for shape {spec.shape}, tensor has {tuple(t.shape)}")
         if t.device.type == "meta":
             return torch.empty(spec.out_shape, dtype=t.dtype, device="meta")
+        k_major = k_major and t.dim() == 2 and t.element_size() in (1, 2, 4)
         src = self._sources.get(id(t))
         if src is None:
             src = _device_source(t, self.device)
@@ -176,6 +206,10 @@ class BatchSlicer:
                 self.device = src.device
         if src.device != self.device:
             raise ValueError(f"batch is on {self.device}, tensor on {src.device}")
+        if k_major:
+            stored = torch.empty(spec.out_shape[::-1], dtype=t.dtype, device=src.device)
+            self._transposing.setdefault(t.element_size(), []).extend(transpose_jobs(spec, t.element_size(), src.data_ptr(), stored.data_ptr()))
+            return stored.t()
         out = torch.empty(spec.out_shape, dtype=t.dtype, device=src.device)
         self._jobs += copy_jobs(spec, t.element_size(), src.data_ptr(), out.data_ptr())
         return out
@@ -187,11 +221,15 @@ class BatchSlicer:
 
     def run(self) -> int:
         """Launch the batch; returns the bytes moved one way."""
+        moved = 0
+        for itemsize, jobs in self._transposing.items():
+            _native.run_transpose_jobs(jobs, itemsize, self.device)
+            moved += sum(j[2] * j[3] for j in jobs) * itemsize
         plan = self.build()
         if plan is None:
-            return 0
+            return moved
         plan.run()
-        return plan.nbytes
+        return moved + plan.nbytes
 
     def close(self) -> None:
         if self.plan is not None:
@@ -200,3 +238,4 @@ class BatchSlicer:
         self._sources.clear()
         self._keep.clear()
         self._jobs = []
+        self._transposing = {}
