@@ -29,6 +29,7 @@ Tuning read_tuning() {
     t.skinny_pair = env_int("TPAMD_SKINNY_PAIR");
     t.skinny_resident = env_int("TPAMD_SKINNY_RESIDENT");
     t.w8_split = env_int("TPAMD_W8_SPLIT");
+    t.gemv_rows = env_int("TPAMD_GEMV_ROWS");
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
     t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");
     t.copy_blocks_per_cu = env_int("TPAMD_COPY_BLOCKS_PER_CU");

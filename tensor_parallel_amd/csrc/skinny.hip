@@ -872,6 +872,134 @@ int launch_gemv(const SkinnyParams &p, hipStream_t s) {
     return TPAMD_OK;
 }
 
+// ---- M <= 3, K <= 8192: every piece of a column's weights in flight at once, all counts known at compile time --------
+// Same mapping as gemv_kernel (a wavefront owns an output column, x in LDS) for the shapes decode meets: a row takes
+// at most NP 1-KiB loads per matrix, issued back to back before x is staged, and multiplied as they arrive in a fully
+// unrolled sequence; the 64 lane sums meet through DPP row operations and four lane reads instead of six LDS-crossbar
+// shuffles. WAVES wavefronts per block share one copy of x.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
+    return v + __builtin_bit_cast(float, t);
+}
+// Sum over the 64 lanes, in every lane: pairs, quads, eights and sixteens inside each row of 16 lanes (quad_perm
+// [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror), then the four row sums as (r0 + r1) + (r2 + r3).
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v = dpp_add<0xb1>(v);
+    v = dpp_add<0x4e>(v);
+    v = dpp_add<0x141>(v);
+    v = dpp_add<0x140>(v);
+    const int r = __builtin_bit_cast(int, v);
+    const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 0)), b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 16));
+    const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 32)), d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 48));
+    return (a + b) + (c + d);
+}
+
+template <int DT, int MODE, int MR, int WAVES, int NP, bool WHOLE>
+__global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(SkinnyParams p) {
+    constexpr int THREADS = WAVES * 64;
+    constexpr int NMAT = MODE == SK_SWIGLU ? 2 : 1;
+    extern __shared__ __align__(16) char xs[];  // x[MR][K]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = blockIdx.x * WAVES + wave;
+    const int row = n < p.N ? n : p.N - 1;
+    const int row_bytes = WHOLE ? NP * 1024 : p.K * 2;  // WHOLE: K is exactly NP pieces, nothing to mask
+    const char *w0 = p.w + static_cast<int64_t>(row) * p.ldw * 2 + lane * 16;
+    const char *w1 = NMAT == 2 ? p.w2 + static_cast<int64_t>(row) * p.ldw * 2 + lane * 16 : nullptr;
+    // x is requested first and the weights right behind it: loads return in order, so x can be staged (and the block
+    // can meet) while the weights are still on their way, and every piece is multiplied as it arrives
+    constexpr int XL = (NP * 64 + THREADS - 1) / THREADS;  // 16-byte pieces of one row of x per thread
+    uint4 xr[MR][XL];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int at = (tid + i * THREADS) * 16;
+            xr[m][i] = *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + (at < row_bytes ? at : 0));
+        }
+    uint4 wv[NMAT][NP];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+        // pieces past K are fetched from the row's start (always valid) and zeroed
+        const bool ok = WHOLE || j * 1024 + lane * 16 < row_bytes;
+        const uint4 a = nt_load_u4(ok ? w0 + j * 1024 : w0 - lane * 16);
+        wv[0][j] = ok ? a : make_uint4(0, 0, 0, 0);
+        if constexpr (NMAT == 2) {
+            const uint4 b = nt_load_u4(ok ? w1 + j * 1024 : w1 - lane * 16);
+            wv[NMAT - 1][j] = ok ? b : make_uint4(0, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int at = (tid + i * THREADS) * 16;
+            if (at < row_bytes) *reinterpret_cast<uint4 *>(xs + m * row_bytes + at) = xr[m][i];
+        }
+    __syncthreads();
+    float acc[NMAT][MR];
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[a][m] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+        const int at = WHOLE || j * 1024 + lane * 16 < row_bytes ? j * 1024 + lane * 16 : 0;
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const uint4 xv = *reinterpret_cast<const uint4 *>(xs + m * row_bytes + at);
+#pragma unroll
+            for (int a = 0; a < NMAT; ++a) acc[a][m] = dot8<DT>(wv[a][j], xv, acc[a][m]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        const float s0 = wave_sum_dpp(acc[0][m]);
+        float s1 = 0.f;
+        if constexpr (NMAT == 2) s1 = wave_sum_dpp(acc[NMAT - 1][m]);
+        if (lane == 0 && n < p.N) skinny_store_output<DT, MODE>(p, s0, s1, m, n);
+    }
+}
+
+template <int DT, int MODE, int WAVES, int NP>
+void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
+    const dim3 grid(static_cast<unsigned>((p.N + WAVES - 1) / WAVES)), block(WAVES * 64);
+    const size_t lds = static_cast<size_t>(p.M) * p.K * 2;
+    const bool whole = p.K == NP * 512;
+#define TPAMD_ROWS_M(MRV) \
+    if (whole) hipLaunchKernelGGL((gemv_rows_kernel<DT, MODE, MRV, WAVES, NP, true>), grid, block, lds, s, p); \
+    else hipLaunchKernelGGL((gemv_rows_kernel<DT, MODE, MRV, WAVES, NP, false>), grid, block, lds, s, p)
+    switch (p.M) {
+        case 1: TPAMD_ROWS_M(1); break;
+        case 2: TPAMD_ROWS_M(2); break;
+        default: TPAMD_ROWS_M(3); break;
+    }
+#undef TPAMD_ROWS_M
+}
+
+// 16-bit weights, M <= 3, K <= 8192. *done = false: not taken.
+template <int DT, int MODE>
+int launch_gemv_rows(const SkinnyParams &p, hipStream_t s, bool *done) {
+    *done = false;
+    const int knob = tuning().gemv_rows;  // wavefronts per block; 0 = the general kernel
+    if (knob == 0 || p.K > 8192 || p.K % 8 != 0) return TPAMD_OK;
+    // measured on the Llama-7B shard at M = 1 (inside a HIP graph): single matrix 4096 x 5504 with 16 / 8 / 4 wavefronts
+    // per block 8.7 / 9.1 / 9.5 us, gated pair 2 x 5504 x 4096 16.8 / 15.1 / 15.6 us
+    const int waves = knob != TUNE_UNSET ? knob : (MODE == SK_LINEAR && p.N >= 4096) ? 16 : 8;
+    const int np = (p.K + 511) / 512;
+#define TPAMD_ROWS_CASE(W) \
+    if (np <= 4) launch_gemv_rows_m<DT, MODE, W, 4>(p, s); else if (np <= 8) launch_gemv_rows_m<DT, MODE, W, 8>(p, s); \
+    else if (np <= 11) launch_gemv_rows_m<DT, MODE, W, 11>(p, s); else if (np <= 12) launch_gemv_rows_m<DT, MODE, W, 12>(p, s); \
+    else launch_gemv_rows_m<DT, MODE, W, 16>(p, s)
+    if (waves == 4) { TPAMD_ROWS_CASE(4); }
+    else if (waves == 16) { TPAMD_ROWS_CASE(16); }
+    else { TPAMD_ROWS_CASE(8); }
+#undef TPAMD_ROWS_CASE
+    TPAMD_HIP(hipGetLastError());
+    *done = true;
+    return TPAMD_OK;
+}
+
 // Column groups per block: as many as keep at least one block per CU and divide N; they pay once x outweighs w.
 inline int pick_cg(const SkinnyParams &p, bool w8, bool swiglu) {
     if (const int v = tuning().skinny_cg; v != TUNE_UNSET) return v == 4 ? 4 : v == 2 ? 2 : 1;
@@ -1068,6 +1196,12 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     const bool bf = dtype == TPAMD_BF16;
     if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
         if (w8) return bf ? launch_gemv<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, true, SK_LINEAR>(p, s);
+        if (!w8) {
+            bool done = false;
+            const int rc = swiglu ? (bf ? launch_gemv_rows<TPAMD_BF16, SK_SWIGLU>(p, s, &done) : launch_gemv_rows<TPAMD_F16, SK_SWIGLU>(p, s, &done))
+                                  : (bf ? launch_gemv_rows<TPAMD_BF16, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, SK_LINEAR>(p, s, &done));
+            if (rc != TPAMD_OK || done) return rc;
+        }
         if (swiglu) return bf ? launch_gemv<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_gemv<TPAMD_F16, false, SK_SWIGLU>(p, s);
         return bf ? launch_gemv<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, false, SK_LINEAR>(p, s);
     }
