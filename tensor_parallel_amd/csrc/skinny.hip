@@ -895,33 +895,60 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return (a + b) + (c + d);
 }
 
-template <int DT, int MODE, int MR, int WAVES, int NP, bool WHOLE>
+// int8 weights (W8, plain linear): a piece is 1024 K elements; the outlier products' operands (at most 128 outlier
+// columns) and the row's scale are requested ahead of everything else, so that no wavefront ends on a memory round trip.
+template <int DT, bool W8, int MODE, int MR, int WAVES, int NP, bool WHOLE>
 __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(SkinnyParams p) {
+    static_assert(!W8 || MODE == SK_LINEAR, "int8 weights: plain linear only");
     constexpr int THREADS = WAVES * 64;
     constexpr int NMAT = MODE == SK_SWIGLU ? 2 : 1;
+    constexpr int PIECE_K = W8 ? 1024 : 512;  // K elements in one wavefront-wide 16-byte load of w
+    constexpr int OB = 2;                     // int8: outlier columns per lane
     extern __shared__ __align__(16) char xs[];  // x[MR][K]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = blockIdx.x * WAVES + wave;
     const int row = n < p.N ? n : p.N - 1;
-    const int row_bytes = WHOLE ? NP * 1024 : p.K * 2;  // WHOLE: K is exactly NP pieces, nothing to mask
-    const char *w0 = p.w + static_cast<int64_t>(row) * p.ldw * 2 + lane * 16;
+    const int K = WHOLE ? NP * PIECE_K : p.K;  // WHOLE: K is exactly NP pieces, nothing to mask
+    const int w_row_bytes = W8 ? K : K * 2, x_row_bytes = K * 2;
+    const int x_lds_row = W8 ? (x_row_bytes + 2047) & ~2047 : x_row_bytes;  // int8: rows of x are permuted within whole 2 KiB
+    const char *w0 = p.w + static_cast<int64_t>(row) * p.ldw * (W8 ? 1 : 2) + lane * 16;
     const char *w1 = NMAT == 2 ? p.w2 + static_cast<int64_t>(row) * p.ldw * 2 + lane * 16 : nullptr;
+    // int8: a lane's 16 weights of a piece meet 32 bytes of x. Stored as they come, the two 16-byte reads of the 64 lanes
+    // would be 32 bytes apart and collide in the LDS banks two by two; so within every 2 KiB of x (one piece) the first
+    // halves of all lanes' 32 bytes are stored together and the second halves behind them: both reads are contiguous.
+    auto x_slot = [](int byte_at) -> int {
+        if constexpr (!W8) return byte_at;
+        else return (byte_at & ~2047) | ((byte_at & 16) << 6) | ((byte_at >> 1) & 1008) | (byte_at & 15);
+    };
+    uint16_t o_w[OB];
+    int o_col[OB];
+    float row_scale = 1.f;
+    if constexpr (W8) {
+        row_scale = p.scale[row];
+#pragma unroll
+        for (int i = 0; i < OB; ++i) {
+            const int o = lane + i * 64;
+            const bool in = o < p.n_out;
+            o_w[i] = in ? reinterpret_cast<const uint16_t *>(p.w_out)[static_cast<int64_t>(row) * p.ld_wout + o] : static_cast<uint16_t>(0);
+            o_col[i] = in ? p.outlier_idx[o] : 0;
+        }
+    }
     // x is requested first and the weights right behind it: loads return in order, so x can be staged (and the block
     // can meet) while the weights are still on their way, and every piece is multiplied as it arrives
-    constexpr int XL = (NP * 64 + THREADS - 1) / THREADS;  // 16-byte pieces of one row of x per thread
+    constexpr int XL = (NP * PIECE_K / 8 + THREADS - 1) / THREADS;  // 16-byte pieces of one row of x per thread
     uint4 xr[MR][XL];
 #pragma unroll
     for (int m = 0; m < MR; ++m)
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
             const int at = (tid + i * THREADS) * 16;
-            xr[m][i] = *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + (at < row_bytes ? at : 0));
+            xr[m][i] = *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + (at < x_row_bytes ? at : 0));
         }
     uint4 wv[NMAT][NP];
 #pragma unroll
     for (int j = 0; j < NP; ++j) {
         // pieces past K are fetched from the row's start (always valid) and zeroed
-        const bool ok = WHOLE || j * 1024 + lane * 16 < row_bytes;
+        const bool ok = WHOLE || j * 1024 + lane * 16 < w_row_bytes;
         const uint4 a = nt_load_u4(ok ? w0 + j * 1024 : w0 - lane * 16);
         wv[0][j] = ok ? a : make_uint4(0, 0, 0, 0);
         if constexpr (NMAT == 2) {
@@ -934,41 +961,65 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(SkinnyParams p) {
 #pragma unroll
         for (int i = 0; i < XL; ++i) {
             const int at = (tid + i * THREADS) * 16;
-            if (at < row_bytes) *reinterpret_cast<uint4 *>(xs + m * row_bytes + at) = xr[m][i];
+            if (at < x_row_bytes) *reinterpret_cast<uint4 *>(xs + m * x_lds_row + x_slot(at)) = xr[m][i];
         }
     __syncthreads();
-    float acc[NMAT][MR];
+    float acc[NMAT][MR], acc2[MR];  // int8: two sums per row of x, so that consecutive products do not wait for each other
 #pragma unroll
-    for (int a = 0; a < NMAT; ++a)
+    for (int m = 0; m < MR; ++m) {
+        acc2[m] = 0.f;
 #pragma unroll
-        for (int m = 0; m < MR; ++m) acc[a][m] = 0.f;
+        for (int a = 0; a < NMAT; ++a) acc[a][m] = 0.f;
+    }
 #pragma unroll
     for (int j = 0; j < NP; ++j) {
-        const int at = WHOLE || j * 1024 + lane * 16 < row_bytes ? j * 1024 + lane * 16 : 0;
+        const int k = WHOLE || j * 1024 + lane * 16 < w_row_bytes ? j * PIECE_K + lane * (PIECE_K / 64) : 0;
+        if constexpr (W8) {
+            uint4 lo, hi;
+            cvt_i8x4<DT>(wv[0][j].x, lo.x, lo.y);
+            cvt_i8x4<DT>(wv[0][j].y, lo.z, lo.w);
+            cvt_i8x4<DT>(wv[0][j].z, hi.x, hi.y);
+            cvt_i8x4<DT>(wv[0][j].w, hi.z, hi.w);
 #pragma unroll
-        for (int m = 0; m < MR; ++m) {
-            const uint4 xv = *reinterpret_cast<const uint4 *>(xs + m * row_bytes + at);
+            for (int m = 0; m < MR; ++m) {
+                const uint4 xv = *reinterpret_cast<const uint4 *>(xs + m * x_lds_row + x_slot(k * 2));
+                const uint4 xv1 = *reinterpret_cast<const uint4 *>(xs + m * x_lds_row + x_slot(k * 2 + 16));
+                acc[0][m] = dot8<DT>(lo, xv, acc[0][m]);
+                acc2[m] = dot8<DT>(hi, xv1, acc2[m]);
+            }
+        } else {
 #pragma unroll
-            for (int a = 0; a < NMAT; ++a) acc[a][m] = dot8<DT>(wv[a][j], xv, acc[a][m]);
+            for (int m = 0; m < MR; ++m) {
+                const uint4 xv = *reinterpret_cast<const uint4 *>(xs + m * x_lds_row + k * 2);
+#pragma unroll
+                for (int a = 0; a < NMAT; ++a) acc[a][m] = dot8<DT>(wv[a][j], xv, acc[a][m]);
+            }
         }
     }
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
-        const float s0 = wave_sum_dpp(acc[0][m]);
+        float s0 = wave_sum_dpp(W8 ? acc[0][m] + acc2[m] : acc[0][m]);
         float s1 = 0.f;
         if constexpr (NMAT == 2) s1 = wave_sum_dpp(acc[NMAT - 1][m]);
+        if constexpr (W8) {
+            float ao = 0.f;
+#pragma unroll
+            for (int i = 0; i < OB; ++i)
+                ao = fmaf(half_to_f32<DT>(*reinterpret_cast<const uint16_t *>(xs + m * x_lds_row + x_slot(o_col[i] * 2))), half_to_f32<DT>(o_w[i]), ao);
+            s0 = s0 * row_scale + wave_sum_dpp(ao);
+        }
         if (lane == 0 && n < p.N) skinny_store_output<DT, MODE>(p, s0, s1, m, n);
     }
 }
 
-template <int DT, int MODE, int WAVES, int NP>
+template <int DT, bool W8, int MODE, int WAVES, int NP>
 void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>((p.N + WAVES - 1) / WAVES)), block(WAVES * 64);
-    const size_t lds = static_cast<size_t>(p.M) * p.K * 2;
-    const bool whole = p.K == NP * 512;
+    const size_t lds = W8 ? static_cast<size_t>(p.M) * ((p.K * 2 + 2047) / 2048 * 2048) : static_cast<size_t>(p.M) * p.K * 2;
+    const bool whole = p.K == NP * (W8 ? 1024 : 512);
 #define TPAMD_ROWS_M(MRV) \
-    if (whole) hipLaunchKernelGGL((gemv_rows_kernel<DT, MODE, MRV, WAVES, NP, true>), grid, block, lds, s, p); \
-    else hipLaunchKernelGGL((gemv_rows_kernel<DT, MODE, MRV, WAVES, NP, false>), grid, block, lds, s, p)
+    if (whole) hipLaunchKernelGGL((gemv_rows_kernel<DT, W8, MODE, MRV, WAVES, NP, true>), grid, block, lds, s, p); \
+    else hipLaunchKernelGGL((gemv_rows_kernel<DT, W8, MODE, MRV, WAVES, NP, false>), grid, block, lds, s, p)
     switch (p.M) {
         case 1: TPAMD_ROWS_M(1); break;
         case 2: TPAMD_ROWS_M(2); break;
@@ -977,20 +1028,26 @@ void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
 #undef TPAMD_ROWS_M
 }
 
-// 16-bit weights, M <= 3, K <= 8192. *done = false: not taken.
-template <int DT, int MODE>
+// M <= 3 and at most 16 pieces per row: K <= 8192 for 16-bit weights, K <= 16384 (and at most 128 outlier columns) for
+// int8. *done = false: not taken.
+template <int DT, bool W8, int MODE>
 int launch_gemv_rows(const SkinnyParams &p, hipStream_t s, bool *done) {
     *done = false;
     const int knob = tuning().gemv_rows;  // wavefronts per block; 0 = the general kernel
-    if (knob == 0 || p.K > 8192 || p.K % 8 != 0) return TPAMD_OK;
+    const int piece_k = W8 ? 1024 : 512;
+    if (knob == 0 || p.K > 16 * piece_k || p.K % (W8 ? 16 : 8) != 0 || (W8 && p.n_out > 128)) return TPAMD_OK;
+    // int8 with 2 or 3 rows of x: every further row costs as much again in LDS reads (32 bytes of x per 16 weights), and
+    // the general kernel's staggered blocks hide that better (Falcon-40B MLP shard, 2 rows: 66 us against 83 us here)
+    if (W8 && p.M > 1) return TPAMD_OK;
     // measured on the Llama-7B shard at M = 1 (inside a HIP graph): single matrix 4096 x 5504 with 16 / 8 / 4 wavefronts
-    // per block 8.7 / 9.1 / 9.5 us, gated pair 2 x 5504 x 4096 16.8 / 15.1 / 15.6 us
-    const int waves = knob != TUNE_UNSET ? knob : (MODE == SK_LINEAR && p.N >= 4096) ? 16 : 8;
-    const int np = (p.K + 511) / 512;
+    // per block 8.7 / 9.1 / 9.5 us, gated pair 2 x 5504 x 4096 16.8 / 15.1 / 15.6 us; int8 16384 x 8192 + 8192 x 16384:
+    // 51.6 / 48.0 / 50.4 us (the general kernel: 58.8 us)
+    const int waves = knob != TUNE_UNSET ? knob : (!W8 && MODE == SK_LINEAR && p.N >= 4096) ? 16 : 8;
+    const int np = (p.K + piece_k - 1) / piece_k;
 #define TPAMD_ROWS_CASE(W) \
-    if (np <= 4) launch_gemv_rows_m<DT, MODE, W, 4>(p, s); else if (np <= 8) launch_gemv_rows_m<DT, MODE, W, 8>(p, s); \
-    else if (np <= 11) launch_gemv_rows_m<DT, MODE, W, 11>(p, s); else if (np <= 12) launch_gemv_rows_m<DT, MODE, W, 12>(p, s); \
-    else launch_gemv_rows_m<DT, MODE, W, 16>(p, s)
+    if (np <= 4) launch_gemv_rows_m<DT, W8, MODE, W, 4>(p, s); else if (np <= 8) launch_gemv_rows_m<DT, W8, MODE, W, 8>(p, s); \
+    else if (np <= 11) launch_gemv_rows_m<DT, W8, MODE, W, 11>(p, s); else if (np <= 12) launch_gemv_rows_m<DT, W8, MODE, W, 12>(p, s); \
+    else launch_gemv_rows_m<DT, W8, MODE, W, 16>(p, s)
     if (waves == 4) { TPAMD_ROWS_CASE(4); }
     else if (waves == 16) { TPAMD_ROWS_CASE(16); }
     else { TPAMD_ROWS_CASE(8); }
@@ -1195,13 +1252,12 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     p.act = act;
     const bool bf = dtype == TPAMD_BF16;
     if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
+        bool done = false;
+        const int rc = w8 ? (bf ? launch_gemv_rows<TPAMD_BF16, true, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, true, SK_LINEAR>(p, s, &done))
+                     : swiglu ? (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_SWIGLU>(p, s, &done) : launch_gemv_rows<TPAMD_F16, false, SK_SWIGLU>(p, s, &done))
+                              : (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, false, SK_LINEAR>(p, s, &done));
+        if (rc != TPAMD_OK || done) return rc;
         if (w8) return bf ? launch_gemv<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, true, SK_LINEAR>(p, s);
-        if (!w8) {
-            bool done = false;
-            const int rc = swiglu ? (bf ? launch_gemv_rows<TPAMD_BF16, SK_SWIGLU>(p, s, &done) : launch_gemv_rows<TPAMD_F16, SK_SWIGLU>(p, s, &done))
-                                  : (bf ? launch_gemv_rows<TPAMD_BF16, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, SK_LINEAR>(p, s, &done));
-            if (rc != TPAMD_OK || done) return rc;
-        }
         if (swiglu) return bf ? launch_gemv<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_gemv<TPAMD_F16, false, SK_SWIGLU>(p, s);
         return bf ? launch_gemv<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, false, SK_LINEAR>(p, s);
     }
