@@ -1,8 +1,10 @@
 """Generic rules for a model without a hand-written table: every Linear is column-parallel, every
 embedding is split on its hidden axis, and a Linear tied to an embedding consumes a split input and sums
-(reference: src/tensor_parallel/autoconfig.py:12-39). Convolution rules of the reference are not carried."""
+(reference: src/tensor_parallel/autoconfig.py:12-39). The reference's convolution rules (autoconfig.py:40-78) are not
+carried: convolution layers get no rule, so every rank keeps them whole and computes them in full."""
 from __future__ import annotations
 
+import logging
 from typing import Sequence
 
 import torch
@@ -11,6 +13,8 @@ from torch.nn.modules import conv
 
 from .config import Config
 from .state_actions import Scale, Split
+
+logger = logging.getLogger(__file__)
 
 
 def get_default_config(module: nn.Module, device_ids: Sequence[torch.device]) -> Config:
@@ -38,8 +42,6 @@ def get_default_config(module: nn.Module, device_ids: Sequence[torch.device]) ->
                 if sub.bias is not None:
                     state_rules[f"^{name}.bias$"] = Scale(world_size=world_size)
         elif isinstance(sub, conv._ConvNd):
-            raise NotImplementedError(
-                f"{name}: convolution layers have no automatic tensor-parallel rules in tensor_parallel_amd; "
-                "pass a Config that leaves them whole"
-            )
+            logger.warning(f"{name}: convolution layers have no automatic tensor-parallel rules here; every rank keeps this "
+                           "layer whole (pass a Config with rules for it to split it)")
     return Config(state_rules, input_rules, output_rules, {})

@@ -9,7 +9,8 @@ src/tensor_parallel/slicing_configs.py:192-201) is re-classed to a subclass whos
 its weight keeps the [in, out] shape every rule and state dict expects but is stored with the `in` axis fastest, which
 is the kernel's [out, in] layout; the transposing mover writes it that way while slicing, or once at the first forward.
 
-Inference only: the kernels have no backward; asking for one raises.
+Inference only: the kernels have no backward; asking for one raises. Autocast is not applied by these modules: the
+input must already have the weight's dtype (a mismatch raises TypeError where `nn.Linear` under autocast would cast).
 """
 from __future__ import annotations
 
@@ -90,6 +91,11 @@ def _gated_mlp_forward(self, x: torch.Tensor) -> torch.Tensor:
     return down(h)
 
 
+def _has_hooks(module: nn.Module) -> bool:
+    return bool(module._forward_hooks or module._forward_pre_hooks or getattr(module, "_forward_hooks_with_kwargs", None)
+                or getattr(module, "_forward_pre_hooks_with_kwargs", None))
+
+
 def is_gated_silu_mlp(module: nn.Module) -> bool:
     # only the module's own children count: a wrapper forwards attribute lookups to the module it wraps
     parts = [module._modules.get(n) for n in ("gate_proj", "up_proj", "down_proj")]
@@ -98,8 +104,31 @@ def is_gated_silu_mlp(module: nn.Module) -> bool:
     gate, up, _ = parts
     if gate.bias is not None or up.bias is not None or gate.weight.dtype not in (torch.bfloat16, torch.float16):
         return False
+    if gate.weight.shape != up.weight.shape:
+        return False
+    # the fused forward reads the two weights directly: hooks on gate_proj / up_proj would be skipped, so leave such
+    # blocks to their own forward (their Linears still run on the kernels)
+    if _has_hooks(gate) or _has_hooks(up) or "forward" in module.__dict__:
+        return False
     act = module._modules.get("act_fn", module.__dict__.get("act_fn"))
     return _is_silu(act)
+
+
+def _gated_mlp_first_forward(self, x: torch.Tensor) -> torch.Tensor:
+    """First call of a block that looks like a SiLU-gated MLP: its own forward and the fused one both run on this input.
+    If they agree the fused forward takes over, otherwise the block keeps its own (a forward that slices its weights
+    for pretraining_tp, adds projections or orders the operations differently is not this pattern)."""
+    del self.forward  # the class's forward is visible again
+    own = type(self).forward(self, x)
+    try:
+        fused = _gated_mlp_forward(self, x)
+        same = isinstance(own, torch.Tensor) and own.shape == fused.shape and torch.allclose(
+            own.detach().float(), fused.detach().float(), rtol=2e-2, atol=2e-2 * float(own.detach().float().std()) + 1e-6)
+    except (TypeError, ValueError, RuntimeError):
+        same = False
+    if same:
+        self.forward = types.MethodType(_gated_mlp_forward, self)
+    return own
 
 
 def install_shard_kernels(shard: nn.Module) -> None:
@@ -111,4 +140,4 @@ def install_shard_kernels(shard: nn.Module) -> None:
             module.__class__ = _shard_conv1d_class(type(module))
     for module in shard.modules():
         if is_gated_silu_mlp(module):
-            module.forward = types.MethodType(_gated_mlp_forward, module)
+            module.forward = types.MethodType(_gated_mlp_first_forward, module)

@@ -76,7 +76,20 @@ class Sharded(nn.Module):
                 )
             modified = module.modified_parameters_names
             replicated_param_names = [n for n, _ in module_shards[0].named_parameters() if n not in modified]
-        self.sharded_param_names = names = tuple(replicated_param_names)
+        names = tuple(replicated_param_names)
+        # one flat buffer holds one dtype: the dtype that most of the named elements have is sharded, parameters of any
+        # other dtype (fp32 norms beside 16-bit weights) stay replicated on every rank
+        by_name0 = dict(module_shards[0].named_parameters())
+        volume = {}
+        for n in names:
+            if n in by_name0:
+                volume[by_name0[n].dtype] = volume.get(by_name0[n].dtype, 0) + by_name0[n].numel()
+        if len(volume) > 1:
+            main = max(volume, key=volume.get)
+            left = [n for n in names if n in by_name0 and by_name0[n].dtype != main]
+            logger.warning(f"{len(left)} parameters are not {main} and stay replicated on every rank: {left[:3]}{'...' if len(left) > 3 else ''}")
+            names = tuple(n for n in names if n not in left)
+        self.sharded_param_names = names
         if not names:
             logger.warning("Did not find any parameters to shard")
             return

@@ -169,3 +169,31 @@ def test_delay_init_parks_shards_on_the_host_until_the_first_forward():
     assert all(p.device == torch.device("cuda", 0) for shard in lazy.module_shards for p in shard.parameters())
     assert torch.equal(out, eager(ids.to("cuda:0")))
     torch.testing.assert_close(out.cpu(), model(ids), rtol=1e-5, atol=1e-5)
+
+
+def test_gated_mlp_fusion_is_checked_at_the_first_forward_and_respects_hooks():
+    """The fused gate/up forward takes over only where it reproduces the block's own forward: a block that looks the
+    same but computes something else, and a block whose gate_proj carries a hook, keep their own forward."""
+    from tensor_parallel_amd.shard_modules import _gated_mlp_forward, install_shard_kernels
+
+    class Odd(LlamaMLP):  # same children, another formula
+        def forward(self, x):
+            return self.down_proj(self.act_fn(self.up_proj(x)) * self.gate_proj(x))
+
+    torch.manual_seed(0)
+    x = torch.randn(5, 64).to(torch.bfloat16).to(DEV)
+    plain, odd, hooked = LlamaMLP(64, 96), Odd(64, 96), LlamaMLP(64, 96)
+    seen = []
+    hooked.gate_proj.register_forward_hook(lambda m, i, o: seen.append(1))
+    holder = nn.ModuleList([plain, odd, hooked]).to(torch.bfloat16).to(DEV)
+    want = [m(x) for m in holder]
+    install_shard_kernels(holder)
+    for m in holder:
+        assert type(m.gate_proj) is ShardLinear
+    with torch.no_grad():
+        got = [m(x) for m in holder] + [m(x) for m in holder]  # the second pass runs what the first pass settled on
+    for i in range(6):
+        torch.testing.assert_close(got[i].float(), want[i % 3].float(), rtol=2e-2, atol=2e-2 * want[i % 3].float().std().item())
+    assert getattr(plain.forward, "__func__", None) is _gated_mlp_forward
+    assert "forward" not in odd.__dict__ and "forward" not in hooked.__dict__
+    assert len(seen) == 3  # the reference call and both passes went through gate_proj's hook

@@ -170,3 +170,36 @@ def test_saved_state_dict_is_the_original_models(world, tensor_parallel):
             torch.testing.assert_close(got[name].cpu(), value, rtol=1e-6, atol=1e-7)
     with torch.no_grad():  # and the model still runs afterwards
         model_tp(input_ids=torch.zeros(1, 8, dtype=torch.long, device=DEV))
+
+
+def test_parameters_of_a_minority_dtype_stay_replicated():
+    """fp32 norms beside bf16 weights: the flat shards hold the dtype most of the replicated elements have; the rest
+    stays whole on every rank and the model computes what it computed before."""
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(16, 16), nn.LayerNorm(16), nn.LayerNorm(16), nn.Linear(16, 4)).to(torch.bfloat16)
+    model[1].float()  # the first norm's 32 elements are fp32, the second norm's stay bf16
+    x = torch.randn(3, 16)
+
+    class Cast(nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, t):
+            t = self.inner[0](t)
+            t = self.inner[1](t.float()).to(torch.bfloat16)
+            return self.inner[3](self.inner[2](t))
+
+    wrapped = Cast(model)
+    extra = nn.Parameter(torch.zeros(64, dtype=torch.bfloat16))  # makes bf16 the majority among the replicated parameters
+    wrapped.register_parameter("extra", extra)
+    with torch.no_grad():
+        want = wrapped(x.to(torch.bfloat16))
+    model_tp = tp.TensorParallel(deepcopy(wrapped), [DEV] * 2, sharded=True)
+    names = set(model_tp.sharding_manager.sharded_param_names)
+    assert "inner.2.weight" in names and "extra" in names and "inner.1.weight" not in names
+    norm32 = model_tp.module_shards[1].inner[1]
+    assert isinstance(norm32.weight, nn.Parameter) and norm32.weight.dtype == torch.float32
+    with torch.no_grad():
+        got = model_tp(x.to(torch.bfloat16).to(DEV))
+    torch.testing.assert_close(got.float().cpu(), want.float(), rtol=2e-2, atol=2e-2)

@@ -531,3 +531,18 @@ def test_reference_import_name_serves_the_same_objects():
         assert getattr(ref_name, name) is getattr(tp, name)
     assert by_ref_path is get_llama_config and split_by_ref_path is tp.Split
     assert ref_name.tensor_parallel.__module__ == "tensor_parallel_amd.factory"
+
+
+def test_convolution_layers_get_no_rule_and_a_warning(caplog):
+    """The automatic config leaves convolution layers whole on every rank (the reference's conv rules,
+    autoconfig.py:40-78, are not carried) instead of refusing the model."""
+    import logging
+
+    from tensor_parallel_amd.autoconfig import get_default_config
+
+    model = nn.Sequential(nn.Conv1d(4, 8, 3), nn.Flatten(), nn.Linear(16, 6))
+    with caplog.at_level(logging.WARNING):
+        cfg = get_default_config(model, [torch.device("cuda", 0)] * 2)
+    assert any("convolution" in r.getMessage() for r in caplog.records)
+    patterns = [p.pattern for p in cfg.state_rules]
+    assert any(p.startswith("^2.") for p in patterns) and not any(p.startswith("^0.") for p in patterns)
