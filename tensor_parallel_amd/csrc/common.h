@@ -46,6 +46,7 @@ struct Tuning {
     int skinny_pair;         // TPAMD_SKINNY_PAIR: 8-column form of the gated pair
     int skinny_resident;     // TPAMD_SKINNY_RESIDENT: x-resident kernel on/off
     int w8_split;            // TPAMD_W8_SPLIT: int8 K-split kernel on/off
+    int skinny_xlds;         // TPAMD_SKINNY_XLDS: 0 = gated pair at 4-16 rows through the older kernels
     int gemv_rows;           // TPAMD_GEMV_ROWS: wavefronts per block of the unrolled M <= 3 kernel (2, 4, 8, 16); 0 = the general kernel
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel
     int copy_tile_units;     // TPAMD_COPY_TILE_UNITS: 16-byte units per copy tile

@@ -29,6 +29,7 @@ Tuning read_tuning() {
     t.skinny_pair = env_int("TPAMD_SKINNY_PAIR");
     t.skinny_resident = env_int("TPAMD_SKINNY_RESIDENT");
     t.w8_split = env_int("TPAMD_W8_SPLIT");
+    t.skinny_xlds = env_int("TPAMD_SKINNY_XLDS");
     t.gemv_rows = env_int("TPAMD_GEMV_ROWS");
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
     t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");

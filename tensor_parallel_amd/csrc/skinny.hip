@@ -1167,6 +1167,188 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     return TPAMD_OK;
 }
 
+// ---- gated pair, 4 <= M <= 16: x through LDS in MFMA operand order, chunk by chunk ------------------------------------
+// One block of NW wavefronts per CU walks an even share of the 8-column tiles (8 gate rows + the 8 up rows of the same
+// columns). K is cut into units of 64 elements (128 bytes of every weight row: two loads of 8 rows x 128 bytes per
+// wavefront, two MFMAs); the units of a chunk of CH units are dealt to the wavefronts in turn. x is not kept in registers
+// (which is what limits the loads in flight of the x-resident kernel) but staged in LDS in operand order: slot (unit, m) of
+// 1 KiB holds for lane (q, j) the 8 elements x[j][unit * 64 + (q + 4 m) * 8 ...], so an operand read is one contiguous
+// ds_read_b128 per lane. Two chunk buffers: while a chunk is multiplied every wavefront fetches its share of the next chunk
+// into registers and stores it behind its last product of the chunk; one block-wide barrier per chunk. The weights go
+// through D register slots per wavefront that are refilled as soon as a unit has been handed to the MFMAs; the list of
+// units a wavefront walks (chunk by chunk, tile by tile) has the same length for every wavefront and entries past the end
+// of K multiply a slot of zeros, so the loop body has no branch and every wait counts exactly the loads issued behind
+// the one it needs. Rows past N and bytes past K are read from valid addresses of the same matrix (never stored; x is
+// zero there). The tiles' partial sums meet in LDS once, at the end, in the then idle x buffers.
+constexpr int XL_UNIT_K = 64;
+constexpr int XL_SROW = 144;   // staged weight row pitch: 128 bytes + 16 pad
+constexpr int XL_T_MAX = 8;    // tiles per block
+constexpr int XL_NW = 8, XL_D = 2, XL_CH = 32;
+constexpr size_t XL_LDS = 2 * XL_CH * 2048 + 2048 + XL_NW * 16 * XL_SROW;
+
+template <int DT, int NW, int D, int CH>
+__global__ __launch_bounds__(NW * 64) void skinny_pair_xlds_kernel(SkinnyParams p) {
+    constexpr int COLS = 8;
+    constexpr int XS = CH * 2 / NW;      // 1 KiB slots of a chunk of x per wavefront
+    constexpr int PER_TILE = CH / NW;    // list entries per tile and chunk
+    static_assert(CH % (NW * D) == 0, "every wavefront gets whole groups of D units of a chunk");
+    static_assert(XL_T_MAX * NW * 4 * 64 * 4 <= 2 * CH * 2048, "the partial sums fit the x buffers");
+    extern __shared__ __align__(16) char smem[];
+    // layout: [x: 2 buffers of CH * 2 KiB][2 KiB of zeros][stage: NW * 16 * XL_SROW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    char *zeros = smem + 2 * CH * 2048;
+    char *stage = zeros + 2048 + wave * (16 * XL_SROW);
+    float *red = reinterpret_cast<float *>(smem);
+
+    const int lr = lane & 15, lg = lane >> 4;
+    const int crow = lane >> 3, cpiece = lane & 7;
+    const int tiles_total = (p.N + COLS - 1) / COLS;
+    const int tb = static_cast<int>(static_cast<int64_t>(tiles_total) * blockIdx.x / gridDim.x);
+    const int te = static_cast<int>(static_cast<int64_t>(tiles_total) * (blockIdx.x + 1) / gridDim.x);
+    const int T = te - tb;
+    const int units_total = (p.K + XL_UNIT_K - 1) / XL_UNIT_K;
+    const int chunks = (units_total + CH - 1) / CH;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+    int ic = 0, it = 0, ij = 0;  // issue cursor: chunk, tile, position in the tile's list
+    uint4 wv[D][2];
+    auto issue = [&](uint4 (&dst)[2]) __attribute__((always_inline)) {
+        const bool live = ic < chunks;
+        const int c = live ? ic : chunks - 1, t = live ? it : T - 1;
+        int u = c * CH + wave + ij * NW;
+        u = u < units_total ? u : units_total - 1;
+        const int n0 = (tb + t) * COLS;
+        const int64_t kbyte = static_cast<int64_t>(u) * (XL_UNIT_K * 2) + cpiece * 16;
+        const int64_t kb = kbyte < static_cast<int64_t>(p.K) * 2 ? kbyte : 0;
+        const int row = n0 + crow < p.N ? n0 + crow : p.N - 1;
+        dst[0] = nt_load_u4(p.w + static_cast<int64_t>(row) * p.ldw * 2 + kb);
+        dst[1] = nt_load_u4(p.w2 + static_cast<int64_t>(row) * p.ldw * 2 + kb);
+        if (live && ++ij == PER_TILE) {
+            ij = 0;
+            if (++it == T) { it = 0; ++ic; }
+        }
+    };
+    // this wavefront's slots of a chunk of x: wave, wave + NW, ...
+    uint4 xr[XS];
+    auto fetch_x = [&](int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            const int sl = wave + i * NW;
+            const int k = (c * CH + (sl >> 1)) * XL_UNIT_K + (lg + 4 * (sl & 1)) * 8;
+            const bool ok = lr < p.M && k < p.K;
+            xr[i] = *reinterpret_cast<const uint4 *>(p.x + (ok ? (static_cast<int64_t>(lr) * p.ldx + k) * 2 : 0));
+        }
+    };
+    auto store_x = [&](int c) __attribute__((always_inline)) {
+        char *xb = smem + (c & 1) * (CH * 2048);
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            const int sl = wave + i * NW;
+            const int k = (c * CH + (sl >> 1)) * XL_UNIT_K + (lg + 4 * (sl & 1)) * 8;
+            const bool ok = lr < p.M && k < p.K;
+            const uint4 v = xr[i];
+            *reinterpret_cast<uint4 *>(xb + (sl * 64 + lane) * 16) = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+        }
+    };
+
+    fetch_x(0);
+#pragma unroll
+    for (int d = 0; d < D; ++d) issue(wv[d]);
+    if (wave < 2) *reinterpret_cast<uint4 *>(zeros + (wave * 64 + lane) * 16) = zero4;
+    store_x(0);
+    __syncthreads();
+
+    f32x4 acc[XL_T_MAX];
+#pragma unroll
+    for (int t = 0; t < XL_T_MAX; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int c = 0; c < chunks; ++c) {
+        const char *xb = smem + (c & 1) * (CH * 2048);
+        if (c + 1 < chunks) fetch_x(c + 1);
+        for (int t = 0; t < T; ++t) {
+            f32x4 cur = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int i0 = 0; i0 < PER_TILE; i0 += D) {
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    const int ul = wave + (i0 + d) * NW;  // unit within the chunk
+                    // fetch order (8 rows x 128 bytes per load) -> MFMA operand order through the wavefront's LDS tile
+                    *reinterpret_cast<uint4 *>(stage + crow * XL_SROW + cpiece * 16) = wv[d][0];
+                    *reinterpret_cast<uint4 *>(stage + (crow + 8) * XL_SROW + cpiece * 16) = wv[d][1];
+                    __builtin_amdgcn_wave_barrier();
+                    const uint4 a0 = *reinterpret_cast<const uint4 *>(stage + lr * XL_SROW + lg * 16);
+                    const uint4 a1 = *reinterpret_cast<const uint4 *>(stage + lr * XL_SROW + (lg + 4) * 16);
+                    const char *xsl = c * CH + ul < units_total ? xb + ul * 2048 : zeros;
+                    const uint4 b0 = *reinterpret_cast<const uint4 *>(xsl + lane * 16);
+                    const uint4 b1 = *reinterpret_cast<const uint4 *>(xsl + 1024 + lane * 16);
+                    __builtin_amdgcn_wave_barrier();
+                    issue(wv[d]);
+                    cur = mfma16<DT>(a0, b0, cur);
+                    cur = mfma16<DT>(a1, b1, cur);
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < XL_T_MAX; ++tt)
+                if (t == tt) acc[tt] += cur;
+        }
+        if (c + 1 < chunks) store_x(c + 1);
+        __syncthreads();  // the next chunk is staged; after the last chunk: everybody is done with x
+    }
+    // the tiles' partial sums meet in the x buffers; element e -> output (tile e / 256, m = e / 16 % 16, column e % 16 < 8)
+#pragma unroll
+    for (int tt = 0; tt < XL_T_MAX; ++tt)
+        if (tt < T) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((tt * NW + wave) * 4 + i) * 64 + lane] = acc[tt][i];
+        }
+    __syncthreads();
+    for (int e = tid; e < T * 256; e += NW * 64) {
+        const int tt = e >> 8, m = (e >> 4) & 15, nl = e & 15;
+        const int n = (tb + tt) * COLS + nl;
+        if (m < p.M && nl < COLS && n < p.N) {
+            const int src_lane = (nl >> 2) * 16 + m, i = nl & 3;
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                s0 += red[((tt * NW + w) * 4 + i) * 64 + src_lane];
+                s1 += red[((tt * NW + w) * 4 + i) * 64 + src_lane + 32];  // row nl + 8 of the tile: the up sum
+            }
+            skinny_store_output<DT, SK_SWIGLU>(p, s0, s1, m, n);
+        }
+    }
+}
+
+// Gated pair with 16-bit weights, 4 <= M <= 16, at most XL_T_MAX tiles of 8 columns per CU. *done = false: not taken.
+template <int DT>
+int launch_pair_xlds(const SkinnyParams &p, int cus, hipStream_t s, bool *done) {
+    *done = false;
+    if (tuning().skinny_xlds == 0) return TPAMD_OK;
+    const int64_t tiles = (p.N + 7) / 8;
+    if (p.M < 4 || p.M > 16 || p.K % 8 != 0 || tiles > static_cast<int64_t>(XL_T_MAX) * cus) return TPAMD_OK;
+    if (tuning().skinny_xlds == TUNE_UNSET) {
+        // Measured against the older kernels (inside a HIP graph, rows 4 / 8 / 16): 5504 columns at K = 4096 19.6 / 21.1 /
+        // 21.9 -> 18.5 / 18.9 / 20.3 us, 2752 columns 13.8 / 15.1 / 16.6 -> 13.6 / 13.7 / 15.1 us, 14336 columns 43.3 / 44.9 /
+        // 41.1 -> 39.1 / 39.6 / 41.0 us. It loses where the last chunk of K is mostly padding (K = 5504: 86 units in chunks
+        // of 32, 11008 columns 46.6 / 50.6 / 48.9 -> 48.1 / 48.8 / 50.1 us) and, below 12 rows, where there is less than one
+        // tile per CU (1376 columns at K = 8192, 8 rows: 13.7 -> 15.8 us; 16 rows: 21.5 -> 17.6 us).
+        const int units = (p.K + XL_UNIT_K - 1) / XL_UNIT_K, padded = (units + XL_CH - 1) / XL_CH * XL_CH;
+        if (padded * 100 > units * 107) return TPAMD_OK;
+        if (tiles < cus && p.M < 12) return TPAMD_OK;
+    }
+    static thread_local int configured_dev = -1;  // per instantiation and host thread
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_pair_xlds_kernel<DT, XL_NW, XL_D, XL_CH>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(XL_LDS)));
+        configured_dev = dev;
+    }
+    const unsigned grid = static_cast<unsigned>(tiles < cus ? tiles : cus);
+    hipLaunchKernelGGL((skinny_pair_xlds_kernel<DT, XL_NW, XL_D, XL_CH>), dim3(grid), dim3(XL_NW * 64), XL_LDS, s, p);
+    TPAMD_HIP(hipGetLastError());
+    *done = true;
+    return TPAMD_OK;
+}
+
 template <int DT, bool W8, int MODE>
 int launch_skinny(const SkinnyParams &p, hipStream_t s) {
     if constexpr (W8) {
@@ -1178,6 +1360,11 @@ int launch_skinny(const SkinnyParams &p, hipStream_t s) {
         int dev = 0, cus = 256;
         TPAMD_HIP(hipGetDevice(&dev));
         if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+        if constexpr (MODE == SK_SWIGLU) {
+            bool done = false;
+            const int rc = launch_pair_xlds<DT>(p, cus, s, &done);
+            if (rc != TPAMD_OK || done) return rc;
+        }
         if (pick_resident<MODE>(p, cus)) return launch_resident<DT, MODE>(p, cus, s);
     }
     if constexpr (MODE == SK_SWIGLU && !W8) {

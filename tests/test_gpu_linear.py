@@ -2,6 +2,7 @@
 
 Tolerances: bf16/fp16 results are compared with the fp32 CPU product of the same bf16/fp16 inputs at
 rtol 2e-2 (atol scaled to the typical output magnitude), fp32 results at rtol 1e-5."""
+import ctypes
 import math
 
 import pytest
@@ -338,6 +339,7 @@ def test_x_resident_weight_streaming_kernel(dtype, M, N, K, tune):
     on a multiple of 8, a ragged last K chunk, K above 4096 and above 6144 (6 and 8 chunks per wavefront), bias and
     GELU, the gated pair."""
     tune("TPAMD_SKINNY_RESIDENT", "1")
+    tune("TPAMD_SKINNY_XLDS", "0")  # the gated pair would otherwise go to the kernel that stages x in LDS
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
@@ -350,7 +352,44 @@ def test_x_resident_weight_streaming_kernel(dtype, M, N, K, tune):
     torch.testing.assert_close(h.float(), plain.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
 
 
-@pytest.mark.parametrize("case", ["tiles256_split", "resident_pair", "resident_single"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [4, 7, 12, 16])
+@pytest.mark.parametrize("N,K", [(8, 64), (64, 64), (133, 200), (1028, 1000), (2740, 4096), (520, 5504), (4100, 2048), (300, 8192), (260, 7000),
+                                 (16400, 512)])
+def test_gated_pair_with_x_staged_in_lds(dtype, M, N, K, tune):
+    """The gated-pair kernel for 4 to 16 rows that stages x in LDS chunk by chunk (forced on every shape): one tile, fewer
+    tiles than CUs, several tiles per block, column counts that are not multiples of 8, K that is not a multiple of the
+    64-element unit, one partly filled chunk of K, several chunks with a ragged last one, 8 tiles per CU (16400 columns:
+    2050 tiles on 256 CUs), and x with a row pitch above K. Against the oracle's gated hidden state and against the older
+    kernels."""
+    tune("TPAMD_SKINNY_XLDS", "1")
+    x_wide = rnd((M, K + 24), 1, 1.0, dtype).to(DEV)
+    x = x_wide[:, 8:K + 8]
+    w, w2 = rnd((N, K), 0, 0.02, dtype), rnd((N, K), 5, 0.02, dtype)
+    h = _native.swiglu_up(x, w.to(DEV), w2.to(DEV))
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float().cpu(), w.float(), w2.float()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    tune("TPAMD_SKINNY_XLDS", "0")
+    older = _native.swiglu_up(x, w.to(DEV), w2.to(DEV))
+    torch.testing.assert_close(h.float(), older.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+
+
+def test_gated_pair_with_x_staged_in_lds_leaves_rows_past_m_and_columns_past_n_alone(tune):
+    tune("TPAMD_SKINNY_XLDS", "1")
+    M, N, K, ldy = 5, 1001, 4096, 1016
+    x, w, w2 = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N, K), 5, 0.02).to(DEV)
+    buf = torch.full((8 * ldy,), 7.0, dtype=torch.bfloat16, device=DEV)
+    y = buf[ldy:ldy + M * ldy].view(M, ldy)
+    rc = _native.lib().tpamd_swiglu_up(x.data_ptr(), w.data_ptr(), w2.data_ptr(), y.data_ptr(), M, N, K, K, K, ldy, _native.dtype_code(torch.bfloat16),
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(y[:, :N].float().cpu(), ofw.gated_mlp_hidden(x.float().cpu(), w.float().cpu(), w2.float().cpu()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    assert bool((y[:, N:] == 7.0).all()) and bool((buf[:ldy] == 7.0).all()) and bool((buf[ldy + M * ldy:] == 7.0).all())
+
+
+@pytest.mark.parametrize("case", ["tiles256_split", "resident_pair", "resident_single", "xlds_pair"])
 def test_other_dispatch_paths_inside_a_hip_graph(case, tune):
     """The 256 x 256 tiling with K split over blocks (two launches sharing the scratch buffer) and the x-resident
     weight-streaming kernel, recorded into a HIP graph after a warm-up call: every replay gives the eager result,
@@ -359,11 +398,15 @@ def test_other_dispatch_paths_inside_a_hip_graph(case, tune):
         tune("TPAMD_GEMM_TILE", "256")
         tune("TPAMD_GEMM_SPLITK256", "3")
         M, N, K = 300, 520, 1088
+    elif case == "xlds_pair":
+        tune("TPAMD_SKINNY_XLDS", "1")
+        M, N, K = 13, 2740, 5504
     else:
         tune("TPAMD_SKINNY_RESIDENT", "1")
+        tune("TPAMD_SKINNY_XLDS", "0")
         M, N, K = 16, 2740, 4096
     x, w, w2 = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N, K), 5, 0.02).to(DEV)
-    fn = (lambda: _native.swiglu_up(x, w, w2)) if case == "resident_pair" else (lambda: _native.linear(x, w))
+    fn = (lambda: _native.swiglu_up(x, w, w2)) if case in ("resident_pair", "xlds_pair") else (lambda: _native.linear(x, w))
     eager = fn()
     torch.cuda.synchronize()
     out = torch.empty_like(eager)
