@@ -51,6 +51,7 @@ struct Tuning {
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel
     int copy_tile_units;     // TPAMD_COPY_TILE_UNITS: 16-byte units per copy tile
     int copy_blocks_per_cu;  // TPAMD_COPY_BLOCKS_PER_CU
+    int copy_sort;           // TPAMD_COPY_SORT: 0 = tiles stay in the order of the jobs instead of the order of their source addresses
     int copy_nt;             // TPAMD_COPY_NT: bit 0 non-temporal loads, bit 1 non-temporal stores of the slicing kernel
 };
 const Tuning &tuning();

@@ -34,6 +34,7 @@ Tuning read_tuning() {
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
     t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");
     t.copy_blocks_per_cu = env_int("TPAMD_COPY_BLOCKS_PER_CU");
+    t.copy_sort = env_int("TPAMD_COPY_SORT");
     t.copy_nt = env_int("TPAMD_COPY_NT");
     return t;
 }
