@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # Fabric bytes per launch of the fused gate/up GEMM at M = 4096, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
 # each scaled by what the same counter reads for the slicing kernel's known 13.476 GB (factors 1.98 and 1.00):
 # profiles/pmc_fetch_write_bench_kernels.txt. A counter reading cannot be taken inside this script.
-MEASURED_TRAFFIC_BYTES_M4096 = 629.3e6
+MEASURED_TRAFFIC_BYTES_M4096 = 628.8e6
 
 
 def cpu_baseline(seconds_budget: float = 15.0) -> dict:
@@ -234,15 +234,15 @@ def ceilings(torch, _native, dev, which="all") -> int:
         sizes = (("llama7b_down_shard_45MB", FFN_SHARD * D_MODEL * 2, 6), ("llama7b_gate_up_shards_90MB", 2 * FFN_SHARD * D_MODEL * 2, 4),
                  ("llama2_7b_split_tensors_13.5GB", 13476298752, 1))
         for label, nbytes, copies in sizes:
-            nbytes = nbytes // 32768 * 32768
+            nbytes = nbytes // 131072 * 131072
             srcs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
             dsts = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(copies)]
             row = {}
             for mode, what, moved in ((0, "read_only", nbytes), (1, "write_only", nbytes), (2, "copy_read_plus_write", 2 * nbytes)):
                 best = None
                 for nt in (1, 0):
-                    for piece in (4096, 16384, 32768):
-                        for per_cu in (4, 8, 16):
+                    for piece in (4096, 16384, 32768, 131072):  # 131072: bursts of one 1024-thread block (1 or 2 blocks per CU)
+                        for per_cu in ((1, 2) if piece == 131072 else (4, 8, 16)):
                             us = settled_us(lambda i: probes.tpamd_probe_stream(mode, nt, piece, vp(srcs[i % copies].data_ptr()), vp(dsts[i % copies].data_ptr()),
                                                                                 nbytes, cus * per_cu, vp(sink.data_ptr()), stream()), 0.05, 20 if nbytes < 1e9 else 4)
                             if best is None or us < best[0]:

@@ -1,7 +1,8 @@
 // Measurement probes, built into their own library (libtpamd_probes.so) and used only by `bench.py --ceilings`: what one
 // MI355X sustains on the two resources the hot path is bound by, measured with nothing else in the way.
 //   tpamd_probe_mfma    a loop of nothing but bf16 MFMAs (no loads, no LDS), operands constant or random
-//   tpamd_probe_stream  a read-only / write-only / copy stream over a buffer, 16 bytes per lane, non-temporal
+//   tpamd_probe_stream  a read-only / write-only / copy stream over a buffer, 16 bytes per lane, plain or non-temporal, in small
+//                       steps of many 256-thread blocks or in 128 KiB bursts of one 1024-thread block per CU
 // The product library does not link this file.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -81,9 +82,40 @@ __global__ __launch_bounds__(256) void stream_kernel(const char *src, char *dst,
     if (MODE == 0 && keep == 0x12345679u) sink[threadIdx.x] = 1.f;
 }
 
+// The same stream in bursts: one 1024-thread block moves 128 KiB at a time, all of its loads first (8 per lane), then, once the
+// last one has arrived, all of its stores. MODE and NT as above.
+template <int MODE, bool NT>
+__global__ __launch_bounds__(1024) void burst_kernel(const char *src, char *dst, uint64_t pieces, float *sink) {
+    constexpr int U = 8;
+    uint32_t keep = 0;
+    for (uint64_t p = blockIdx.x; p < pieces; p += gridDim.x) {
+        const uint64_t off = p * 131072 + threadIdx.x * 16;
+        v4u v[U];
+#pragma unroll
+        for (int i = 0; i < U; ++i) {
+            if constexpr (MODE == 1) v[i] = v4u{static_cast<uint32_t>(p), 1u, 2u, 3u};
+            else if constexpr (NT) v[i] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(src + off + i * 16384));
+            else v[i] = *reinterpret_cast<const v4u *>(src + off + i * 16384);
+        }
+        if constexpr (MODE == 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < U; ++i) {
+            if constexpr (MODE == 0) keep ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+            else if constexpr (NT) __builtin_nontemporal_store(v[i], reinterpret_cast<v4u *>(dst + off + i * 16384));
+            else *reinterpret_cast<v4u *>(dst + off + i * 16384) = v[i];
+        }
+    }
+    if (MODE == 0 && keep == 0x12345679u) sink[threadIdx.x] = 1.f;
+}
+
 template <int MODE>
 void launch_stream(bool nt, int piece, int blocks, hipStream_t s, const char *src, char *dst, uint64_t bytes, float *sink) {
     const uint64_t pieces = bytes / piece;
+    if (piece == 131072) {
+        if (nt) hipLaunchKernelGGL((burst_kernel<MODE, true>), dim3(blocks), dim3(1024), 0, s, src, dst, pieces, sink);
+        else hipLaunchKernelGGL((burst_kernel<MODE, false>), dim3(blocks), dim3(1024), 0, s, src, dst, pieces, sink);
+        return;
+    }
 #define TPAMD_PROBE_CASE(NTV, P) \
     if (nt == NTV && piece == P) hipLaunchKernelGGL((stream_kernel<MODE, NTV, P>), dim3(blocks), dim3(256), 0, s, src, dst, pieces, sink)
     TPAMD_PROBE_CASE(true, 16384); TPAMD_PROBE_CASE(false, 16384);
@@ -109,11 +141,12 @@ extern "C" double tpamd_probe_mfma_flops(int shape, int blocks, int iters) {
     return per_wave_iter * 4.0 * blocks * iters;
 }
 
-// mode 0 read, 1 write, 2 copy; nt != 0: non-temporal accesses; piece: 4096, 16384 or 32768 bytes per block step;
-// bytes must be a multiple of 32768.
+// mode 0 read, 1 write, 2 copy; nt != 0: non-temporal accesses; piece: 4096, 16384 or 32768 bytes per step of a 256-thread
+// block, or 131072: bursts of a 1024-thread block; bytes must be a multiple of 32768 (of 131072 for bursts).
 extern "C" int tpamd_probe_stream(int mode, int nt, int piece, const void *src_dev, void *dst_dev, uint64_t bytes, int blocks,
                                   void *sink_dev, void *stream) {
-    if (bytes % 32768 != 0 || blocks <= 0 || (piece != 4096 && piece != 16384 && piece != 32768)) return -1;
+    if (bytes % 32768 != 0 || blocks <= 0 || (piece != 4096 && piece != 16384 && piece != 32768 && piece != 131072)) return -1;
+    if (piece == 131072 && bytes % 131072 != 0) return -1;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const char *src = static_cast<const char *>(src_dev);
     char *dst = static_cast<char *>(dst_dev);
