@@ -41,11 +41,11 @@ struct Tuning {
     int gemm_splitk;         // TPAMD_GEMM_SPLITK: K splits of the 128 x 128 tiling
     int gemm_splitk256;      // TPAMD_GEMM_SPLITK256: K splits of the 256 x 256 tiling
     int gemm_tile;           // TPAMD_GEMM_TILE: 256 or 128
-    int gemm_balance;        // TPAMD_GEMM_BALANCE: 0 = never split the tiles of a last, partly filled round over K
     int skinny_cg;           // TPAMD_SKINNY_CG: column groups per block (1, 2, 4)
     int skinny_pair;         // TPAMD_SKINNY_PAIR: 8-column form of the gated pair
     int skinny_resident;     // TPAMD_SKINNY_RESIDENT: x-resident kernel on/off
     int w8_split;            // TPAMD_W8_SPLIT: int8 K-split kernel on/off
+    int w8_cols;             // TPAMD_W8_COLS: int8 K-split kernel whose wavefronts own columns (x of the split in LDS): 0 = off, 1 = whenever the shape allows
     int skinny_xlds;         // TPAMD_SKINNY_XLDS: 0 = gated pair at 4-16 rows through the older kernels
     int gemv_rows;           // TPAMD_GEMV_ROWS: wavefronts per block of the unrolled M <= 3 kernel (2, 4, 8, 16); 0 = the general kernel
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel

@@ -24,11 +24,11 @@ Tuning read_tuning() {
     t.gemm_splitk = env_int("TPAMD_GEMM_SPLITK");
     t.gemm_splitk256 = env_int("TPAMD_GEMM_SPLITK256");
     t.gemm_tile = env_int("TPAMD_GEMM_TILE");
-    t.gemm_balance = env_int("TPAMD_GEMM_BALANCE");
     t.skinny_cg = env_int("TPAMD_SKINNY_CG");
     t.skinny_pair = env_int("TPAMD_SKINNY_PAIR");
     t.skinny_resident = env_int("TPAMD_SKINNY_RESIDENT");
     t.w8_split = env_int("TPAMD_W8_SPLIT");
+    t.w8_cols = env_int("TPAMD_W8_COLS");
     t.skinny_xlds = env_int("TPAMD_SKINNY_XLDS");
     t.gemv_rows = env_int("TPAMD_GEMV_ROWS");
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");

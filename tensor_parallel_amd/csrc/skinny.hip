@@ -705,15 +705,288 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParam
     }
 }
 
-// y[m][n] = act(sum over splits of part[split][m][n] + bias[n])
-template <int DT>
+// y[m][n] = act(sum over splits of part[split][m][n] + bias[n]); VEC: four consecutive n per thread (N a multiple of 4),
+// the planes requested eight at a time and added in plane order
+template <int DT, bool VEC>
 __global__ __launch_bounds__(256) void skinny_w8_finish_kernel(SkinnyParams p, const float *part, int splits) {
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (e >= static_cast<int64_t>(p.M) * p.N) return;
-    const int m = static_cast<int>(e / p.N), n = static_cast<int>(e % p.N);
-    float v = 0.f;
-    for (int sp = 0; sp < splits; ++sp) v += part[static_cast<int64_t>(sp) * p.M * p.N + e];
-    skinny_store_output<DT, SK_LINEAR>(p, v, 0.f, m, n);
+    const int64_t plane = static_cast<int64_t>(p.M) * p.N;
+    if constexpr (VEC) {
+        const int64_t e = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+        if (e >= plane) return;
+        const int m = static_cast<int>(e / p.N), n = static_cast<int>(e % p.N);
+        f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+        int sp = 0;
+        for (; sp + 8 <= splits; sp += 8) {
+            f32x4 t[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) t[j] = *reinterpret_cast<const f32x4 *>(part + (sp + j) * plane + e);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v += t[j];
+        }
+        for (; sp < splits; ++sp) v += *reinterpret_cast<const f32x4 *>(part + sp * plane + e);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) skinny_store_output<DT, SK_LINEAR>(p, v[i], 0.f, m, n + i);
+    } else {
+        const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+        if (e >= plane) return;
+        const int m = static_cast<int>(e / p.N), n = static_cast<int>(e % p.N);
+        float v = 0.f;
+        for (int sp = 0; sp < splits; ++sp) v += part[sp * plane + e];
+        skinny_store_output<DT, SK_LINEAR>(p, v, 0.f, m, n);
+    }
+}
+
+// Launches the finishing pass over [splits][M][N] partial sums.
+template <int DT>
+int launch_w8_finish(const SkinnyParams &p, const float *part, int splits, hipStream_t s) {
+    const int64_t outputs = static_cast<int64_t>(p.M) * p.N;
+    if (p.N % 4 == 0) hipLaunchKernelGGL((skinny_w8_finish_kernel<DT, true>), dim3(static_cast<unsigned>((outputs / 4 + 255) / 256)), dim3(256), 0, s, p, part, splits);
+    else hipLaunchKernelGGL((skinny_w8_finish_kernel<DT, false>), dim3(static_cast<unsigned>((outputs + 255) / 256)), dim3(256), 0, s, p, part, splits);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
+// ---- int8 weights, up to 64 rows: K split over blocks, x of the split resident in LDS, wavefronts own columns ----------
+// The grid is (column ranges, K splits of KU * 128 elements [+ blocks for the outlier columns]). A block first stages the
+// M rows of x of its K split in LDS in MFMA operand order (slot ((unit * 4 + o) * MT + t) of 1 KiB: lane (m = lane % 16,
+// g = lane / 16) holds the 8 elements x[16 t + m][unit * 128 + (o / 2) * 64 + g * 16 + (o % 2) * 8 ...], which is what
+// meets the two halves of a 16-byte int8 fragment); that is the only block-wide barrier. After it a wavefront owns every
+// NW-th tile of 16 weight rows of the block's column range over the whole split and walks them two at a time: a unit is 128
+// bytes of the 32 rows of a pair (four loads of 8 rows x 128 bytes), D units are in flight in registers, a unit goes from
+// fetch order to operand order through a wavefront-private LDS tile (rows of 128 bytes, pieces swizzled instead of padded),
+// is converted to the activation dtype, and every x operand read from LDS meets both tiles of the pair. Nothing is
+// exchanged between wavefronts: a tile's sums are scaled per weight row and stored to the [plane][M][N] fp32 array straight
+// from the accumulators (DIRECT, a single plane: bias, activation and the store to y happen here). Every weight load is
+// issued unconditionally (past the last tile: the first bytes of the matrix, which stay in cache), so that each wait counts
+// exactly the loads issued behind the one it needs. Timed with the products removed the kernel is no faster: its pace is
+// set by the weight stream, the staging of x before the first product, and the partial sums (M * N * 4 bytes per plane,
+// written here and read again by skinny_w8_finish_kernel, which adds the planes). The outlier columns of x (gathered into
+// LDS in operand order, groups of 32) meet w_out in blocks of their own, one tile per wavefront, which fill one more plane.
+constexpr int WC_NW = 8, WC_UNIT_K = 128, WC_STAGE = 32 * 128;  // per wavefront: two tiles of 16 staged rows
+
+template <int DT, int MT, int KU, bool DIRECT>
+__global__ __launch_bounds__(WC_NW * 64) void skinny_w8_cols_kernel(SkinnyParams p, float *part, int cols_per_block, int k_planes) {
+    constexpr int NW = WC_NW;
+    extern __shared__ __align__(16) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    const int crow = lane >> 3, cpiece = lane & 7;
+    const int plane = blockIdx.y;
+    const int col_begin = blockIdx.x * cols_per_block;
+    const int col_end = col_begin + cols_per_block < p.N ? col_begin + cols_per_block : p.N;
+    const int tiles = (col_end - col_begin + 15) / 16;
+    const int my_tiles = tiles > wave ? (tiles - wave + NW - 1) / NW : 0;  // tiles wave, wave + NW, ...
+    const int pairs = (my_tiles + 1) / 2;
+
+    auto store_tile = [&](const f32x4 (&v)[MT], int n0, int to_plane) __attribute__((always_inline)) {
+        // D[n_local][m_local]: lane -> m_local = lr, register i -> n_local = 4 * lg + i
+        const int n = n0 + lg * 4;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = t * 16 + lr;
+            if (m >= p.M) continue;
+            if constexpr (DIRECT) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < col_end) skinny_store_output<DT, SK_LINEAR>(p, v[t][i], 0.f, m, n + i);
+            } else {
+                float *dst = part + (static_cast<int64_t>(to_plane) * p.M + m) * p.N + n;
+                if (n + 3 < col_end && (p.N & 3) == 0) *reinterpret_cast<f32x4 *>(dst) = v[t];
+                else
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < col_end) dst[i] = v[t][i];
+            }
+        }
+    };
+
+    if (plane >= k_planes) {
+        // The outlier plane: x values of the outlier columns in LDS (slot g * MT + t: lane (m, q) holds outliers
+        // 32 g + 8 q ... + 8 of row 16 t + m), then one MFMA per tile, group and 16 rows of x. Block (bx, k_planes + j)
+        // takes tiles 8 j ... 8 j + 7 of the column range, one per wavefront. Every gather is issued unconditionally
+        // from a clamped address, so that the eight of a group are in flight together.
+        const int groups = (p.n_out + 31) / 32;
+        const uint16_t *xs = reinterpret_cast<const uint16_t *>(p.x);
+        for (int sl = wave; sl < groups * MT; sl += NW) {
+            const int g = sl / MT, t = sl % MT;
+            const int m = t * 16 + lr < p.M ? t * 16 + lr : p.M - 1;
+            int idx[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int o = g * 32 + lg * 8 + j;
+                idx[j] = p.outlier_idx[o < p.n_out ? o : p.n_out - 1];
+            }
+            uint32_t val[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) val[j] = xs[static_cast<int64_t>(m) * p.ldx + idx[j]];
+            uint32_t q[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const bool ok = g * 32 + lg * 8 + j < p.n_out && t * 16 + lr < p.M;
+                q[j >> 1] |= (ok ? val[j] : 0u) << ((j & 1) * 16);
+            }
+            *reinterpret_cast<uint4 *>(smem + (sl * 64 + lane) * 16) = make_uint4(q[0], q[1], q[2], q[3]);
+        }
+        __syncthreads();
+        const uint16_t *wo = reinterpret_cast<const uint16_t *>(p.w_out);
+        const int tile = (plane - k_planes) * NW + wave;
+        if (tile >= tiles) return;
+        const int n0 = col_begin + tile * 16;
+        const int wr = n0 + lr < p.N ? n0 + lr : p.N - 1;
+        f32x4 acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int g = 0; g < groups; ++g) {
+            uint32_t val[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int o = g * 32 + lg * 8 + j;
+                val[j] = wo[static_cast<int64_t>(wr) * p.ld_wout + (o < p.n_out ? o : p.n_out - 1)];
+            }
+            uint32_t q[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j >> 1] |= (g * 32 + lg * 8 + j < p.n_out ? val[j] : 0u) << ((j & 1) * 16);
+            const uint4 a = make_uint4(q[0], q[1], q[2], q[3]);
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[t] = mfma16<DT>(a, *reinterpret_cast<const uint4 *>(smem + ((g * MT + t) * 64 + lane) * 16), acc[t]);
+        }
+        store_tile(acc, n0, k_planes);
+        return;
+    }
+
+    char *stage = smem + KU * 4 * MT * 1024 + wave * WC_STAGE;
+    const int64_t k_begin = static_cast<int64_t>(plane) * (KU * WC_UNIT_K);
+
+    // x of this split first (it comes from L2 and must not queue behind the weights: loads return in order)
+    constexpr int XS = KU * 4 * MT / NW;
+    uint4 xr[XS];
+#pragma unroll
+    for (int j = 0; j < XS; ++j) {
+        const int sl = wave + j * NW;
+        const int t = sl % MT, o = (sl / MT) & 3, u = sl / (4 * MT);
+        const int64_t k = k_begin + u * WC_UNIT_K + (o >> 1) * 64 + lg * 16 + (o & 1) * 8;
+        const int m = t * 16 + lr;
+        const bool ok = m < p.M && k < p.K;
+        xr[j] = *reinterpret_cast<const uint4 *>(p.x + (ok ? (static_cast<int64_t>(m) * p.ldx + k) * 2 : 0));
+    }
+
+    // weights: unit u of the pair of tiles (2 q, 2 q + 1) of this wavefront into ring slot S; for a tile past the last one the
+    // first bytes of the matrix. A slot: [tile A rows 0-7, A rows 8-15, B rows 0-7, B rows 8-15], 128 bytes of each row.
+    // The four row addresses of a pair are worked out once (set_pair); a unit is an immediate offset from them. In the last
+    // plane of a K that does not fill it, units past the end of K read the first bytes of the matrix instead (x is 0 there).
+    constexpr int D = 4;
+    static_assert(KU % D == 0, "the ring divides a tile");
+    uint4 wv[D][4];
+    const char *rowp[4];
+    const bool k_ragged = k_begin + KU * WC_UNIT_K > p.K;  // uniform over the block
+    auto set_pair = [&](int q) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int i = 2 * q + h;
+            const int n0 = col_begin + (wave + i * NW) * 16;
+            const bool live = i < my_tiles;
+            const int r0 = n0 + crow < p.N ? n0 + crow : p.N - 1;
+            const int r1 = n0 + crow + 8 < p.N ? n0 + crow + 8 : p.N - 1;
+            rowp[2 * h] = p.w + (live ? static_cast<int64_t>(r0) * p.ldw + k_begin : 0) + cpiece * 16;
+            rowp[2 * h + 1] = p.w + (live ? static_cast<int64_t>(r1) * p.ldw + k_begin : 0) + cpiece * 16;
+        }
+    };
+    auto issue = [&](auto sc_, auto uc) __attribute__((always_inline)) {
+        constexpr int S = decltype(sc_)::value, u = decltype(uc)::value;
+        if (k_ragged) {
+            const bool in_k = k_begin + u * WC_UNIT_K + cpiece * 16 < p.K;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) wv[S][r] = nt_load_u4(in_k ? rowp[r] + u * WC_UNIT_K : p.w + cpiece * 16);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) wv[S][r] = nt_load_u4(rowp[r] + u * WC_UNIT_K);
+        }
+    };
+    set_pair(0);
+    static_for<D>([&](auto sc_) { issue(sc_, sc_); });
+
+#pragma unroll
+    for (int j = 0; j < XS; ++j) {
+        const int sl = wave + j * NW;
+        const int t = sl % MT, o = (sl / MT) & 3, u = sl / (4 * MT);
+        const int64_t k = k_begin + u * WC_UNIT_K + (o >> 1) * 64 + lg * 16 + (o & 1) * 8;
+        const bool ok = t * 16 + lr < p.M && k < p.K;
+        const uint4 v = xr[j];
+        *reinterpret_cast<uint4 *>(smem + (sl * 64 + lane) * 16) = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    }
+    __syncthreads();
+
+    // staged rows are 128 bytes, piece c of row r at piece c ^ (r / 2 % 8): conflict-free for the writes (8 rows x 8 pieces)
+    // and for the reads (16 rows x 1 piece per quarter wavefront) without padding
+    const int wr_off = crow * 128 + ((cpiece ^ (crow >> 1)) * 16);           // rows crow and crow + 8 share r / 2 % 8 ^ 4
+    const int wr_off8 = (crow + 8) * 128 + ((cpiece ^ ((crow >> 1) + 4)) * 16);
+    int rd_off[2];
+#pragma unroll
+    for (int v = 0; v < 2; ++v) rd_off[v] = lr * 128 + (((v * 4 + lg) ^ ((lr >> 1) & 7)) * 16);
+
+    for (int q = 0; q < pairs; ++q) {
+        f32x4 acc[2][MT];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[h][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // the tiles' scales are requested before further weights
+        float sc[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = col_begin + (wave + (2 * q + h) * NW) * 16 + lg * 4 + e;
+                sc[h][e] = p.scale[n < p.N ? n : p.N - 1];
+            }
+        static_for<KU>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            constexpr int S = u % D;
+            *reinterpret_cast<uint4 *>(stage + wr_off) = wv[S][0];
+            *reinterpret_cast<uint4 *>(stage + wr_off8) = wv[S][1];
+            *reinterpret_cast<uint4 *>(stage + 2048 + wr_off) = wv[S][2];
+            *reinterpret_cast<uint4 *>(stage + 2048 + wr_off8) = wv[S][3];
+            __builtin_amdgcn_wave_barrier();
+            uint4 wt[2][2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int v = 0; v < 2; ++v) wt[h][v] = *reinterpret_cast<const uint4 *>(stage + h * 2048 + rd_off[v]);
+            __builtin_amdgcn_wave_barrier();
+            if constexpr (u + D == KU) set_pair(q + 1);  // the units requested from here on belong to the next pair
+            issue(std::integral_constant<int, S>{}, std::integral_constant<int, (u + D) % KU>{});
+#pragma unroll
+            for (int v = 0; v < 2; ++v) {
+                uint4 w0[2], w1[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    cvt_i8x4<DT>(wt[h][v].x, w0[h].x, w0[h].y);
+                    cvt_i8x4<DT>(wt[h][v].y, w0[h].z, w0[h].w);
+                    cvt_i8x4<DT>(wt[h][v].z, w1[h].x, w1[h].y);
+                    cvt_i8x4<DT>(wt[h][v].w, w1[h].z, w1[h].w);
+                }
+                const char *xs0 = smem + (((u * 4 + v * 2) * MT) * 64 + lane) * 16;
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const uint4 x0 = *reinterpret_cast<const uint4 *>(xs0 + t * 1024);
+                    const uint4 x1 = *reinterpret_cast<const uint4 *>(xs0 + (MT + t) * 1024);
+                    acc[0][t] = mfma16<DT>(w0[0], x0, acc[0][t]);
+                    acc[1][t] = mfma16<DT>(w0[1], x0, acc[1][t]);
+                    acc[0][t] = mfma16<DT>(w1[0], x1, acc[0][t]);
+                    acc[1][t] = mfma16<DT>(w1[1], x1, acc[1][t]);
+                }
+            }
+        });
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[h][t][e] *= sc[h][e];
+            store_tile(acc[h], col_begin + (wave + (2 * q + h) * NW) * 16, plane);  // past the last tile: nothing is inside the range
+        }
+    }
 }
 
 // ---- M <= 4: row-streaming kernel --------------------------------------------------------------------
@@ -1160,11 +1433,80 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     else if (p.M <= 32) hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 2, 2, false>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
     else hipLaunchKernelGGL((skinny_w8_split_kernel<DT, 4, 1, false>), grid, dim3(SK_THREADS), 0, s, p, part, cols_per_block);
     TPAMD_HIP(hipGetLastError());
-    const int64_t outputs = static_cast<int64_t>(p.M) * p.N;
-    hipLaunchKernelGGL((skinny_w8_finish_kernel<DT>), dim3(static_cast<unsigned>((outputs + 255) / 256)), dim3(256), 0, s, p, part, splits);
-    TPAMD_HIP(hipGetLastError());
+    if (int rc_f = launch_w8_finish<DT>(p, part, splits, s); rc_f != TPAMD_OK) return rc_f;
     *done = true;
     return TPAMD_OK;
+}
+
+// int8 weights, wavefronts own columns: K a multiple of 16, at most 64 rows and 256 outlier columns, and enough columns
+// that every wavefront of a block gets a tile. *done = false: not taken.
+template <int DT, int MT, bool DIRECT>
+int configure_w8_cols(int dev, size_t lds) {
+    static thread_local int configured_dev = -1;  // per instantiation and host thread
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_w8_cols_kernel<DT, MT, 8, DIRECT>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        configured_dev = dev;
+    }
+    return TPAMD_OK;
+}
+
+template <int DT, int MT>
+int launch_w8_cols_mt(const SkinnyParams &p, int dev, int cus, hipStream_t s, bool *done) {
+    constexpr int KU = 8;
+    const int k_planes = (p.K + KU * WC_UNIT_K - 1) / (KU * WC_UNIT_K);
+    const int planes = k_planes + (p.n_out > 0 ? 1 : 0);
+    if (k_planes > cus) return TPAMD_OK;
+    int col_blocks = cus / k_planes;
+    int cols_per_block = (p.N + col_blocks - 1) / col_blocks;
+    cols_per_block = (cols_per_block + 16 * WC_NW - 1) / (16 * WC_NW) * (16 * WC_NW);
+    col_blocks = (p.N + cols_per_block - 1) / cols_per_block;
+    const size_t lds = static_cast<size_t>(KU) * 4 * MT * 1024 + WC_NW * WC_STAGE;
+    // the outlier plane is worked on by one block per 8 tiles of a column range (a tile per wavefront)
+    const int outlier_blocks = p.n_out > 0 ? (cols_per_block / 16 + WC_NW - 1) / WC_NW : 0;
+    const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>(k_planes + outlier_blocks));
+    if (planes == 1) {
+        if (int rc = configure_w8_cols<DT, MT, true>(dev, lds); rc != TPAMD_OK) return rc;
+        hipLaunchKernelGGL((skinny_w8_cols_kernel<DT, MT, KU, true>), grid, dim3(WC_NW * 64), lds, s, p, nullptr, cols_per_block, k_planes);
+        TPAMD_HIP(hipGetLastError());
+        *done = true;
+        return TPAMD_OK;
+    }
+    if (int rc = configure_w8_cols<DT, MT, false>(dev, lds); rc != TPAMD_OK) return rc;
+    const size_t need = static_cast<size_t>(planes) * p.M * p.N * sizeof(float);
+    std::lock_guard<std::mutex> hold(splitk_mutex());
+    void *ws = nullptr;
+    const int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
+    if (rc != TPAMD_OK) return rc;
+    if (ws == nullptr) return TPAMD_OK;
+    float *part = static_cast<float *>(ws);
+    hipLaunchKernelGGL((skinny_w8_cols_kernel<DT, MT, KU, false>), grid, dim3(WC_NW * 64), lds, s, p, part, cols_per_block, k_planes);
+    TPAMD_HIP(hipGetLastError());
+    if (int rc_f = launch_w8_finish<DT>(p, part, planes, s); rc_f != TPAMD_OK) return rc_f;
+    *done = true;
+    return TPAMD_OK;
+}
+
+template <int DT>
+int launch_w8_cols(const SkinnyParams &p, hipStream_t s, bool *done) {
+    *done = false;
+    if (tuning().w8_cols == 0) return TPAMD_OK;
+    if (p.M > 64 || p.K % 16 != 0 || p.n_out > 256) return TPAMD_OK;
+    if (tuning().w8_cols == TUNE_UNSET) {
+        if (tuning().w8_split != TUNE_UNSET) return TPAMD_OK;  // an explicit choice between the two older kernels
+        // Measured on the Falcon-40B MLP shard (16384 x 8192 and 8192 x 16384, inside a HIP graph, finishing pass included)
+        // against the two older kernels, rows 4 / 8 / 16 / 32 / 64: 30.3 + 34.6 / 34.1 + 37.0 / 37.8 + 40.1 / 46.9 + 50.1 /
+        // 71.5 + 73.9 us -> 29.5 + 30.6 / 31.0 + 31.7 / 34.0 + 34.5 / 39.6 + 39.1 / 54.4 + 52.9 us. Small matrices, where a
+        // block's column range has fewer tiles than wavefronts, stay with the older kernels.
+        if (p.M < 4 || p.K < 4096 || static_cast<int64_t>(p.N) * p.K < (1ll << 25)) return TPAMD_OK;
+    }
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+    if (p.M <= 16) return launch_w8_cols_mt<DT, 1>(p, dev, cus, s, done);
+    if (p.M <= 32) return launch_w8_cols_mt<DT, 2>(p, dev, cus, s, done);
+    if (p.M <= 48) return launch_w8_cols_mt<DT, 3>(p, dev, cus, s, done);
+    return launch_w8_cols_mt<DT, 4>(p, dev, cus, s, done);
 }
 
 // ---- gated pair, 4 <= M <= 16: x through LDS in MFMA operand order, chunk by chunk ------------------------------------
@@ -1353,7 +1695,9 @@ template <int DT, bool W8, int MODE>
 int launch_skinny(const SkinnyParams &p, hipStream_t s) {
     if constexpr (W8) {
         bool done = false;
-        const int rc = launch_w8_split<DT>(p, s, &done);
+        int rc = launch_w8_cols<DT>(p, s, &done);
+        if (rc != TPAMD_OK || done) return rc;
+        rc = launch_w8_split<DT>(p, s, &done);
         if (rc != TPAMD_OK || done) return rc;
     }
     if constexpr (!W8) {

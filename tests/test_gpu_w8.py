@@ -72,10 +72,10 @@ def test_falcon_mlp_shard_full_shape():
     torch.testing.assert_close(down.double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * scale_y)
 
 
-@pytest.mark.parametrize("M", [1, 16, 32, 64])
+@pytest.mark.parametrize("M", [1, 4, 16, 32, 64])
 def test_falcon_mlp_shard_full_shape_every_decode_batch(M):
     """BASELINE config 5 at its real shape through the DEFAULT dispatch at batch 1, 16, 32 and 64 (the row-streaming
-    kernel at 1, the K-split kernel from 12 rows on at this size): both matrices against the closed-form definition in
+    kernel at 1, the K-split kernel whose wavefronts own columns from 4 rows on at this size): both matrices against the closed-form definition in
     float64. The down projection is fed the device's own hidden activations."""
     d, f = 8192, 16384
     x, wq1, s1, c1, o1 = make_case(M, f, d, 41, torch.float16, 0)
@@ -142,7 +142,7 @@ def test_16bit_decode_kernels_column_groups(dtype, M, cg, column_groups):
 @pytest.mark.parametrize("N,K,n_out", [(64, 4096, 0), (200, 4128, 5), (1000, 8192, 41), (528, 6144, 33), (48, 16384, 256)])
 def test_k_split_kernel(dtype, M, N, K, n_out, tune):
     """The int8 kernel that splits K over blocks and keeps its x fragments in registers (forced; by default it
-    serves 12 or more rows on large matrices): 1, 2 and 4 row tiles, a single split and several, a last split that
+    serves 12 or more rows on matrices the column-owning kernel does not take): 1, 2 and 4 row tiles, a single split and several, a last split that
     is partly or wholly past the end of K, column ranges whose last tile is masked, outlier columns on wavefronts
     0 to 7 of split 0, more than 64 rows (slabs), bias and GELU. Same products as the unsplit kernel in another
     order: both are compared with the definition, and with each other."""
@@ -162,10 +162,38 @@ def test_k_split_kernel(dtype, M, N, K, n_out, tune):
     torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * sigma)
 
 
-def test_k_split_kernel_inside_a_hip_graph(tune):
-    """The K-split int8 kernel and its finishing pass (two launches sharing the library's scratch buffer) recorded
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 9, 16, 17, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("N,K,n_out", [(64, 4096, 0), (200, 4128, 5), (1000, 8192, 41), (528, 6144, 33), (48, 16384, 256),
+                                       (256, 1024, 0), (2068, 1040, 7)])
+def test_k_split_kernel_whose_wavefronts_own_columns(dtype, M, N, K, n_out, tune):
+    """The int8 kernel that keeps the x rows of its K split in LDS and gives every wavefront whole 16-row weight tiles
+    (forced; by default it serves 4 or more rows on large matrices): 1 to 4 row tiles of x, one K plane (results
+    stored directly) and several, a last plane that is partly past the end of K, column ranges with fewer tiles than
+    wavefronts and with a ragged last tile, N not a multiple of 4, the outlier plane with 1 to 8 groups of 32
+    columns, bias and GELU. Compared with the definition, and with the unsplit kernel."""
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, dtype, seed=4)
+    args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+            torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None,
+            torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(5)) * 0.1).to(dtype).to(DEV)
+    tune("TPAMD_W8_COLS", "1")
+    got = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
+    tune("TPAMD_W8_COLS", "0")
+    tune("TPAMD_W8_SPLIT", "0")
+    plain = _native.linear_w8(*args, bias=bias, act=_native.ACT_GELU)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out) + bias.double().cpu().numpy()
+    want = 0.5 * want * (1.0 + np.vectorize(math.erf)(want / math.sqrt(2.0)))
+    sigma = 0.02 * math.sqrt(K + 400 * n_out)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
+    torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * sigma)
+
+
+@pytest.mark.parametrize("knob", ["TPAMD_W8_SPLIT", "TPAMD_W8_COLS"])
+def test_k_split_kernel_inside_a_hip_graph(knob, tune):
+    """Either K-split int8 kernel and its finishing pass (two launches sharing the library's scratch buffer) recorded
     into a HIP graph after a warm-up call: every replay gives the eager result, with eager work in between."""
-    tune("TPAMD_W8_SPLIT", "1")
+    tune(knob, "1")
     M, N, K, n_out = 32, 200, 8192, 41
     x, wq, scale, cols, w_out = make_case(M, N, K, n_out, torch.float16, seed=6)
     args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
