@@ -63,10 +63,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, lq = lane >> 4;
-    const int bh = blockIdx.y, b = bh / p.Hkv, hkv = bh % p.Hkv;
     const int nrows = p.G * p.Sq;
-    // causal: blocks with the highest positions have the longest key ranges; they are launched first
-    const int row_tile = p.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+    // Causal: a block's key range grows with the positions of its rows, and blocks are handed to the 8 XCDs in turn, so
+    // the order must not let block lengths repeat with a period that divides 8 (position tiles within a head do:
+    // one XCD would get every longest block and the kernel would take as long as without the mask). The (batch, kv head)
+    // index runs fastest, so equally long blocks are neighbours and spread over the XCDs; the row tiles follow with the
+    // longest first: all heads' last position tile, then the one before, ... when heads are whole numbers of
+    // tiles, else simply the row tiles from the last to the first.
+    int bh = blockIdx.y, row_tile = blockIdx.x;
+    if (p.causal) {
+        const int lin = blockIdx.x + gridDim.x * blockIdx.y;
+        bh = lin % gridDim.y;
+        const int slow = lin / gridDim.y;  // 0 ... gridDim.x - 1
+        const int pt_per_head = p.Sq / ROWS;
+        if (pt_per_head > 0 && p.Sq % ROWS == 0) row_tile = (slow % p.G) * pt_per_head + pt_per_head - 1 - slow / p.G;
+        else row_tile = gridDim.x - 1 - slow;
+    }
+    const int b = bh / p.Hkv, hkv = bh % p.Hkv;
     const int row0 = row_tile * ROWS;
     const int shift = p.Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
 
