@@ -72,7 +72,7 @@ struct Entry {
     size_t bytes;
 };
 std::vector<Entry> g_cache;  // guarded by splitk_mutex()
-constexpr int MAX_BUFFERS_PER_DEVICE = 8;
+constexpr int MAX_BUFFERS_PER_DEVICE = 33;  // 32 streams (a framework's stream pool) and the spare
 
 }  // namespace
 
@@ -88,7 +88,7 @@ std::mutex &splitk_mutex() {
 // it. Allocating is not allowed while a stream is being captured, so the first allocation on a device also sets one
 // spare buffer aside, and the first capturing stream that has no buffer of its own takes it over (frameworks capture
 // on a stream of their own that runs nothing else). NULL comes back when a capturing stream finds no spare, when `need`
-// is larger than the stream's buffer, and for the ninth buffer of a device.
+// is larger than the stream's buffer, and when the device already has its 33 buffers (32 streams and the spare).
 // Inside a StaticScratchScope (noalloc.hip) the library's fixed array is handed out instead.
 static int allocate_entry(int dev, hipStream_t stream, bool spare, size_t bytes, void **out) {
     void *ptr = nullptr;
