@@ -178,7 +178,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(SkinnyParams p) {
         for (int t = 0; t < MT; ++t) acc[a][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int nchunks = (p.K + CHUNK_K - 1) / CHUNK_K;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
 
     // Register double buffers for the weights (and for x when it is small enough). Buffer indices are
     // compile-time constants so that the arrays stay in registers.
@@ -193,10 +192,11 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(SkinnyParams p) {
 #pragma unroll
             for (int i = 0; i < WV; ++i) {
                 const int byte = (i >> 1) * 128 + cpiece * 16;            // inside the chunk's 256 bytes of the row
+                // Past the end of K the row's first bytes are fetched instead (always a load, never a branch, and nothing
+                // is done to the value until it is multiplied): x is zero there, so the product is too.
                 const bool ok = c * CHUNK_K + byte / wbytes < p.K;
                 const char *base = (a % NMAT == 0 ? wp[i & 1] : wp2[i & 1]) + (a / NMAT) * cg_stride;
-                const uint4 raw = nt_load_u4(ok ? base + off + (i >> 1) * 128 : base - cpiece * 16);  // unconditional
-                wv[buf][a][i] = ok ? raw : zero4;
+                wv[buf][a][i] = nt_load_u4(ok ? base + off + (i >> 1) * 128 : base - cpiece * 16);
             }
     };
     // registers in fetch order -> registers in MFMA operand order, through this wavefront's LDS tile
@@ -238,16 +238,25 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(SkinnyParams p) {
             for (int i = 0; i < XV; ++i) {
                 const int byte = (i >> 1) * 128 + cpiece * 16;
                 const bool ok = xokc[t][i & 1] && c * CHUNK_K + byte / 2 < p.K;
-                xv[buf][t][i] = ok ? *reinterpret_cast<const uint4 *>(xpc[t][i & 1] + xoff + (i >> 1) * 128) : zero4;
+                // requested unconditionally (the first bytes of x when out of range) and zeroed in compute(): a branch
+                // around a load, or a use right behind it, makes every later wait drain all loads
+                xv[buf][t][i] = *reinterpret_cast<const uint4 *>(ok ? xpc[t][i & 1] + xoff + (i >> 1) * 128 : p.x);
             }
     };
-    auto compute = [&](auto bufc) {
+    auto compute = [&](auto bufc, int c) {
         constexpr int buf = decltype(bufc)::value;
         constexpr int xb = XPRE ? buf : 0;
 #pragma unroll
         for (int a = 0; a < NA; ++a) transpose_w(wv[PRE ? buf : 0][a]);
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
+#pragma unroll
+            for (int i = 0; i < XV; ++i) {
+                const int byte = (i >> 1) * 128 + cpiece * 16;
+                const bool ok = xokc[t][i & 1] && c * CHUNK_K + byte / 2 < p.K;
+                const uint4 v = xv[xb][t][i];
+                xv[xb][t][i] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+            }
             transpose(&xv[xb][t][0]);
             if constexpr (W8) transpose(&xv[xb][t][4]);  // second 256 bytes of the row's chunk
         }
@@ -283,36 +292,33 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(SkinnyParams p) {
     // This wavefront's chunks are wave, wave + SK_WAVES, ... The next chunk's loads are issued before the
     // current one is multiplied. Loads return in order, so whatever the multiply waits for is issued
     // ahead of the prefetch.
+    // A prefetch past the wavefront's last chunk is a chunk past the end of K (loads of the rows' first bytes): every
+    // pass through the loop issues the same loads, so each wait counts exactly the loads behind the one it needs.
+    auto in_k = [&](int c) { return c < nchunks ? c : nchunks; };
     if constexpr (PRE) {
         int c = wave;
-        if (c < nchunks) {
-            load_w(B0{}, c);
-            if constexpr (XPRE) load_x(B0{}, c);
-        }
+        load_w(B0{}, in_k(c));
+        if constexpr (XPRE) load_x(B0{}, in_k(c));
         while (c < nchunks) {
             int cn = c + NW;
             if constexpr (!XPRE) load_x(B0{}, c);
-            if (cn < nchunks) {
-                load_w(B1{}, cn);
-                if constexpr (XPRE) load_x(B1{}, cn);
-            }
-            compute(B0{});
+            load_w(B1{}, in_k(cn));
+            if constexpr (XPRE) load_x(B1{}, in_k(cn));
+            compute(B0{}, c);
             c = cn;
             if (c >= nchunks) break;
             cn = c + NW;
             if constexpr (!XPRE) load_x(B0{}, c);
-            if (cn < nchunks) {
-                load_w(B0{}, cn);
-                if constexpr (XPRE) load_x(B0{}, cn);
-            }
-            compute(B1{});
+            load_w(B0{}, in_k(cn));
+            if constexpr (XPRE) load_x(B0{}, in_k(cn));
+            compute(B1{}, c);
             c = cn;
         }
     } else {
         for (int c = wave; c < nchunks; c += NW) {
             load_w(B0{}, c);
             load_x(B0{}, c);
-            compute(B0{});
+            compute(B0{}, c);
         }
     }
 
@@ -443,7 +449,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
     const int st_wr = crow * TROW + cpiece * 16;   // + (i&1)*8*TROW + (i/2)*128
     const int st_rd = lr * TROW + lg * 16;         // + v*64
     const int nchunks = (p.K + CHUNK_K - 1) / CHUNK_K;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
     const int col_begin = static_cast<int>(static_cast<int64_t>(blockIdx.x) * p.N / gridDim.x);
     const int col_end = static_cast<int>(static_cast<int64_t>(blockIdx.x + 1) * p.N / gridDim.x);
 
@@ -470,9 +475,22 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
             const int m = crow + 8 * (i & 1);
             const int byte = (i >> 1) * 128 + cpiece * 16;
             const bool ok = c < nchunks && m < p.M && c * CHUNK_K + byte / 2 < p.K;
-            xq[j][i] = ok ? *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte) : zero4;
+            // requested unconditionally (the first bytes of x when out of range) and zeroed where the value is used:
+            // a branch around a load, or a use right behind it, makes every later wait drain all loads
+            xq[j][i] = *reinterpret_cast<const uint4 *>(p.x + (ok ? static_cast<int64_t>(m) * p.ldx * 2 + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte : 0));
         }
     }
+    auto zero_x_out_of_range = [&](int j) __attribute__((always_inline)) {
+        const int c = wave + j * NW;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = crow + 8 * (i & 1);
+            const int byte = (i >> 1) * 128 + cpiece * 16;
+            const bool ok = c < nchunks && m < p.M && c * CHUNK_K + byte / 2 < p.K;
+            const uint4 v = xq[j][i];
+            xq[j][i] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+        }
+    };
 
     uint4 wv[DEPTH][4];
     // chunk j of the tile whose first column is n0 (columns from n_valid on do not belong to this block)
@@ -485,16 +503,21 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
             const int col = PAIR ? crow : crow + 8 * h;              // column of the tile this row belongs to
             const char *base = (PAIR && h == 1 ? p.w2 : p.w) + static_cast<int64_t>(n0 + col) * p.ldw * 2;
             const int byte = (i >> 1) * 128 + cpiece * 16;
+            // Out of range (a chunk past K, a column of another block, no further tile): the first bytes of the matrix,
+            // requested all the same. x is zero past K, and the sums of such columns are never stored.
             const bool ok = c < nchunks && col < n_valid && c * CHUNK_K + byte / 2 < p.K;
-            wv[j % DEPTH][i] = ok ? nt_load_u4(base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte) : zero4;
+            wv[j % DEPTH][i] = nt_load_u4(ok ? base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte : p.w);
         }
     };
     auto for_each_chunk = [&](auto &&f) { static_for<NCH>(f); };
 
     int n0 = col_begin;
-    if (n0 < col_end) static_for<DEPTH>([&](auto jc) { load_w(jc, n0, col_end - n0); });
+    static_for<DEPTH>([&](auto jc) { load_w(jc, n0, col_end - n0); });
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) transpose(xq[j]);
+    for (int j = 0; j < NCH; ++j) {
+        zero_x_out_of_range(j);
+        transpose(xq[j]);
+    }
 
     for (int t = 0; n0 < col_end; ++t, n0 += COLS) {
         const int n_valid = col_end - n0 < COLS ? col_end - n0 : COLS;
@@ -508,7 +531,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
 #pragma unroll
             for (int v = 0; v < 4; ++v) acc = mfma16<DT>(wv[j % DEPTH][v], xq[j][v], acc);
             if constexpr (j + DEPTH < NCH) load_w(std::integral_constant<int, j + DEPTH>{}, n0, n_valid);
-            else if (n_next < col_end) load_w(std::integral_constant<int, j + DEPTH - NCH>{}, n_next, col_end - n_next);
+            else load_w(std::integral_constant<int, j + DEPTH - NCH>{}, n_next, col_end - n_next);  // no further tile: n_valid <= 0
         });
         float(*rd)[4][64] = red[t & 1];
 #pragma unroll
@@ -1346,27 +1369,34 @@ inline bool pick_pair(const SkinnyParams &p) {
     return p.M <= 32;
 }
 
-// The x-resident kernel pays when x is large enough to matter and a CU would otherwise re-read it for several weight
-// tiles. Measured on Llama-7B-sized shapes: gated pair from 9 rows and 1.25 tiles per CU on (5504 columns, K = 4096,
-// 16 rows: 31 -> 22 us; 11008 columns, K = 5504: 74 -> 49 us), single matrix from 12 rows and 1.5 tiles per CU or 14
-// rows and one tile per CU on (4096 columns at 16 rows: K = 4096 14 -> 11.5 us, K = 5504 17 -> 16 us: all of x is
-// requested up front instead of chunk by chunk); with fewer rows, or K = 2048, the plain kernel, with more blocks per
-// CU, is as fast or faster. 16-bit weights, at most 16 rows, K up to 8192 (the x fragments have to fit the registers).
+// The x-resident kernel against the plain one (more blocks per CU, x re-read per tile) and, for the gated pair, the one
+// that stages x in LDS. Measured inside a HIP graph at 4 / 8 / 12 / 16 rows (us; plain | resident | x in LDS):
+//   pair 5504 x 4096:   18.9 19.7 20.5 20.5 | 17.9 17.9 18.0 17.8 | 19.1 19.5 20.2 20.2
+//   pair 11008 x 5504:  45.6 46.3 48.9 51.6 | 42.1 40.9 41.0 41.6 | 48.4 47.4 48.2 49.0
+//   pair 2752 x 4096:   12.5 13.0 13.5 14.3 | 11.6 11.7 11.7 11.8 | 13.1 13.3 13.8 14.3
+//   pair 1376 x 8192:   11.8 12.7 13.7 14.6 | 11.9 11.9 12.1 12.1 | 15.1 15.6 16.6 17.9
+//   pair 16384 x 8192:  85.1 84.9 88.2 93.2 | 93.1 92.4 94.8 95.4 | 86.7 86.6 86.8 87.8
+//   pair 4096 x 2048:    9.2  9.3  9.7 10.0 | 10.5 10.5 10.4 10.6 |  9.5  9.6  9.9 10.2
+//   4096 x 5504:        10.6 11.0 11.3 11.7 | 11.7 12.0 12.1 12.6       (one tile per CU: the plain kernel)
+//   11008 x 4096:       18.1 18.7 23.1 23.7 | 19.1 19.3 19.4 19.8       (2.7 tiles per CU)
+//   32000 x 4096:       43.9 45.1 48.4 49.0 | 44.6 44.8 43.7 44.0
+//   4608 x 8192:        20.7 21.1 21.8 22.7 | 18.4 18.5 18.9 18.8       (1.125 tiles per CU: the plain kernel's blocks fill
+//   8192 x 8192:        25.7 26.0 32.7 32.8 | 30.7 30.5 30.0 30.7        the CUs unevenly)
+//   16384 x 8192:       47.1 47.4 47.8 47.6 | 48.7 49.5 48.9 49.1
+// 16-bit weights, 4 to 16 rows, K from 3072 to 8192 (the x fragments have to fit the registers: 4 chunks per wavefront
+// and 4 register slots for the weights up to K = 4096, 6 and 3 up to 6144, 8 and 2 up to 8192).
 template <int MODE>
 inline bool pick_resident(const SkinnyParams &p, int cus) {
     if (p.M > 16 || p.K > 8192) return false;
     if (tuning().skinny_resident != TUNE_UNSET) return tuning().skinny_resident != 0;
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
-    if (p.K < 3072) return false;
-    if (p.K > 6144) {
-        // 8 chunks per wavefront leave 2 register slots for the weights: gated pair from 12 rows on (16384 columns,
-        // K = 8192, 16 rows: 144 -> 96 us), single matrix only where the plain kernel's blocks do not fill the CUs
-        // evenly (4608 columns = 1.125 tiles per CU, 16 rows: 38 -> 33 us; at 2 tiles per CU it loses)
-        if (MODE == SK_SWIGLU) return p.M >= 12 && tiles * 4 >= 5ll * cus;
-        return p.M >= 14 && tiles >= cus && tiles * 2 < 3ll * cus;
+    if (p.M < 3 || p.K < 3072) return false;
+    if (MODE == SK_SWIGLU) {
+        if (p.K <= 6144) return tiles * 2 >= cus;
+        return p.M >= 8 && tiles < cus;
     }
-    if (MODE == SK_SWIGLU) return p.M >= 9 && tiles * 4 >= 5ll * cus;
-    return (p.M >= 12 && tiles * 2 >= 3ll * cus) || (p.M >= 14 && tiles >= cus);
+    if (p.K <= 6144) return p.M >= 12 && tiles * 2 >= 3ll * cus;
+    return (tiles >= cus && tiles * 2 < 3ll * cus) || (p.M >= 10 && tiles >= cus && tiles * 2 <= 5ll * cus);
 }
 
 template <int DT, int MODE>
@@ -1498,7 +1528,7 @@ int launch_w8_cols(const SkinnyParams &p, hipStream_t s, bool *done) {
         // against the two older kernels, rows 4 / 8 / 16 / 32 / 64: 30.3 + 34.6 / 34.1 + 37.0 / 37.8 + 40.1 / 46.9 + 50.1 /
         // 71.5 + 73.9 us -> 29.5 + 30.6 / 31.0 + 31.7 / 34.0 + 34.5 / 39.6 + 39.1 / 54.4 + 52.9 us. Small matrices, where a
         // block's column range has fewer tiles than wavefronts, stay with the older kernels.
-        if (p.M < 4 || p.K < 4096 || static_cast<int64_t>(p.N) * p.K < (1ll << 25)) return TPAMD_OK;
+        if (p.M < 2 || p.K < 4096 || static_cast<int64_t>(p.N) * p.K < (1ll << 25)) return TPAMD_OK;
     }
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
@@ -1705,11 +1735,18 @@ int launch_skinny(const SkinnyParams &p, hipStream_t s) {
         TPAMD_HIP(hipGetDevice(&dev));
         if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
         if constexpr (MODE == SK_SWIGLU) {
+            if (tuning().skinny_xlds == 1) {  // asked for by name: before the x-resident kernel
+                bool done = false;
+                const int rc = launch_pair_xlds<DT>(p, cus, s, &done);
+                if (rc != TPAMD_OK || done) return rc;
+            }
+        }
+        if (pick_resident<MODE>(p, cus)) return launch_resident<DT, MODE>(p, cus, s);
+        if constexpr (MODE == SK_SWIGLU) {
             bool done = false;
             const int rc = launch_pair_xlds<DT>(p, cus, s, &done);
             if (rc != TPAMD_OK || done) return rc;
         }
-        if (pick_resident<MODE>(p, cus)) return launch_resident<DT, MODE>(p, cus, s);
     }
     if constexpr (MODE == SK_SWIGLU && !W8) {
         if (p.M <= 32 && pick_pair(p)) {
@@ -1782,7 +1819,15 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ld_wout = ld_wout;
     p.act = act;
     const bool bf = dtype == TPAMD_BF16;
-    if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
+    // 3 rows of a large matrix are faster through the MFMA kernels (Llama-7B MLP shard step: 36.4 us here, 28.3 us there,
+    // as at 4 rows), and so are 2 and 3 rows of int8 weights through the K-split kernel where it applies
+    if (w8 && M >= 2 && M <= GEMV_MAX_M) {
+        bool done = false;
+        const int rc = bf ? launch_w8_cols<TPAMD_BF16>(p, s, &done) : launch_w8_cols<TPAMD_F16>(p, s, &done);
+        if (rc != TPAMD_OK || done) return rc;
+    }
+    const bool rows3_to_mfma = !w8 && M == 3 && K >= 3072 && K <= 8192;
+    if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES && !rows3_to_mfma) {
         bool done = false;
         const int rc = w8 ? (bf ? launch_gemv_rows<TPAMD_BF16, true, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, true, SK_LINEAR>(p, s, &done))
                      : swiglu ? (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_SWIGLU>(p, s, &done) : launch_gemv_rows<TPAMD_F16, false, SK_SWIGLU>(p, s, &done))
