@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(head[r]) * p.q_sh + static_cast<int64_t>(sq[r]) * p.q_ss) * 2;
 #pragma unroll
         for (int kk = 0; kk < DK; ++kk)
-            qf[r][kk] = row_ok[r] ? *reinterpret_cast<const uint4 *>(qrow + (32 * kk + 8 * lq) * 2) : make_uint4(0, 0, 0, 0);
+            qf[r][kk] = *reinterpret_cast<const uint4 *>(qrow + (32 * kk + 8 * lq) * 2);  // rows past the end: row 0 of the group, never stored
     }
 
     // ---- key range of this block

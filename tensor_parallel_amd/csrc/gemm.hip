@@ -194,17 +194,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
     auto load_global = [&](int kt) {
         const int k = kt * BK + ld_chunk * 8;
         const bool ok = k < p.K;  // K is a multiple of 8: a chunk is entirely inside or outside
-        const int64_t off = static_cast<int64_t>(kt) * BK * 2;
+        // Past the end of K the row's first chunk is fetched instead: a load, not a branch around one (which would turn
+        // into a branch per dword). store_lds() writes zeros for x there, so whatever w holds is multiplied by zero.
+        const int64_t off = ok ? static_cast<int64_t>(kt) * BK * 2 : -static_cast<int64_t>(ld_chunk) * 16;
 #pragma unroll
-        for (int i = 0; i < XC; ++i) xr[i] = ok ? *reinterpret_cast<const uint4 *>(xg[i] + off) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < XC; ++i) xr[i] = *reinterpret_cast<const uint4 *>(xg[i] + off);
 #pragma unroll
-        for (int i = 0; i < WC; ++i) wr[i] = ok ? *reinterpret_cast<const uint4 *>(wg[i] + off) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < WC; ++i) wr[i] = *reinterpret_cast<const uint4 *>(wg[i] + off);
     };
-    auto store_lds = [&](int stage) {
+    auto store_lds = [&](int stage, int kt) {
         char *xs = smem + stage * STAGE;
         char *ws = xs + BM * LDS_ROW;
+        const bool ok = kt * BK + ld_chunk * 8 < p.K;
 #pragma unroll
-        for (int i = 0; i < XC; ++i) *reinterpret_cast<uint4 *>(xs + st_off + i * (NT / 8) * LDS_ROW) = xr[i];
+        for (int i = 0; i < XC; ++i)
+            *reinterpret_cast<uint4 *>(xs + st_off + i * (NT / 8) * LDS_ROW) = make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
 #pragma unroll
         for (int i = 0; i < WC; ++i) *reinterpret_cast<uint4 *>(ws + st_off + i * (NT / 8) * LDS_ROW) = wr[i];
     };
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 
     const int KT = (p.K + BK - 1) / BK;
     load_global(0);
-    store_lds(0);
+    store_lds(0, 0);
     __syncthreads();
 
     for (int kt = 0; kt < KT; ++kt) {
@@ -252,7 +256,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 #pragma unroll
                 for (int b = 0; b < TN; ++b) acc[a][b] = mfma32<DT>(wf[b], xf[a], acc[a][b]);
         }
-        if (more) store_lds((kt + 1) & 1);
+        if (more) store_lds((kt + 1) & 1, kt + 1);
         __syncthreads();
     }
 

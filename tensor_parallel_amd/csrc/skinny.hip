@@ -611,7 +611,8 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParam
                 const int byte = (i >> 1) * 128 + cpiece * 16;
                 const int64_t k0 = chunk_k0(j);
                 const bool ok = m < p.M && k0 + byte / 2 < p.K;
-                xq[j][t][i] = ok ? *reinterpret_cast<const uint4 *>(p.x + static_cast<int64_t>(m) * p.ldx * 2 + k0 * 2 + byte) : zero4;
+                // always a load (the first bytes of x when out of range), zeroed below where it is first used
+                xq[j][t][i] = *reinterpret_cast<const uint4 *>(p.x + (ok ? static_cast<int64_t>(m) * p.ldx * 2 + k0 * 2 + byte : 0));
             }
 #pragma unroll
     for (int j = 0; j < NCH; ++j)
@@ -619,6 +620,14 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParam
         for (int t = 0; t < MT; ++t)
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int i = half * 4; i < half * 4 + 4; ++i) {
+                    const int m = t * 16 + crow + 8 * (i & 1);
+                    const int byte = (i >> 1) * 128 + cpiece * 16;
+                    const bool ok = m < p.M && chunk_k0(j) + byte / 2 < p.K;
+                    const uint4 v = xq[j][t][i];
+                    xq[j][t][i] = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+                }
                 stage_in(&xq[j][t][half * 4]);
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
@@ -654,11 +663,12 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParam
         for (int i = 0; i < 4; ++i) {
             const int row = n0 + crow + 8 * (i & 1);
             const int byte = (i >> 1) * 128 + cpiece * 16;
+            // rows of another block and bytes past K: the first bytes of the matrix (x is zero past K, such rows are not stored)
             const bool ok = row < col_end && k0 + byte < p.K;
-            wv[j][i] = ok ? nt_load_u4(p.w + static_cast<int64_t>(row) * p.ldw + k0 + byte) : zero4;
+            wv[j][i] = nt_load_u4(p.w + (ok ? static_cast<int64_t>(row) * p.ldw + k0 + byte : 0));
         }
     };
-    if (col_begin < col_end) static_for<NCH>([&](auto jc) { load_w(jc, col_begin); });
+    static_for<NCH>([&](auto jc) { load_w(jc, col_begin); });
 
     int t_index = 0;
     for (int n0 = col_begin; n0 < col_end; n0 += 16, ++t_index) {
@@ -672,7 +682,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_w8_split_kernel(SkinnyParam
 #pragma unroll
             for (int v = 0; v < 4; ++v) wt[v] = *reinterpret_cast<const uint4 *>(stage + st_rd + v * 64);
             stage_done();
-            if (n0 + 16 < col_end) load_w(jc, n0 + 16);
+            load_w(jc, n0 + 16);  // past the last tile: every row is out of range
 #pragma unroll
             for (int v = 0; v < 4; ++v) {  // 16 int8 -> two operands of 8
                 uint4 w0, w1;
