@@ -23,7 +23,7 @@ PEAK_HBM_GBS = 8000.0
 # Fabric bytes per launch of the fused gate/up GEMM at M = 4096, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
 # each scaled by what the same counter reads for the slicing kernel's known 13.476 GB (factors 1.98 and 1.00):
 # profiles/pmc_fetch_write_bench_kernels.txt. A counter reading cannot be taken inside this script.
-MEASURED_TRAFFIC_BYTES_M4096 = 628.8e6
+MEASURED_TRAFFIC_BYTES_M4096 = 629.1e6
 
 
 def cpu_baseline(seconds_budget: float = 15.0) -> dict:
