@@ -501,12 +501,15 @@ __global__ __launch_bounds__(NW * 64) void skinny_resident_kernel(SkinnyParams p
         for (int i = 0; i < 4; ++i) {
             const int h = i & 1;
             const int col = PAIR ? crow : crow + 8 * h;              // column of the tile this row belongs to
-            const char *base = (PAIR && h == 1 ? p.w2 : p.w) + static_cast<int64_t>(n0 + col) * p.ldw * 2;
+            // Out of range, a load all the same: a column of another block reads the tile's first row again and one past the
+            // last tile the matrix's last row (cached; such sums are never stored), a chunk past K reads its own row's first
+            // bytes (x is zero there, so what a column adds up never depends on another row's weights).
+            int row = col < n_valid ? n0 + col : n0;
+            row = row < p.N ? row : p.N - 1;
+            const char *base = (PAIR && h == 1 ? p.w2 : p.w) + static_cast<int64_t>(row) * p.ldw * 2;
             const int byte = (i >> 1) * 128 + cpiece * 16;
-            // Out of range (a chunk past K, a column of another block, no further tile): the first bytes of the matrix,
-            // requested all the same. x is zero past K, and the sums of such columns are never stored.
-            const bool ok = c < nchunks && col < n_valid && c * CHUNK_K + byte / 2 < p.K;
-            wv[j % DEPTH][i] = nt_load_u4(ok ? base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte : p.w);
+            const bool in_k = c < nchunks && c * CHUNK_K + byte / 2 < p.K;
+            wv[j % DEPTH][i] = nt_load_u4(in_k ? base + static_cast<int64_t>(c) * (CHUNK_K * 2) + byte : base);
         }
     };
     auto for_each_chunk = [&](auto &&f) { static_for<NCH>(f); };
