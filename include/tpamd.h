@@ -15,7 +15,7 @@
  *   - every entry point may be called concurrently from several host threads. Besides the thread-local error
  *     message the library keeps one piece of state: tpamd_linear / tpamd_linear_add / tpamd_swiglu_up split K for
  *     shapes with few output tiles (M from 17 to a few thousand, decided by a cost model), tpamd_linear_w8 does so
- *     from 4 rows on large matrices, tpamd_attention splits long key ranges, and they keep fp32 scratch buffers for
+ *     from 2 rows on large matrices, tpamd_attention splits long key ranges, and they keep fp32 scratch buffers for
  *     the partial results: one per (device, stream), 64 MiB on a 256-CU part, allocated with hipMalloc at the
  *     stream's first such call and kept until the process ends (at most 32 streams per device get one; calls on
  *     further streams run unsplit). Streams never share a buffer, so such calls on different streams of a device

@@ -1160,7 +1160,7 @@ __global__ __launch_bounds__(GV_WAVES * 64) void gemv_kernel(SkinnyParams p) {
     }
 }
 
-constexpr int GEMV_MAX_M = 3;  // from 4 rows on the MFMA kernel is faster
+constexpr int GEMV_MAX_M = 3;  // the row kernels take at most 3 rows (large matrices go to the MFMA kernels from 3 rows on, see skinny_dispatch)
 constexpr int64_t GEMV_MAX_X_BYTES = 64 * 1024;  // x[M][K] lives in LDS
 
 template <int DT, bool W8, int MODE>

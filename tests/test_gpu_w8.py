@@ -72,10 +72,10 @@ def test_falcon_mlp_shard_full_shape():
     torch.testing.assert_close(down.double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * scale_y)
 
 
-@pytest.mark.parametrize("M", [1, 4, 16, 32, 64])
+@pytest.mark.parametrize("M", [1, 2, 4, 16, 32, 64])
 def test_falcon_mlp_shard_full_shape_every_decode_batch(M):
     """BASELINE config 5 at its real shape through the DEFAULT dispatch at batch 1, 16, 32 and 64 (the row-streaming
-    kernel at 1, the K-split kernel whose wavefronts own columns from 4 rows on at this size): both matrices against the closed-form definition in
+    kernel at 1, the K-split kernel whose wavefronts own columns from 2 rows on at this size): both matrices against the closed-form definition in
     float64. The down projection is fed the device's own hidden activations."""
     d, f = 8192, 16384
     x, wq1, s1, c1, o1 = make_case(M, f, d, 41, torch.float16, 0)
@@ -168,7 +168,7 @@ def test_k_split_kernel(dtype, M, N, K, n_out, tune):
                                        (256, 1024, 0), (2068, 1040, 7)])
 def test_k_split_kernel_whose_wavefronts_own_columns(dtype, M, N, K, n_out, tune):
     """The int8 kernel that keeps the x rows of its K split in LDS and gives every wavefront whole 16-row weight tiles
-    (forced; by default it serves 4 or more rows on large matrices): 1 to 4 row tiles of x, one K plane (results
+    (forced; by default it serves 2 or more rows on large matrices): 1 to 4 row tiles of x, one K plane (results
     stored directly) and several, a last plane that is partly past the end of K, column ranges with fewer tiles than
     wavefronts and with a ragged last tile, N not a multiple of 4, the outlier plane with 1 to 8 groups of 32
     columns, bias and GELU. Compared with the definition, and with the unsplit kernel."""
