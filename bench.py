@@ -377,7 +377,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     state-dict slicing (every split tensor of a Llama-2-7B-shaped dict, all ranks' shards, W = 2, HBM-bound)."""
     extra = {}
     n_sets = len(sets)
-    for m in (1, 16):
+    for m in (1, 4, 16, 64):
         x = torch.randn(m, D_MODEL, device=dev).to(torch.bfloat16)
 
         def fn(i):
