@@ -292,19 +292,36 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(AttnParams p) {
     const int bh = blockIdx.y;
     if (e >= static_cast<int64_t>(nrows) * per_row) return;
     const int row = static_cast<int>(e / per_row), d4 = static_cast<int>(e % per_row) * 4;
+    // the splits' partials are requested eight at a time (a loop that loads, waits and adds per split costs a memory
+    // round trip per split: 16 splits took 5.9 us)
+    const int64_t split_pitch = static_cast<int64_t>(gridDim.y) * p.rows_pad * (D + 4);
+    const float *pr0 = p.part + (static_cast<int64_t>(bh) * p.rows_pad + row) * (D + 4);
     float M = -INFINITY;
-    for (int s = 0; s < p.nsplit; ++s) {
-        const float *pr = p.part + ((static_cast<int64_t>(s) * gridDim.y + bh) * p.rows_pad + row) * (D + 4);
-        M = fmaxf(M, pr[D]);
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float ms[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ms[j] = pr0[(s0 + j < p.nsplit ? s0 + j : s0) * split_pitch + D];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) M = fmaxf(M, ms[j]);
     }
     const float m_use = M == -INFINITY ? 0.f : M;
     float o[4] = {0.f, 0.f, 0.f, 0.f}, l = 0.f;
-    for (int s = 0; s < p.nsplit; ++s) {
-        const float *pr = p.part + ((static_cast<int64_t>(s) * gridDim.y + bh) * p.rows_pad + row) * (D + 4);
-        const float w = exp2f(pr[D] - m_use);
-        l += w * pr[D + 1];
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float2 ml[8];
+        f32x4 ov[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] += w * pr[d4 + i];
+        for (int j = 0; j < 8; ++j) {
+            const float *pr = pr0 + (s0 + j < p.nsplit ? s0 + j : s0) * split_pitch;
+            ml[j] = *reinterpret_cast<const float2 *>(pr + D);
+            ov[j] = *reinterpret_cast<const f32x4 *>(pr + d4);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float w = s0 + j < p.nsplit ? exp2f(ml[j].x - m_use) : 0.f;
+            l += w * ml[j].y;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] += w * ov[j][i];
+        }
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     const int b = bh / p.Hkv, hkv = bh % p.Hkv, g = row / p.Sq, sq = row % p.Sq;
