@@ -39,6 +39,7 @@ def check(q, k, v, causal, scale=None):
     (1, 2, 1, 70, 70, 64),      # row tiles that straddle heads, ragged
     (1, 4, 2, 130, 130, 128),   # head_dim 128
     (3, 6, 3, 1, 17, 128),      # fewer keys than a tile
+    (2, 8, 2, 256, 256, 64),    # several position tiles per head and several (batch, kv head) pairs: the causal block order
 ])
 def test_attention_matches_oracle(dtype, causal, B, Hq, Hkv, Sq, Skv, D):
     check(*make(B, Hq, Hkv, Sq, Skv, D, dtype), causal)
