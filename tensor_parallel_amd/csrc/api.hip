@@ -27,8 +27,29 @@ int attention_dispatch(const void *q, const void *k, const void *v, void *o, int
 
 namespace {
 
-// Largest M served by the weight-streaming kernel; above it the tiled MFMA kernel takes over.
+// Largest M served by the weight-streaming kernels; above it the tiled MFMA kernels take over.
 constexpr int64_t SKINNY_MAX_M = 16;
+
+// A single 16-bit matrix with few output tiles per CU stays with the weight-streaming kernel for more rows: the tiled
+// kernels split K over blocks there and pay a second launch. Measured inside a HIP graph (us, tiled | streaming) at
+// 17 / 32 / 48 / 64 rows: 2048 x 4096 13.4 14.1 14.7 15.0 | 9.3 10.3 12.8 13.4; 4096 x 4096 14.5 14.8 15.4 15.9 | 10.8 12.1 14.8 15.7;
+// 4096 x 5504 16.7 17.4 17.8 18.5 | 13.7 15.1 17.9 19.7; 11008 x 4096 24.6 25.4 25.3 26.5 | 26.5 29.0 36.2 39.0. (The gated
+// pair is faster through the tiled kernels at all of these sizes.)
+int skinny_row_limit(int64_t N, int64_t K, int64_t *rows) {
+    *rows = SKINNY_MAX_M;
+    if (tuning().skinny_max_m != TUNE_UNSET) {
+        *rows = tuning().skinny_max_m < 64 ? tuning().skinny_max_m : 64;
+        return TPAMD_OK;
+    }
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (int rc = device_cus(dev, &cus); rc != TPAMD_OK) return rc;
+    const int64_t tiles = (N + 15) / 16;
+    if (K < 2048 || K > 8192) return TPAMD_OK;
+    if (tiles * 2 <= cus) *rows = 64;
+    else if (tiles <= cus) *rows = 32;
+    return TPAMD_OK;
+}
 constexpr int64_t SKINNY_W8_SLAB = 64;
 
 // What the MFMA kernels need from 16-bit operands: 16-byte aligned rows of x and w, 8-byte aligned groups of 4
@@ -72,7 +93,12 @@ int tpamd::linear_entry(const char *who, const void *x_dev, const void *w_dev, c
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, w_dev, nullptr, bias_dev, y_dev, N, K, ldx, ldw, ldy) &&
                       (addend_dev == nullptr || (aligned(addend_dev, 8) && ldadd % 4 == 0));
-    if (fast && M <= SKINNY_MAX_M)
+    int64_t skinny_rows = SKINNY_MAX_M;
+    if (fast && M > SKINNY_MAX_M && M <= 64) {
+        rc = skinny_row_limit(N, K, &skinny_rows);
+        if (rc != TPAMD_OK) return rc;
+    }
+    if (fast && M <= skinny_rows)
         return skinny_dispatch(x_dev, w_dev, nullptr, bias_dev, addend_dev, ldadd, nullptr, nullptr, nullptr, 0, y_dev, M, N, K,
                                ldx, ldw, ldy, 0, dtype, act, false, false, s);
     return gemm_dispatch(x_dev, w_dev, nullptr, bias_dev, addend_dev, ldadd, y_dev, M, N, K, ldx, ldw, ldy, dtype, act, false,

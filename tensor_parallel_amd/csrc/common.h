@@ -46,6 +46,7 @@ struct Tuning {
     int skinny_resident;     // TPAMD_SKINNY_RESIDENT: x-resident kernel on/off
     int w8_split;            // TPAMD_W8_SPLIT: int8 K-split kernel on/off
     int w8_cols;             // TPAMD_W8_COLS: int8 K-split kernel whose wavefronts own columns (x of the split in LDS): 0 = off, 1 = whenever the shape allows
+    int skinny_max_m;        // TPAMD_SKINNY_MAX_M: most rows of a single 16-bit matrix that go to the weight-streaming kernels (16 to 64; unset: by shape)
     int skinny_xlds;         // TPAMD_SKINNY_XLDS: 0 = gated pair at 4-16 rows through the older kernels
     int gemv_rows;           // TPAMD_GEMV_ROWS: wavefronts per block of the unrolled M <= 3 kernel (2, 4, 8, 16); 0 = the general kernel
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel

@@ -30,6 +30,7 @@ Tuning read_tuning() {
     t.w8_split = env_int("TPAMD_W8_SPLIT");
     t.w8_cols = env_int("TPAMD_W8_COLS");
     t.skinny_xlds = env_int("TPAMD_SKINNY_XLDS");
+    t.skinny_max_m = env_int("TPAMD_SKINNY_MAX_M");
     t.gemv_rows = env_int("TPAMD_GEMV_ROWS");
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
     t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");

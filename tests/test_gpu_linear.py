@@ -353,6 +353,31 @@ def test_x_resident_weight_streaming_kernel(dtype, M, N, K, tune):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(2048, 4096), (4096, 5504), (1000, 2056), (132, 8192)])
+def test_single_matrix_with_few_tiles_at_17_to_64_rows(dtype, M, N, K):
+    """A single 16-bit matrix with at most one 16-column tile per CU stays on the weight-streaming kernel up to 32 rows
+    (up to 64 with at most half a tile per CU): two and four row tiles of x, a partly filled last one, a ragged last K
+    chunk, bias and GELU; and the same shapes with the rows limited to 16 (the tiled kernels) agree."""
+    x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
+    got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
+    check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
+
+
+def test_rows_limit_of_the_weight_streaming_kernels_can_be_forced(tune):
+    """TPAMD_SKINNY_MAX_M = 64 sends 17 to 64 rows of any single 16-bit matrix to the weight-streaming kernel, 16 sends
+    them to the tiled kernels: same result within rounding."""
+    M, N, K = 40, 4608, 4096
+    x, w = rnd((M, K), 1), rnd((N, K), 0, 0.02)
+    tune("TPAMD_SKINNY_MAX_M", "64")
+    streamed = _native.linear(x.to(DEV), w.to(DEV))
+    tune("TPAMD_SKINNY_MAX_M", "16")
+    tiled = _native.linear(x.to(DEV), w.to(DEV))
+    check_half(streamed, F.linear(x.float(), w.float()), K)
+    check_half(tiled, F.linear(x.float(), w.float()), K)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [4, 7, 12, 16])
 @pytest.mark.parametrize("N,K", [(8, 64), (64, 64), (133, 200), (1028, 1000), (2740, 4096), (520, 5504), (4100, 2048), (300, 8192), (260, 7000),
                                  (16400, 512)])

@@ -43,6 +43,13 @@ def test_fused_add_equals_linear_then_add(dtype, M, N, K):
     check_fused(x, w, None, a, act=_native.ACT_GELU)
 
 
+@pytest.mark.parametrize("M", [17, 32, 40, 64])
+def test_fused_add_on_the_weight_streaming_kernel_above_16_rows(M):
+    """Few output tiles per CU: 17 to 64 rows of a single matrix stay on the weight-streaming kernel."""
+    x, w, a = rnd((M, 4096), 1).to(DEV), rnd((1024, 4096), 0, 0.05).to(DEV), rnd((M, 1024), 5).to(DEV)
+    check_fused(x, w, None, a)
+
+
 @pytest.mark.parametrize("M,N,K", [(5, 7, 3), (70, 10, 36), (33, 130, 8)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_fused_add_on_the_scalar_kernel(dtype, M, N, K):
