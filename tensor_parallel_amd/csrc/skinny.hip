@@ -801,7 +801,7 @@ int launch_w8_finish(const SkinnyParams &p, const float *part, int splits, hipSt
 constexpr int WC_NW = 8, WC_UNIT_K = 128, WC_STAGE = 32 * 128;  // per wavefront: two tiles of 16 staged rows
 
 template <int DT, int MT, int KU, bool DIRECT>
-__global__ __launch_bounds__(WC_NW * 64) void skinny_w8_cols_kernel(SkinnyParams p, float *part, int cols_per_block, int k_planes) {
+__global__ __launch_bounds__(WC_NW * 64, MT == 1 ? 4 : 2) void skinny_w8_cols_kernel(SkinnyParams p, float *part, int cols_per_block, int k_planes) {
     constexpr int NW = WC_NW;
     extern __shared__ __align__(16) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -911,7 +911,10 @@ __global__ __launch_bounds__(WC_NW * 64) void skinny_w8_cols_kernel(SkinnyParams
     // first bytes of the matrix. A slot: [tile A rows 0-7, A rows 8-15, B rows 0-7, B rows 8-15], 128 bytes of each row.
     // The four row addresses of a pair are worked out once (set_pair); a unit is an immediate offset from them. In the last
     // plane of a K that does not fill it, units past the end of K read the first bytes of the matrix instead (x is 0 there).
-    constexpr int D = 4;
+    // Units in flight per wavefront. Up to 16 rows two of them keep the kernel within 128 registers, so that two blocks
+    // fit a CU (64 KiB of LDS each): the blocks of the outlier plane then run beside the others instead of after them
+    // (Falcon-40B MLP shard at 2 / 4 / 16 rows: 29.0 + 30.2 / 29.4 + 30.4 / 34.1 + 34.5 -> 26.7 + 28.7 / 27.5 + 29.2 / 32.2 + 33.9 us).
+    constexpr int D = MT == 1 ? 2 : 4;
     static_assert(KU % D == 0, "the ring divides a tile");
     uint4 wv[D][4];
     const char *rowp[4];
