@@ -801,7 +801,7 @@ int launch_w8_finish(const SkinnyParams &p, const float *part, int splits, hipSt
 constexpr int WC_NW = 8, WC_UNIT_K = 128, WC_STAGE = 32 * 128;  // per wavefront: two tiles of 16 staged rows
 
 template <int DT, int MT, int KU, bool DIRECT>
-__global__ __launch_bounds__(WC_NW * 64, MT == 1 ? 4 : 2) void skinny_w8_cols_kernel(SkinnyParams p, float *part, int cols_per_block, int k_planes) {
+__global__ __launch_bounds__(WC_NW * 64, MT == 1 ? 4 : 1) void skinny_w8_cols_kernel(SkinnyParams p, float *part, int cols_per_block, int k_planes) {
     constexpr int NW = WC_NW;
     extern __shared__ __align__(16) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
