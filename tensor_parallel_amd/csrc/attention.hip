@@ -34,6 +34,15 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+typedef __attribute__((ext_vector_type(4))) short i16x4;
+
+// ds_read_b64_tr_b16: every lane gives the LDS address of four 16-bit elements; within each group of 16 lanes,
+// lane i receives element i % 4 of lanes i / 4, 4 + i / 4, 8 + i / 4 and 12 + i / 4 (in that order).
+__device__ __forceinline__ uint2 lds_transpose_b64(const char *lds_ptr) {
+    auto *ptr = reinterpret_cast<__attribute__((address_space(3))) i16x4 *>(reinterpret_cast<uintptr_t>(lds_ptr));
+    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(ptr));
+}
+
 struct AttnParams {
     const char *q, *k, *v;
     char *o;
@@ -54,12 +63,12 @@ constexpr int AT_KEYS = 64;   // keys per tile
 // AGPRs the compiler keeps MFMA results in ordinary VGPRs, where the softmax can use them without copies.
 template <int DT, int D, int RT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) void attention_kernel(AttnParams p) {
-    constexpr int KP = D * 2 + 16;        // K tile row pitch (bytes): conflict-free 16-byte reads
-    constexpr int VP = AT_KEYS * 2 + 8;   // V^T tile row pitch (bytes), 8-byte aligned
+    constexpr int KP = D * 2 + 16;   // K tile row pitch (bytes): conflict-free 16-byte reads
+    constexpr int VP = D * 2 + 32;   // V tile row pitch (bytes): 8 consecutive keys' 32-byte pieces cover all banks
     constexpr int DT16 = D / 16, DK = D / 32;
     constexpr int ROWS = 64 * RT;
-    __shared__ __align__(16) char ks[AT_KEYS * KP];
-    __shared__ __align__(16) char vt[D * VP];
+    __shared__ __align__(16) char ks[2][AT_KEYS * KP];  // two tiles each: one is multiplied while the next is written
+    __shared__ __align__(16) char vs[2][AT_KEYS * VP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, lq = lane >> 4;
@@ -127,45 +136,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     const char *kbase = p.k + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh) * 2;
     const char *vbase = p.v + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh) * 2;
 
-    // K / V tiles travel global -> registers -> LDS; the registers of tile i+1 are requested before tile i is
-    // multiplied, so the loads fly during the MFMAs and the softmax. Keys past the end are zero (and masked below).
+    // K / V tiles travel global -> registers -> LDS (row-major, both). The registers of tile i+2 are requested right after
+    // tile i+1 has been written to the other LDS buffer, so the loads fly during a whole tile's MFMAs and softmax, and a
+    // tile costs one barrier. A full tile's addresses are a loop-invariant per-thread pointer plus a uniform offset.
     constexpr int CH = D / 8;                    // 16-byte chunks per key
     constexpr int LPT = AT_KEYS * CH / 256;      // chunks per thread per tile (2 for head_dim 64, 4 for 128)
+    constexpr int KSTEP = 256 / CH;              // keys between a thread's chunks
     uint4 kreg[LPT], vreg[LPT];
-    const int key_j0 = tid / CH, chunk = tid % CH;  // thread's key inside a tile for j = 0; j adds 256 / CH keys
-    const char *kthr = kbase + chunk * 16, *vthr = vbase + chunk * 16;
+    const int key_j0 = tid / CH, chunk = tid % CH;  // thread's key inside a tile for j = 0
     const int64_t k_pitch = p.k_ss * 2, v_pitch = p.v_ss * 2;
+    const char *kthr = kbase + chunk * 16 + key_j0 * k_pitch, *vthr = vbase + chunk * 16 + key_j0 * v_pitch;
     auto fetch = [&](int k0) {
+        if (k0 + AT_KEYS <= k_end) {  // uniform
 #pragma unroll
-        for (int j = 0; j < LPT; ++j) {
-            const int key = k0 + key_j0 + j * (256 / CH);
-            const bool ok = key < k_end;
-            // unconditional loads (first key of the range when out of it) keep all of them in flight together
-            const int64_t kr = ok ? key : k_begin;
-            const uint4 kv4 = *reinterpret_cast<const uint4 *>(kthr + kr * k_pitch);
-            const uint4 vv4 = *reinterpret_cast<const uint4 *>(vthr + kr * v_pitch);
-            kreg[j] = ok ? kv4 : make_uint4(0, 0, 0, 0);
-            vreg[j] = ok ? vv4 : make_uint4(0, 0, 0, 0);
-        }
-    };
-    auto stage = [&]() {
+            for (int j = 0; j < LPT; ++j) {
+                kreg[j] = *reinterpret_cast<const uint4 *>(kthr + static_cast<int64_t>(k0 + j * KSTEP) * k_pitch);
+                vreg[j] = *reinterpret_cast<const uint4 *>(vthr + static_cast<int64_t>(k0 + j * KSTEP) * v_pitch);
+            }
+        } else {
 #pragma unroll
-        for (int j = 0; j < LPT; ++j) {
-            const int e = tid + j * 256, key = e / CH, c = e % CH;
-            *reinterpret_cast<uint4 *>(ks + key * KP + c * 16) = kreg[j];
-            const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * i) * VP + key * 2) = static_cast<uint16_t>(w[i] & 0xffffu);
-                *reinterpret_cast<uint16_t *>(vt + (c * 8 + 2 * i + 1) * VP + key * 2) = static_cast<uint16_t>(w[i] >> 16);
+            for (int j = 0; j < LPT; ++j) {
+                const int key = k0 + key_j0 + j * KSTEP;
+                const bool ok = key < k_end;
+                // unconditional loads (first key of the range when out of it) keep all of them in flight together;
+                // keys past the end are zero (and masked below)
+                const int64_t kr = ok ? key : k_begin;
+                const uint4 kv4 = *reinterpret_cast<const uint4 *>(kbase + chunk * 16 + kr * k_pitch);
+                const uint4 vv4 = *reinterpret_cast<const uint4 *>(vbase + chunk * 16 + kr * v_pitch);
+                kreg[j] = ok ? kv4 : make_uint4(0, 0, 0, 0);
+                vreg[j] = ok ? vv4 : make_uint4(0, 0, 0, 0);
             }
         }
     };
-    if (k_begin < k_end) fetch(k_begin);
-    for (int k0 = k_begin; k0 < k_end; k0 += AT_KEYS) {
-        stage();
-        __syncthreads();
-        if (k0 + AT_KEYS < k_end) fetch(k0 + AT_KEYS);
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < LPT; ++j) {
+            const int key = key_j0 + j * KSTEP;
+            *reinterpret_cast<uint4 *>(ks[buf] + key * KP + chunk * 16) = kreg[j];
+            *reinterpret_cast<uint4 *>(vs[buf] + key * VP + chunk * 16) = vreg[j];
+        }
+    };
+    // The transposed V fragments come from the LDS transpose load: the 16 lanes of a group point at 4 keys x 16 head-dim
+    // elements (lane j: key j / 4, elements 4 (j % 4) ...) and lane i gets back, for head-dim element i, its 4 keys.
+    // This lane's address inside a V tile: key 4 lq + l16 / 4, element 4 (l16 % 4); (u, half, dt) add (32 u + 16 half)
+    // keys and 16 dt elements.
+    const int v_lane = (4 * lq + (l16 >> 2)) * VP + (l16 & 3) * 8;
+    if (k_begin < k_end) {
+        fetch(k_begin);
+        stage(0);
+        if (k_begin + AT_KEYS < k_end) fetch(k_begin + AT_KEYS);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = k_begin; k0 < k_end; k0 += AT_KEYS, buf ^= 1) {
+        const char *kt = ks[buf], *vtile = vs[buf];
 
         // ---- S^T = K Q^T: s[r][t][i] = score of key k0 + 16 t + 4 lq + i against query row r of this lane
         f32x4 s[RT][4];
@@ -175,7 +199,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
             for (int r = 0; r < RT; ++r) s[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < DK; ++kk) {
-                const uint4 kf = *reinterpret_cast<const uint4 *>(ks + (16 * t + l16) * KP + (32 * kk + 8 * lq) * 2);
+                const uint4 kf = *reinterpret_cast<const uint4 *>(kt + (16 * t + l16) * KP + (32 * kk + 8 * lq) * 2);
 #pragma unroll
                 for (int r = 0; r < RT; ++r) s[r][t] = mfma16<DT>(kf, qf[r][kk], s[r][t]);
             }
@@ -204,16 +228,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 #pragma unroll
                     for (int i = 0; i < 4; ++i) s[r][t][i] = (16 * t + i < vis) ? s[r][t][i] : -INFINITY;
             }
-            float mx = fmaxf(fmaxf(s[r][0][0], s[r][0][1]), fmaxf(s[r][0][2], s[r][0][3]));
+            // x = score * scale log2 e - reference; the products are canonical numbers, so their maximum is a plain chain
+            // of 3-input maxima (the MFMA results themselves would each be canonicalised first)
+            const float neg_ref = m_run[r] == -INFINITY ? 0.f : -m_run[r];
 #pragma unroll
-            for (int t = 1; t < 4; ++t) mx = fmaxf(mx, fmaxf(fmaxf(s[r][t][0], s[r][t][1]), fmaxf(s[r][t][2], s[r][t][3])));
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            mx *= p.scale_log2;  // scale > 0: the maximum of the scaled scores
-            if (__any(mx > m_run[r] + LAZY)) {  // wavefront-uniform: some row's maximum outgrew its reference
-                const float m_new = mx > m_run[r] + LAZY ? mx : m_run[r];
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[r][t][i] = fmaf(s[r][t][i], p.scale_log2, neg_ref);
+            float mx = fmaxf(s[r][0][0], s[r][0][1]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = (t == 0 ? 2 : 0); i < 4; i += 2) mx = fmaxf(fmaxf(mx, s[r][t][i]), s[r][t][i + 1]);
+            // every lane looks at its own 16 keys: only when one of them outgrew the reference (or the row has none yet)
+            // do the 4 lanes of a row exchange their maxima
+            if (__any(mx > LAZY || m_run[r] == -INFINITY)) {
+                mx = fmaxf(mx, __shfl_xor(mx, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                // in absolute units; a row that keeps its reference goes through the same arithmetic with factor 1
+                const float m_abs = mx - neg_ref;
+                const bool up = m_abs > m_run[r] + LAZY;  // false for -inf on either side
+                const float m_new = up ? m_abs : m_run[r];
                 const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row with nothing visible yet
                 const float alpha = __builtin_amdgcn_exp2f(m_run[r] - m_use);
+                const float move = -neg_ref - m_use;  // x was taken against the old reference
                 m_run[r] = m_new;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) l_acc[r][i] *= alpha;
@@ -221,12 +259,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
                 for (int dt = 0; dt < DT16; ++dt)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) acc[r][dt][i] *= alpha;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[r][t][i] += move;
             }
-            const float neg_ref = m_run[r] == -INFINITY ? 0.f : -m_run[r];
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) s[r][t][i] = __builtin_amdgcn_exp2f(fmaf(s[r][t][i], p.scale_log2, neg_ref));
+                for (int i = 0; i < 4; ++i) s[r][t][i] = __builtin_amdgcn_exp2f(s[r][t][i]);
             // the lane's probabilities as the second MFMA operand. K slot (lq, e): e < 4 -> key 32 u + 4 lq + e,
             // e >= 4 -> key 32 u + 16 + 4 lq + e - 4
 #pragma unroll
@@ -243,15 +284,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         for (int u = 0; u < 2; ++u) {
 #pragma unroll
             for (int dt = 0; dt < DT16; ++dt) {
-                const char *vrow = vt + (16 * dt + l16) * VP + (32 * u + 4 * lq) * 2;
-                const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
-                const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 32);
+                const uint2 lo = lds_transpose_b64(vtile + v_lane + (32 * u) * VP + 32 * dt);
+                const uint2 hi = lds_transpose_b64(vtile + v_lane + (32 * u + 16) * VP + 32 * dt);
                 const uint4 vf = make_uint4(lo.x, lo.y, hi.x, hi.y);
 #pragma unroll
                 for (int r = 0; r < RT; ++r) acc[r][dt] = mfma16<DT>(vf, pf[r][u], acc[r][dt]);
             }
 #pragma unroll
             for (int r = 0; r < RT; ++r) l_acc[r] = mfma16<DT>(ones, pf[r][u], l_acc[r]);
+        }
+        // the next tile into the other buffer (last read one tile ago, before the previous barrier)
+        if (k0 + AT_KEYS < k_end) {
+            stage(buf ^ 1);
+            if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
         }
         __syncthreads();
     }
