@@ -10,7 +10,7 @@
 //   online softmax in exp2 domain (scale * log2 e folded in),
 //   O^T += V^T P^T the lane's 8 probabilities of two key tiles are exactly the second operand of the next MFMA
 //                 (the K index of an MFMA may be permuted freely as long as both operands agree), the first
-//                 operand comes from a transposed copy of the V tile in LDS.
+//                 operand comes from the row-major V tile in LDS through the LDS transpose load.
 // O^T leaves a lane with 4 consecutive head-dim elements of one query row: one 8-byte store into [B, Sq, Hq, D].
 //
 // Long key ranges with few rows (decode) are split over blockIdx.z; every split leaves (m, l, unnormalised O) in
@@ -206,11 +206,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         }
         // ---- online softmax per row (the 4 lanes l16 + 16 * {0..3} hold the same row).
         // Probabilities are taken relative to a reference maximum m_run (in units of scale * log2 e) that is only
-        // raised when the running maximum outgrows it by more than 2^LAZY: then the accumulators (which live in
-        // AGPRs: rescaling them costs three instructions per element) are rescaled; otherwise
-        // p = 2^(x - m_run) <= 2^LAZY, well inside what 16-bit p and fp32 sums hold. A tile fully visible to every
-        // row of the wavefront skips the masking. The row sums come out of the MFMA pipe (a row of ones appended
-        // to V^T) instead of 16 additions per row and tile.
+        // raised when the running maximum outgrows it by more than 2^LAZY: then the accumulators are rescaled;
+        // otherwise p = 2^(x - m_run) <= 2^LAZY, well inside what 16-bit p and fp32 sums hold. A tile fully visible to
+        // every row of the wavefront skips the masking. The row sums come out of the MFMA pipe (a row of ones appended
+        // to V^T) instead of 16 additions per row and tile. The loop is paced by the vector instructions around the
+        // MFMAs as much as by the MFMAs (on a SIMD the two did not overlap in any arrangement that was timed), so the
+        // fast path of a tile is one fma, one exp2, half a 3-input maximum and half a pack per score, nothing else.
         constexpr float LAZY = 6.0f;
         uint4 pf[RT][2];
         bool tile_free = k0 + AT_KEYS <= k_end;
