@@ -45,6 +45,40 @@ def test_attention_matches_oracle(dtype, causal, B, Hq, Hkv, Sq, Skv, D):
     check(*make(B, Hq, Hkv, Sq, Skv, D, dtype), causal)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Skv", [64, 65, 127, 128, 129, 192, 200, 256, 321])
+@pytest.mark.parametrize("Sq", [1, 40, 130])
+def test_key_counts_around_the_tile_size(Sq, Skv, causal):
+    """1 to 6 key tiles of 64, full and ragged: the tiles alternate between two LDS buffers and the tile after next is
+    prefetched, so every count of tiles ends the pipeline differently."""
+    if causal and Sq > Skv:
+        pytest.skip("more new positions than keys")
+    check(*make(2, 4, 2, Sq, Skv, 64, torch.bfloat16, seed=Sq * 1000 + Skv), causal)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Sq,causal", [(1, False), (96, False), (96, True)])
+def test_reference_maximum_moves_along_the_keys(dtype, Sq, causal):
+    """Scores that grow along the keys, in steps larger and smaller than the 2^6 the running reference tolerates, then
+    fall again: the accumulators are rescaled several times and most tiles take the path without any rescaling."""
+    B, Hq, Hkv, Skv, D = 1, 4, 2, 640, 64
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, Hq, Sq, D, generator=g)
+    k = torch.randn(B, Hkv, Skv, D, generator=g) * 0.05
+    v = torch.randn(B, Hkv, Skv, D, generator=g)
+    # keys aligned with the mean query direction get a score that depends on their position
+    direction = q.mean(dim=(0, 1, 2))
+    direction = direction / direction.norm()
+    level = torch.zeros(Skv)
+    level[64:128] = 2.0      # a small step: inside the tolerance
+    level[128:320] = 12.0    # a large one
+    level[320:384] = 40.0    # larger still, for one tile
+    level[384:] = 11.0       # and back
+    k = k + level[None, None, :, None] * direction[None, None, None, :]
+    q = q + 3.0 * direction  # every query has a clearly positive component along it
+    check(q.to(dtype), k.to(dtype), v.to(dtype), causal, scale=1.0)
+
+
 def test_strided_inputs_as_projection_outputs_produce_them():
     """q / k / v as views of [B, S, H, D] projection outputs (what the attention modules pass), sliced cache."""
     B, Hq, Hkv, S, D = 2, 8, 2, 96, 64
