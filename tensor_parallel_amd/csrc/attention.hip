@@ -92,13 +92,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     const int row0 = row_tile * ROWS;
     const int shift = p.Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
 
+    // Causal: the wavefronts that own a block's first rows stop early (below), and a wavefront's number fixes its SIMD, so
+    // every other row tile hands the rows out in the opposite order.
+    const int wave_rows = (p.causal && (row_tile & 1)) ? 3 - wave : wave;
     // ---- this lane's query rows and their Q fragments (second MFMA operand): 8 head-dim elements at 32*kk + 8*lq
     int row[RT], sq[RT], head[RT], my_lim[RT];
     bool row_ok[RT];
     uint4 qf[RT][DK];
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
-        row[r] = row0 + (wave * RT + r) * 16 + l16;
+        row[r] = row0 + (wave_rows * RT + r) * 16 + l16;
         row_ok[r] = row[r] < nrows;
         const int g = row_ok[r] ? row[r] / p.Sq : 0;
         sq[r] = row_ok[r] ? row[r] % p.Sq : 0;
@@ -188,7 +191,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     }
     __syncthreads();
     int buf = 0;
-    for (int k0 = k_begin; k0 < k_end; k0 += AT_KEYS, buf ^= 1) {
+    // Causal: a wavefront multiplies only the tiles some row of its own can see (the block's range ends with the last row of
+    // the block); for the tiles behind them it only takes part in the staging and the barriers.
+    int wave_lim = my_lim[0];
+#pragma unroll
+    for (int r = 1; r < RT; ++r) wave_lim = max(wave_lim, my_lim[r]);
+#pragma unroll
+    for (int d = 1; d < 16; d *= 2) wave_lim = max(wave_lim, __shfl_xor(wave_lim, d));
+    wave_lim = __builtin_amdgcn_readfirstlane(wave_lim);
+    const int k_stop = min(k_end, wave_lim + 1);
+    int k0 = k_begin;
+    for (; k0 < k_stop; k0 += AT_KEYS, buf ^= 1) {
         const char *kt = ks[buf], *vtile = vs[buf];
 
         // ---- S^T = K Q^T: s[r][t][i] = score of key k0 + 16 t + 4 lq + i against query row r of this lane
@@ -295,6 +308,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
             for (int r = 0; r < RT; ++r) l_acc[r] = mfma16<DT>(ones, pf[r][u], l_acc[r]);
         }
         // the next tile into the other buffer (last read one tile ago, before the previous barrier)
+        if (k0 + AT_KEYS < k_end) {
+            stage(buf ^ 1);
+            if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
+        }
+        __syncthreads();
+    }
+    for (; k0 < k_end; k0 += AT_KEYS, buf ^= 1) {
         if (k0 + AT_KEYS < k_end) {
             stage(buf ^ 1);
             if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
