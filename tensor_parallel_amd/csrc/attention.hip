@@ -191,15 +191,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     }
     __syncthreads();
     int buf = 0;
-    // Causal: a wavefront multiplies only the tiles some row of its own can see (the block's range ends with the last row of
-    // the block); for the tiles behind them it only takes part in the staging and the barriers.
+    // A wavefront multiplies only the tiles some row of its own can see (causal: the block's range ends with the last row
+    // of the block); for the tiles behind them it only takes part in the staging and the barriers.
     int wave_lim = my_lim[0];
 #pragma unroll
     for (int r = 1; r < RT; ++r) wave_lim = max(wave_lim, my_lim[r]);
 #pragma unroll
     for (int d = 1; d < 16; d *= 2) wave_lim = max(wave_lim, __shfl_xor(wave_lim, d));
     wave_lim = __builtin_amdgcn_readfirstlane(wave_lim);
-    const int k_stop = min(k_end, wave_lim + 1);
+    // ... and none at all when all its rows lie past the end (decode: 16 rows in a block of 64)
+    bool any_row = false;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) any_row = any_row || row_ok[r];
+    const int k_stop = __any(any_row) ? min(k_end, wave_lim + 1) : k_begin;
     int k0 = k_begin;
     for (; k0 < k_stop; k0 += AT_KEYS, buf ^= 1) {
         const char *kt = ks[buf], *vtile = vs[buf];
