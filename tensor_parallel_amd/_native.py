@@ -438,10 +438,12 @@ def swiglu_up(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor) -> torch.Tens
     return h.view(*x.shape[:-1], N)
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None, causal: bool = True) -> torch.Tensor:
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None, causal: bool = True,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """softmax(scale * q k^T [+ causal]) v. q [B, Hq, Sq, D], k / v [B, Hkv, Skv, D] -> [B, Sq, Hq, D] (the layout the
     attention output projection consumes). Grouped-query heads when Hq > Hkv; causal is aligned to the END of the key
-    range (query i sees keys j <= i + Skv - Sq)."""
+    range (query i sees keys j <= i + Skv - Sq). `out`, if given, is a [B, Sq, Hq, D] tensor (or view) of q's dtype and
+    device whose rows are contiguous and start on 8-byte boundaries."""
     require_device(q, "attention")
     if not (q.dtype == k.dtype == v.dtype) or q.dtype not in (torch.bfloat16, torch.float16):
         raise TypeError("attention: q, k, v must share bfloat16 or float16")
@@ -452,7 +454,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional
     B, Hq, Sq, D = q.shape
     Hkv, Skv = k.shape[1], k.shape[2]
     q, k, v = (t if t.stride(3) == 1 else t.contiguous() for t in (q, k, v))
-    out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+    elif out.shape != (B, Sq, Hq, D) or out.dtype != q.dtype or out.device != q.device or out.stride(3) != 1:
+        raise ValueError(f"attention: out must be a [{B}, {Sq}, {Hq}, {D}] {q.dtype} tensor on {q.device} with contiguous rows")
     strides = (ctypes.c_int64 * 12)(q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
                                     v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2))
     with _on_device(q.device):

@@ -79,6 +79,22 @@ def test_reference_maximum_moves_along_the_keys(dtype, Sq, causal):
     check(q.to(dtype), k.to(dtype), v.to(dtype), causal, scale=1.0)
 
 
+@pytest.mark.parametrize("Sq", [1, 200])
+def test_output_rows_on_8_byte_boundaries_only(Sq):
+    """The output may be a view whose rows start on 8-byte boundaries (the ABI asks for no more), with other data between
+    the rows."""
+    B, Hq, Hkv, Skv, D = 2, 4, 2, 200, 64
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, torch.bfloat16, seed=11)
+    want = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=True)
+    store = torch.full((B, Sq, Hq, D + 4), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = store[..., 4:]  # rows at byte offsets 8, 144, ...: 8-byte but not 16-byte aligned
+    assert out.data_ptr() % 16 == 8
+    got = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=True, out=out)
+    assert got.data_ptr() == out.data_ptr()
+    torch.testing.assert_close(got, want, rtol=0, atol=0)
+    assert bool((store[..., :4] == 7.0).all())
+
+
 def test_strided_inputs_as_projection_outputs_produce_them():
     """q / k / v as views of [B, S, H, D] projection outputs (what the attention modules pass), sliced cache."""
     B, Hq, Hkv, S, D = 2, 8, 2, 96, 64
