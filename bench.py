@@ -68,10 +68,6 @@ def main() -> int:
     ap.add_argument("--tokens", type=int, default=4096)
     ap.add_argument("--settle", type=int, default=240, help="untimed steps before the counted warm-up (clock settling)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--ceilings", nargs="?", const="all", default=None, choices=["all", "mfma", "streams", "gemm", "decode"],
-                    help="instead of the benchmark, measure what this part sustains on the two bounding resources (MFMA-only "
-                         "loop, read / write / copy streams) and time hipBLASLt on the benchmark's GEMM shapes beside this "
-                         "library's kernels; prints a table and one JSON line")
     ap.add_argument("--no-extra", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -88,8 +84,6 @@ def main() -> int:
         return 1
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
-    if args.ceilings:
-        return ceilings(torch, _native, dev, args.ceilings)
     M = args.tokens
     g = torch.Generator(device=dev).manual_seed(0)
 
@@ -172,167 +166,6 @@ def main() -> int:
         out["extra"] = extra_measurements(torch, _native, dev, sets, other)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
-    print(json.dumps(out), flush=True)
-    return 0
-
-
-def ceilings(torch, _native, dev, which="all") -> int:
-    """What bounds the kernels on this part, measured in one process. Every figure is taken after the part has run the
-    same load for a while (its clock settles over tens of milliseconds), as the average over the launches that follow.
-    `which` picks one section (mfma, streams, gemm, decode) or all of them."""
-    import ctypes
-
-    from tensor_parallel_amd.build import PROBES_LIB
-
-    probes = ctypes.CDLL(str(PROBES_LIB))
-    vp, ci, u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64
-    probes.tpamd_probe_mfma.argtypes = [ci, vp, vp, ci, ci, vp]
-    probes.tpamd_probe_mfma_flops.restype = ctypes.c_double
-    probes.tpamd_probe_mfma_flops.argtypes = [ci, ci, ci]
-    probes.tpamd_probe_stream.argtypes = [ci, ci, ci, vp, vp, u64, ci, vp, vp]
-    stream = lambda: vp(torch.cuda.current_stream(dev).cuda_stream)  # noqa: E731
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    sink = torch.zeros(256, device=dev)
-    out = {"device": torch.cuda.get_device_name(dev), "cus": cus}
-
-    def settled_us(fn, settle_s=0.25, iters=40):
-        """Average launch time of fn(i) after running it for settle_s seconds."""
-        t0, i = time.perf_counter(), 0
-        while time.perf_counter() - t0 < settle_s:
-            fn(i)
-            i += 1
-            if i % 16 == 0:
-                torch.cuda.synchronize()
-        torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for j in range(iters):
-            fn(i + j)
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / iters * 1e3
-
-    def mfma_only():
-        """Nothing but MFMAs: constant operands against random ones, both instruction shapes."""
-        n_vec = cus * 256 * 8
-        ops = {"constant": torch.full((n_vec * 8,), 1.0, device=dev).to(torch.bfloat16),
-               "random": (torch.randn(n_vec * 8, device=dev, generator=torch.Generator(device=dev).manual_seed(0)) * 2).to(torch.bfloat16)}
-        rows = {}
-        for shape, name in ((16, "v_mfma_f32_16x16x32_bf16"), (32, "v_mfma_f32_32x32x16_bf16")):
-            iters = 20000
-            flops = probes.tpamd_probe_mfma_flops(shape, cus, iters)
-            for kind, buf in ops.items():
-                us = settled_us(lambda i: probes.tpamd_probe_mfma(shape, vp(buf.data_ptr()), vp(sink.data_ptr()), cus, iters, stream()), 0.4, 10)
-                rows[f"{name} {kind} operands"] = {"us": us, "TFLOPs": flops / us / 1e6, "frac_of_2500": flops / us / 1e6 / PEAK_BF16_TFLOPS}
-        return rows
-
-    def stream_probes():
-        """Read-only, write-only and copy streams at the byte counts of the HBM-bound kernels: the down matrix, the gate
-        and up matrices, every split tensor of the state dict. Best of plain / non-temporal accesses, 4 / 16 / 32 KiB per
-        block step and 4 / 8 / 16 blocks per CU; buffers rotated so that the 256 MB Infinity Cache cannot serve them."""
-        rows = {}
-        sizes = (("llama7b_down_shard_45MB", FFN_SHARD * D_MODEL * 2, 6), ("llama7b_gate_up_shards_90MB", 2 * FFN_SHARD * D_MODEL * 2, 4),
-                 ("llama2_7b_split_tensors_13.5GB", 13476298752, 1))
-        for label, nbytes, copies in sizes:
-            nbytes = nbytes // 131072 * 131072
-            srcs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
-            dsts = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(copies)]
-            row = {}
-            for mode, what, moved in ((0, "read_only", nbytes), (1, "write_only", nbytes), (2, "copy_read_plus_write", 2 * nbytes)):
-                best = None
-                for nt in (1, 0):
-                    for piece in (4096, 16384, 32768, 131072):  # 131072: bursts of one 1024-thread block (1 or 2 blocks per CU)
-                        for per_cu in ((1, 2) if piece == 131072 else (4, 8, 16)):
-                            us = settled_us(lambda i: probes.tpamd_probe_stream(mode, nt, piece, vp(srcs[i % copies].data_ptr()), vp(dsts[i % copies].data_ptr()),
-                                                                                nbytes, cus * per_cu, vp(sink.data_ptr()), stream()), 0.05, 20 if nbytes < 1e9 else 4)
-                            if best is None or us < best[0]:
-                                best = (us, per_cu, nt, piece)
-                row[what] = {"us": best[0], "GBps": moved / best[0] / 1e3, "frac_of_8000": moved / best[0] / 1e3 / PEAK_HBM_GBS, "blocks_per_cu": best[1],
-                             "non_temporal": bool(best[2]), "piece_bytes": best[3]}
-            us = settled_us(lambda i: dsts[i % copies].copy_(srcs[i % copies]), 0.15, 20 if nbytes < 1e9 else 5)
-            row["device_to_device_copy_of_the_runtime"] = {"us": us, "GBps": 2 * nbytes / us / 1e3, "frac_of_8000": 2 * nbytes / us / 1e3 / PEAK_HBM_GBS}
-            rows[label] = row
-            del srcs, dsts
-        return rows
-
-    def gemm_side_by_side():
-        """hipBLASLt (through torch.matmul) on the benchmark's GEMM shapes beside this library's kernels."""
-        M = 4096
-        g = torch.Generator(device=dev).manual_seed(0)
-        w = lambda shape: (torch.randn(shape, generator=g, device=dev) * 0.02).to(torch.bfloat16)  # noqa: E731
-        sets = [(w((FFN_SHARD, D_MODEL)), w((FFN_SHARD, D_MODEL)), w((D_MODEL, FFN_SHARD)), torch.cat([w((FFN_SHARD, D_MODEL)), w((FFN_SHARD, D_MODEL))]))
-                for _ in range(3)]
-        x = torch.randn(M, D_MODEL, generator=g, device=dev).to(torch.bfloat16)
-        h = torch.randn(M, FFN_SHARD, generator=g, device=dev).to(torch.bfloat16) * 0.1
-        other = torch.randn(M, D_MODEL, generator=g, device=dev).to(torch.bfloat16)
-        y = torch.empty(M, D_MODEL, device=dev, dtype=torch.bfloat16)
-        gu = torch.empty(M, 2 * FFN_SHARD, device=dev, dtype=torch.bfloat16)
-        f_up, f_down = 4.0 * M * D_MODEL * FFN_SHARD, 2.0 * M * D_MODEL * FFN_SHARD
-        rows = {}
-
-        def row(label, fn, flops):
-            us = settled_us(fn, 0.3, 40)
-            rows[label] = {"us": us, "TFLOPs": flops / us / 1e6, "frac_of_2500": flops / us / 1e6 / PEAK_BF16_TFLOPS}
-
-        row("gate_up: this library, tpamd_swiglu_up (GEMM + SiLU gate fused)", lambda i: _native.swiglu_up(x, sets[i % 3][0], sets[i % 3][1]), f_up)
-        row("gate_up: hipBLASLt, one GEMM on the stacked [11008 x 4096] weight, no SiLU gate", lambda i: torch.matmul(x, sets[i % 3][3].t(), out=gu), f_up)
-        row("down: this library, tpamd_linear", lambda i: _native.linear(h, sets[i % 3][2], out=y), f_down)
-        row("down: this library, tpamd_linear_add (2-partial sum in the epilogue)", lambda i: _native.linear(h, sets[i % 3][2], addend=other, out=y), f_down)
-        row("down: hipBLASLt", lambda i: torch.matmul(h, sets[i % 3][2].t(), out=y), f_down)
-        return rows
-
-    def decode_floor():
-        """The M = 1 decode step's two weight streams (gate + up matrices: 90 MB, down matrix: 45 MB) as read-only probe
-        launches inside a HIP graph, beside this library's two kernels captured the same way: what two dependent launches
-        that only read those bytes cost here. Four buffers of each size are rotated."""
-        rows = {}
-        x = torch.randn(1, D_MODEL, device=dev).to(torch.bfloat16)
-        h = torch.randn(1, FFN_SHARD, device=dev).to(torch.bfloat16)
-        wgu = [((torch.randn(FFN_SHARD, D_MODEL, device=dev) * 0.02).to(torch.bfloat16), (torch.randn(FFN_SHARD, D_MODEL, device=dev) * 0.02).to(torch.bfloat16))
-               for _ in range(4)]
-        wd = [(torch.randn(D_MODEL, FFN_SHARD, device=dev) * 0.02).to(torch.bfloat16) for _ in range(4)]
-        for label, nbytes in (("down_45MB", FFN_SHARD * D_MODEL * 2), ("gate_up_90MB", 2 * FFN_SHARD * D_MODEL * 2)):
-            nbytes = nbytes // 32768 * 32768
-            bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(4)]
-            best = None
-            for per_cu in (4, 8, 16):
-                for piece in (4096, 32768):
-                    us = _graph_us(torch, lambda i: probes.tpamd_probe_stream(0, 1, piece, vp(bufs[i % 4].data_ptr()), None, nbytes, cus * per_cu,
-                                                                              vp(sink.data_ptr()), stream()))
-                    if best is None or us < best[0]:
-                        best = (us, per_cu, piece)
-            rows[f"read-only probe, {label}"] = {"us": best[0], "GBps": nbytes / best[0] / 1e3, "frac_of_8000": nbytes / best[0] / 1e3 / PEAK_HBM_GBS,
-                                                 "blocks_per_cu": best[1], "piece_bytes": best[2]}
-            del bufs
-        us = _graph_us(torch, lambda i: _native.linear(h, wd[i % 4]))
-        by = FFN_SHARD * D_MODEL * 2
-        rows["this library, down M=1 (tpamd_linear)"] = {"us": us, "GBps": by / us / 1e3, "frac_of_8000": by / us / 1e3 / PEAK_HBM_GBS}
-        us = _graph_us(torch, lambda i: _native.swiglu_up(x, *wgu[i % 4]))
-        rows["this library, gate/up M=1 (tpamd_swiglu_up)"] = {"us": us, "GBps": 2 * by / us / 1e3, "frac_of_8000": 2 * by / us / 1e3 / PEAK_HBM_GBS}
-        return rows
-
-    if which in ("all", "mfma"):
-        out["mfma_only_loop_4_wavefronts_per_cu"] = mfma_only()
-    if which in ("all", "streams"):
-        out["streams"] = stream_probes()
-    if which in ("all", "gemm"):
-        out["gemm_side_by_side_m4096"] = gemm_side_by_side()
-    if which in ("all", "decode"):
-        out["decode_m1_inside_hip_graph"] = decode_floor()
-    for section in ("mfma_only_loop_4_wavefronts_per_cu", "gemm_side_by_side_m4096"):
-        if section in out:
-            print(f"# {section}")
-            for k, v in out[section].items():
-                print(f"  {k:86s} {v['us']:10.1f} us {v['TFLOPs']:8.1f} TFLOP/s  {v['frac_of_2500']:.3f} of 2500")
-    if "streams" in out:
-        print("# streams")
-        for label, rowd in out["streams"].items():
-            for what, v in rowd.items():
-                print(f"  {label:34s} {what:38s} {v['us']:10.1f} us {v['GBps']:8.1f} GB/s  {v['frac_of_8000']:.3f} of 8000")
-    if "decode_m1_inside_hip_graph" in out:
-        print("# decode_m1_inside_hip_graph")
-        for k, v in out["decode_m1_inside_hip_graph"].items():
-            print(f"  {k:73s} {v['us']:10.2f} us {v['GBps']:8.1f} GB/s  {v['frac_of_8000']:.3f} of 8000")
     print(json.dumps(out), flush=True)
     return 0
 

@@ -14,7 +14,6 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 OUT_DIR = PKG / "_lib"
 LIB = OUT_DIR / "libtpamd.so"
-PROBES_LIB = OUT_DIR / "libtpamd_probes.so"  # measurement probes of `bench.py --ceilings`; not part of the product library
 SOURCES = ["api.hip", "runtime.hip", "noalloc.hip", "slice.hip", "reduce.hip", "gemm.hip", "skinny.hip", "attention.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -57,13 +56,6 @@ def build(verbose: bool = True, jobs: int = 4) -> Path:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
-    probes = _compile("probes.hip", verbose)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(PROBES_LIB), str(probes)]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"link of the probes failed:\n{res.stderr}")
     return LIB
 
 

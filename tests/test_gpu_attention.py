@@ -1,5 +1,6 @@
-"""Rank-local attention core on the GPU against the oracle (float64 on the CPU): rtol 2e-2 on 16-bit inputs,
-plus an absolute floor of 2e-2 of the value scale (outputs are convex combinations of v rows)."""
+"""Rank-local attention core on the GPU against the oracle (float64 on the CPU): rtol 2e-2 on 16-bit inputs, plus an
+absolute floor of 2e-2 standard deviations of the expected output (outputs are convex combinations of v rows: over
+2048 keys with N(0,1) values their spread is 0.03-0.04, so a floor in units of the values would hide a lost key tile)."""
 import numpy as np
 import pytest
 import torch
@@ -20,13 +21,18 @@ def make(B, Hq, Hkv, Sq, Skv, D, dtype, seed=0):
     return q, k, v
 
 
+def close(got, want):
+    want = torch.from_numpy(want)
+    torch.testing.assert_close(got.double().cpu(), want, rtol=RTOL, atol=RTOL * want.std().item())
+
+
 def check(q, k, v, causal, scale=None):
     D = q.shape[-1]
     scale = D ** -0.5 if scale is None else scale
     got = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), scale=scale, causal=causal)
     assert got.shape == (q.shape[0], q.shape[2], q.shape[1], D) and got.dtype == q.dtype
     want = oat.attention_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale, causal)
-    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL)
+    close(got, want)
     return got
 
 
@@ -106,7 +112,7 @@ def test_strided_inputs_as_projection_outputs_produce_them():
     assert not q.is_contiguous()
     got = _native.attention(q, k, v, causal=True)
     want = oat.attention_f64(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), D ** -0.5, True)
-    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL)
+    close(got, want)
     assert torch.equal(got, _native.attention(q.contiguous(), k.contiguous(), v.contiguous(), causal=True))
 
 
@@ -120,7 +126,23 @@ def test_falcon_40b_rank_shard_decode_and_prefill():
     assert torch.isfinite(got.float()).all()
     heads = [0, 17, 63]
     want = oat.attention_f64(q[:, heads].float().numpy(), k[:, [0, 1, 3]].float().numpy(), v[:, [0, 1, 3]].float().numpy(), 64 ** -0.5, True)
-    torch.testing.assert_close(got[:, :, heads].double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL)
+    close(got[:, :, heads], want)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_falcon_40b_rank_shard_prefill_at_batch_8(causal):
+    """The benchmark's prefill shape (8 x 1024 positions, 64 query heads on 4 key/value heads, 16 key tiles and 8 row
+    tiles per head), sampled (batch, head) pairs against the oracle: first, middle and last of both axes, so that a
+    block order or a row-to-wavefront mapping that goes wrong late in the grid shows."""
+    B = 8
+    q, k, v = make(B, 64, 4, 1024, 1024, 64, torch.bfloat16, seed=6)
+    got = _native.attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal)
+    assert torch.isfinite(got.float()).all()
+    for b, heads in [(0, [0, 15, 16, 63]), (3, [31, 47]), (7, [0, 33, 63])]:
+        for h in heads:
+            want = oat.attention_f64(q[b:b + 1, h:h + 1].float().numpy(), k[b:b + 1, h // 16:h // 16 + 1].float().numpy(),
+                                     v[b:b + 1, h // 16:h // 16 + 1].float().numpy(), 64 ** -0.5, causal)
+            close(got[b:b + 1, :, h:h + 1], want)
 
 
 def test_split_and_unsplit_key_ranges_agree():
