@@ -20,43 +20,101 @@ if str(ROOT) not in sys.path:
 D_MODEL, FFN_SHARD = 4096, 5504
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
-# Fabric bytes per launch of the fused gate/up GEMM at M = 4096, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
-# each scaled by what the same counter reads for the slicing kernel's known 13.476 GB (factors 1.98 and 1.00):
-# profiles/pmc_fetch_write_bench_kernels.txt. A counter reading cannot be taken inside this script.
-MEASURED_TRAFFIC_BYTES_M4096 = 629.1e6
+# Fabric bytes per launch of the fused gate/up GEMM at M = 4096 come from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE, WRITE_SIZE, each scaled by what the same counter reads for the slicing kernel's known 13.476 GB); a
+# counter cannot be read from inside the script, so the figure is taken from the committed summary of those runs.
+PMC_SUMMARY = ROOT / "profiles" / "pmc_fetch_write_bench_kernels.txt"
+PMC_ROW = "gate/up M=4096"
 
 
-def cpu_baseline(seconds_budget: float = 15.0) -> dict:
-    """The reference path on the host, restated by the oracle: both rank shards of the MLP on two threads,
-    torch CPU ops in bf16, then the sum (device_ids=['cpu','cpu'] in the reference). Bounded sample."""
+def measured_traffic_bytes():
+    """fetch + write MB per launch of the row `PMC_ROW` of the PMC summary, in bytes; None when there is no such row."""
+    try:
+        for line in PMC_SUMMARY.read_text().splitlines():
+            if PMC_ROW in line and line.lstrip().startswith("gemm_"):
+                cols = line.split(PMC_ROW)[1].split()
+                return (float(cols[1]) + float(cols[2])) * 1e6  # n, fetch MB, write MB, ...
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
+
+
+def cpu_baseline(tokens: int = 4096, seconds_budget: float = 12.0) -> dict:
+    """The reference path on the host, restated by the oracle, on bounded samples of the same workloads:
+    `value`: both rank shards of the MLP on two threads at the benchmark's token count, torch CPU ops in bf16, then the
+             sum (device_ids=['cpu','cpu'] in the reference: tensor_parallel.py:237-287);
+    `decode_m1`: the same step on one token;
+    `slicing`: state actions + the copy that installs the shard (shard.py:160) over the seven split tensors of one
+             Llama-2-7B decoder layer, every rank at W = 2, in GB/s read + written (32 such layers and the two
+             embedding-sized matrices make up the dict the GPU figure is quoted on)."""
+    import numpy as np
     import torch
 
     from oracle import shard_forward as ofw
+    from oracle import slicing as osl
 
-    m = 256
     g = torch.Generator().manual_seed(0)
     shards = []
     for _ in range(2):
         wg, wu = ((torch.randn(FFN_SHARD, D_MODEL, generator=g) * 0.02).bfloat16() for _ in range(2))
         wd = (torch.randn(D_MODEL, FFN_SHARD, generator=g) * 0.02).bfloat16()
         shards.append((wg, wu, wd))
-    x = torch.randn(m, D_MODEL, generator=torch.Generator().manual_seed(1)).bfloat16()
-    ofw.run_mlp_shards(x, shards, threads=True)  # warm
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        ofw.run_mlp_shards(x, shards, threads=True)
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt > seconds_budget:
-            break
+
+    def timed(m, budget):
+        x = torch.randn(m, D_MODEL, generator=torch.Generator().manual_seed(1)).bfloat16()
+        ofw.run_mlp_shards(x, shards, threads=True)  # warm
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            ofw.run_mlp_shards(x, shards, threads=True)
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > budget:
+                return reps, dt
+
+    reps, dt = timed(tokens, seconds_budget)
+    d_reps, d_dt = timed(1, 3.0)
+
+    # slicing: one decoder layer, both ranks
+    rng = np.random.default_rng(0)
+    layer = {name: rng.integers(0, 1 << 16, size=shape, dtype=np.uint16)
+             for name, shape in (("q", (4096, 4096)), ("k", (4096, 4096)), ("v", (4096, 4096)), ("o", (4096, 4096)),
+                                 ("gate", (11008, 4096)), ("up", (11008, 4096)), ("down", (4096, 11008)))}
+    world = 2
+
+    def slice_layer():
+        moved = 0
+        for r in range(world):
+            for name, t in layer.items():
+                if name in ("q", "k", "v"):
+                    out = osl.split_in_chunks(t, world, 0, 128, r)
+                elif name == "o":
+                    out = osl.split_in_chunks(t, world, 1, 128, r)
+                elif name == "down":
+                    out = osl.split(t, world, 1, r)
+                else:
+                    out = osl.split(t, world, 0, r)
+                moved += 2 * out.nbytes
+        return moved
+
+    slice_layer()
+    s_reps, s_bytes, t0 = 0, 0, time.perf_counter()
+    while time.perf_counter() - t0 < 4.0:
+        s_bytes += slice_layer()
+        s_reps += 1
+    s_dt = time.perf_counter() - t0
     return {
-        "value": m * reps / dt,
+        "value": tokens * reps / dt,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{reps} forwards of {m} tokens through both W=2 shards (2 threads) + sum, bf16 on host, {dt:.1f} s",
+        "sample": f"{reps} forwards of {tokens} tokens through both W=2 shards (2 threads) + sum, bf16 on host, {dt:.1f} s",
         "host_cpus": os.cpu_count(),
         "torch": torch.__version__,
+        "decode_m1": {"value": d_reps / d_dt, "unit": "tokens/s", "us_per_step": d_dt / d_reps * 1e6,
+                      "sample": f"{d_reps} forwards of 1 token, same shards and threads, {d_dt:.1f} s"},
+        "slicing": {"value": s_bytes / s_dt / 1e9, "unit": "GB/s read + written", "cores": 1,
+                    "sample": f"{s_reps} passes over the 7 split tensors of one Llama-2-7B decoder layer (404.8 MB), both ranks at W=2: "
+                              f"state action + contiguous copy in numpy, {s_dt:.1f} s; the full dict is 32 such layers + 2 x 262 MB"},
     }
 
 
@@ -133,8 +191,8 @@ def main() -> int:
     if mfma_bound:
         achieved = up_flops / (up_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES_M4096 if M == 4096 else None,
-                    "traffic_unit": "bytes per launch (L2<->fabric, rocprofv3 --pmc; algorithmic 168.8e6)",
+                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic_bytes() if M == 4096 else None,
+                    "traffic_unit": "bytes per launch (L2<->fabric, rocprofv3 --pmc, read from profiles/pmc_fetch_write_bench_kernels.txt; algorithmic 168.8e6)",
                     "kernel": "gemm_direct4_kernel<bf16, swiglu> (tpamd_swiglu_up)", "avg_launch_ms": up_ms,
                     "algorithmic_flops_per_launch": up_flops}
     else:
@@ -165,7 +223,7 @@ def main() -> int:
     if not args.no_extra:
         out["extra"] = extra_measurements(torch, _native, dev, sets, other)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(M)
     print(json.dumps(out), flush=True)
     return 0
 
@@ -257,6 +315,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     for m in (1, 16, 32, 64):
         extra[f"w8_decode_m{m}"] = w8_decode(torch, _native, dev, m)
     extra["attention_falcon40b_shard"] = attention_extra(torch, _native, dev)
+    extra["c4_decode_step"] = falcon_attention_decode_step(torch, _native, dev)
 
     from types import SimpleNamespace
 
@@ -336,6 +395,50 @@ def attention_extra(torch, _native, dev) -> dict:
     out["prefill_b8_s1024"] = {"us_per_call": us, "TFLOPs": flops / us / 1e6, "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS,
                                "algorithmic_flops": flops}
     return out
+
+
+def falcon_attention_decode_step(torch, _native, dev) -> dict:
+    """BASELINE config 4, decode, as one step of the rank-0 attention shard of a Falcon-40B-shape layer at W = 2: fused
+    QKV projection [4608 x 8192] on 8 new tokens, rotary embedding + hand-over to the rank-local cache (position 2047 of
+    2048), attention core over the 2048 cached positions (64 query heads on 4 key/value heads of 64), dense projection
+    [8192 x 4096] (the row-parallel partial). Algorithmic bytes: both weights and the key/value cache once; three weight
+    and cache sets are rotated."""
+    B, L, Hq, Hkv, D, d_model = 8, 2048, 64, 4, 64, 8192
+    per = Hq // Hkv
+    g = torch.Generator(device=dev).manual_seed(0)
+    n_sets = 3
+    sets = []
+    for _ in range(n_sets):
+        wqkv = (torch.randn((Hq + 2 * Hkv) * D, d_model, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        wdense = (torch.randn(d_model, Hq * D, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        kc = torch.randn(B, Hkv, L, D, device=dev, generator=g).to(torch.bfloat16)
+        vc = torch.randn(B, Hkv, L, D, device=dev, generator=g).to(torch.bfloat16)
+        sets.append((wqkv, wdense, kc, vc))
+    x = torch.randn(B, 1, d_model, device=dev, generator=g).to(torch.bfloat16)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
+    ang = torch.cat([(L - 1) * inv, (L - 1) * inv])[None, None, :]
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+    q_rot = torch.empty(B, Hq, 1, D, device=dev, dtype=torch.bfloat16)
+    attn = torch.empty(B, 1, Hq, D, device=dev, dtype=torch.bfloat16)
+
+    def fn(i):
+        wqkv, wdense, kc, vc = sets[i % n_sets]
+        fused = _native.linear(x, wqkv).view(B, 1, Hkv, per + 2, D)
+        _native.rope_append(fused[:, :, :, :per], fused[:, :, :, per], fused[:, :, :, per + 1], cos, sin, kc, vc, L - 1, q_out=q_rot)
+        _native.attention(q_rot, kc, vc, causal=True, out=attn)
+        return _native.linear(attn.view(B, Hq * D), wdense)
+
+    by = 2.0 * ((Hq + 2 * Hkv) * D * d_model + d_model * Hq * D) + 2.0 * B * Hkv * L * D * 2
+    us = _time_us(torch, fn, 10, 100)
+    entry = {"us_per_step": us, "tokens_per_s": B / us * 1e6, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
+             "algorithmic_bytes": by, "launch": "eager (one C-ABI call per kernel)",
+             "step": "qkv projection + rotary/cache append + attention core (keys split, 2 launches) + dense projection"}
+    try:
+        gus = _graph_us(torch, fn, per=24)
+        entry["graph"] = {"us_per_step": gus, "tokens_per_s": B / gus * 1e6, "GBps": by / gus / 1e3, "hbm_frac": by / gus / 1e3 / PEAK_HBM_GBS}
+    except Exception as e:  # noqa: BLE001 - the eager figure stands on its own
+        entry["graph"] = {"error": str(e)[:200]}
+    return entry
 
 
 def w8_decode(torch, _native, dev, m=1) -> dict:

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TPAMD_ABI_VERSION 2
+#define TPAMD_ABI_VERSION 3
 
 typedef enum tpamd_status {
     TPAMD_OK = 0,
@@ -224,6 +224,30 @@ int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void *wu_dev, v
 int tpamd_attention(const void *q_dev, const void *k_dev, const void *v_dev, void *out_dev, int64_t B, int64_t Hq,
                     int64_t Hkv, int64_t Sq, int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal,
                     int dtype, void *stream);
+
+/* Rotary position embedding of the new query / key rows and their hand-over to the rank-local key/value cache, in
+ * one launch: the step between a rank shard's QKV projection and tpamd_attention. In the reference the wrapped
+ * transformers attention module does this with torch ops on the rank's share of the heads
+ * (TensorParallelWrapper.forward, src/tensor_parallel/wrapper.py:69-72; Falcon-40B shard: fused query_key_value split
+ * by src/tensor_parallel/slicing_configs.py:430-432, head counts by :455-461), and the cache tensors it returns are
+ * routed per rank by select_kv_for_rank / gather_kv (src/tensor_parallel/aux_actions.py:7-15, used at
+ * slicing_configs.py:440,446). Here the cache is the rank's own preallocated buffer and the new rows are written in place.
+ *   q [B, S, Hq, D], k / v [B, S, Hkv, D]: views of the projection output (any batch / position / head strides, D
+ *   contiguous; Hq a multiple of Hkv, and query head h sits at (h / g) * "q group" + (h % g) * "q head" with
+ *   g = Hq / Hkv, so a fused output that interleaves each key/value head with its query heads is one view);
+ *   cos / sin [B or 1, S, D] in `dtype` (batch stride 0 when shared);
+ *   q_out [B, Hq, S, D] receives   q * cos + rotate_half(q) * sin,   rotate_half(x) = cat(-x[D/2:], x[:D/2]);
+ *   k_cache / v_cache [B, Hkv, cache_len, D]: positions pos0 .. pos0 + S - 1 receive the rotated k rows and the v rows.
+ *   Each of the two products and their sum is rounded to `dtype` (BF16 or F16), which is what the three torch ops of
+ *   transformers' apply_rotary_pos_emb produce on tensors of that dtype.
+ *   strides: 21 element strides, {q batch, q position, q head, k batch, k position, k head, v batch, v position, v head,
+ *   cos/sin batch, cos/sin position, q_out batch, q_out head, q_out position, k_cache batch, k_cache head, k_cache
+ *   position, v_cache batch, v_cache head, v_cache position, q group (= g * q head for a plain [B, S, Hq, D] view)}; all
+ *   multiples of 8, all pointers 16-byte aligned.
+ * D is 64 or 128 and the whole head is rotated (TPAMD_ERR_UNSUPPORTED otherwise). q_out may not overlap q. */
+int tpamd_rope_append(const void *q_dev, const void *k_dev, const void *v_dev, const void *cos_dev, const void *sin_dev,
+                      void *q_out_dev, void *k_cache_dev, void *v_cache_dev, int64_t B, int64_t S, int64_t Hq, int64_t Hkv,
+                      int64_t D, int64_t pos0, int64_t cache_len, const int64_t *strides, int dtype, void *stream);
 
 /* Weight-only int8 shard Linear with fp16/bf16 outlier columns:
  *   y[m,n] = act( scale[n] * sum_k x[m,k]*wq[n,k]  +  sum_j x[m,outlier_idx[j]] * w_out[n,j]  + bias[n] )

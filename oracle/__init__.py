@@ -14,6 +14,9 @@ Modules and the reference code each one follows:
                     (src/tensor_parallel/wrapper.py:69-72, tensor_parallel.py:237-287), torch on CPU
   attention.py      the attention core the wrapped module runs on a rank's heads (softmax(q k^T) v, grouped-query,
                     causal aligned to the end of the keys), float64; the reference has no attention code of its own
+  rope.py           rotary embedding of the new query / key rows and their hand-over to the rank-local cache, in the
+                    arithmetic of the wrapped transformers module (the reference only routes the cache tensors:
+                    src/tensor_parallel/aux_actions.py:7-15)
   sharding.py       flat per-rank shards of the replicated parameters and their recombination
                     (src/tensor_parallel/sharding.py:96-180)
   quant.py          int8 weight-only quantisation with outlier columns - NOT in the reference: parity
@@ -29,6 +32,8 @@ How each function is pinned (tests/test_oracle_*.py):
                both in fp64
   attention    torch's CPU scaled_dot_product_attention where it covers the case, explicit loops on tiny inputs for
                grouped heads and Sq < Skv causal, rows of probabilities sum to one, a single visible key returns its value
+  rope         transformers' apply_rotary_pos_emb bit for bit (bf16, fp16, fp32), the complex-rotation closed form in
+               fp64, norm preservation, identity at position 0
   sharding     combine(make(x)) == x on ragged sizes, equal flat lengths, the parameter counts asserted by the
                reference's own test (tests/test_basic.py:110-135)
   quant        dequantised weights within scale/2 of the originals; fp64 matmul of the definition

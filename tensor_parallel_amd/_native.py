@@ -35,9 +35,10 @@ EXPORTS = (
     "tpamd_swiglu_up",
     "tpamd_linear_w8",
     "tpamd_attention",
+    "tpamd_rope_append",
 )
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 BF16, F16, F32 = 0, 1, 2
 ACCUM_STEPWISE, ACCUM_F32 = 0, 1
@@ -115,6 +116,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_swiglu_up.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
     lib.tpamd_attention.restype = ci
     lib.tpamd_attention.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, c.POINTER(i64), c.c_float, ci, ci, vp]
+    lib.tpamd_rope_append.restype = ci
+    lib.tpamd_rope_append.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, c.POINTER(i64), ci, vp]
     lib.tpamd_linear_w8.restype = ci
     lib.tpamd_linear_w8.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, i64, i64, i64, i64, i64, i64, i64, ci, ci, vp]
 
@@ -468,6 +471,60 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional
             "tpamd_attention",
         )
     return out
+
+
+def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                k_cache: torch.Tensor, v_cache: torch.Tensor, pos0: int, q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotary embedding of the new rows and their hand-over to the rank-local cache, one launch.
+    q [B, S, Hq, D] or [B, S, Hkv, Hq / Hkv, D] (the query heads of each key/value head, as a fused projection that
+    interleaves them with their key and value lays them out), k / v [B, S, Hkv, D] (all views of a projection output),
+    cos / sin [B or 1, S, D];
+    k_cache / v_cache [B, Hkv, L, D] are written in place at positions pos0 .. pos0 + S - 1 (rotated k, v);
+    returns the rotated q as [B, Hq, S, D], the layout `attention` takes."""
+    require_device(q, "rope_append")
+    if not (q.dtype == k.dtype == v.dtype == cos.dtype == sin.dtype == k_cache.dtype == v_cache.dtype) or q.dtype not in (
+            torch.bfloat16, torch.float16):
+        raise TypeError("rope_append: every tensor must share bfloat16 or float16")
+    if q.dim() not in (4, 5) or k.dim() != 4 or v.shape != k.shape or q.shape[:2] != k.shape[:2] or q.shape[-1] != k.shape[3] or (
+            q.dim() == 5 and q.shape[2] != k.shape[2]):
+        raise ValueError(f"rope_append: shapes q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit")
+    B, S, Hkv, D = k.shape
+    Hq = q.shape[2] if q.dim() == 4 else q.shape[2] * q.shape[3]
+    if Hq % Hkv:
+        raise ValueError(f"rope_append: {Hq} query heads over {Hkv} key/value heads")
+    q_head, q_group = (q.stride(2), q.stride(2) * (Hq // Hkv)) if q.dim() == 4 else (q.stride(3), q.stride(2))
+    if cos.dim() == 2:
+        cos, sin = cos.unsqueeze(0), sin.unsqueeze(0)
+    if cos.shape != sin.shape or cos.dim() != 3 or cos.shape[0] not in (1, B) or cos.shape[1:] != (S, D):
+        raise ValueError(f"rope_append: cos / sin must be [{B} or 1, {S}, {D}], got {tuple(cos.shape)} / {tuple(sin.shape)}")
+    if k_cache.dim() != 4 or v_cache.shape != k_cache.shape or k_cache.shape[0] != B or k_cache.shape[1] != Hkv or k_cache.shape[3] != D:
+        raise ValueError(f"rope_append: caches must be [{B}, {Hkv}, L, {D}], got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    for name, t in (("k", k), ("v", v), ("cos", cos), ("sin", sin), ("k_cache", k_cache), ("v_cache", v_cache)):
+        if t.device != q.device:
+            raise ValueError(f"rope_append: q is on {q.device}, {name} on {t.device}")
+        if t.stride(-1) != 1:
+            raise ValueError(f"rope_append: {name} must have contiguous rows")
+    if q.stride(-1) != 1:
+        raise ValueError("rope_append: q must have contiguous rows")
+    if sin.stride() != cos.stride():
+        sin = sin.contiguous()
+        cos = cos.contiguous()
+    if q_out is None:
+        q_out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
+    elif q_out.shape != (B, Hq, S, D) or q_out.dtype != q.dtype or q_out.device != q.device or q_out.stride(3) != 1:
+        raise ValueError(f"rope_append: q_out must be a [{B}, {Hq}, {S}, {D}] {q.dtype} tensor on {q.device} with contiguous rows")
+    strides = (ctypes.c_int64 * 21)(q.stride(0), q.stride(1), q_head, k.stride(0), k.stride(1), k.stride(2),
+                                    v.stride(0), v.stride(1), v.stride(2), cos.stride(0) if cos.shape[0] > 1 else 0, cos.stride(1),
+                                    q_out.stride(0), q_out.stride(1), q_out.stride(2), k_cache.stride(0), k_cache.stride(1),
+                                    k_cache.stride(2), v_cache.stride(0), v_cache.stride(1), v_cache.stride(2), q_group)
+    with _on_device(q.device):
+        _check(
+            lib().tpamd_rope_append(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(), q_out.data_ptr(),
+                                    k_cache.data_ptr(), v_cache.data_ptr(), B, S, Hq, Hkv, D, int(pos0), k_cache.shape[2], strides,
+                                    dtype_code(q.dtype), ctypes.c_void_p(current_stream_ptr(q.device))),
+            "tpamd_rope_append",
+        )
+    return q_out
 
 
 def linear_w8(x: torch.Tensor, wq: torch.Tensor, scale_: torch.Tensor, outlier_idx: Optional[torch.Tensor],

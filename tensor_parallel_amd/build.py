@@ -14,7 +14,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 OUT_DIR = PKG / "_lib"
 LIB = OUT_DIR / "libtpamd.so"
-SOURCES = ["api.hip", "runtime.hip", "noalloc.hip", "slice.hip", "reduce.hip", "gemm.hip", "skinny.hip", "attention.hip"]
+SOURCES = ["api.hip", "runtime.hip", "noalloc.hip", "slice.hip", "reduce.hip", "gemm.hip", "skinny.hip", "attention.hip", "rope.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
