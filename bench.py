@@ -316,6 +316,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
         extra[f"w8_decode_m{m}"] = w8_decode(torch, _native, dev, m)
     extra["attention_falcon40b_shard"] = attention_extra(torch, _native, dev)
     extra["c4_decode_step"] = falcon_attention_decode_step(torch, _native, dev)
+    extra.update(api_level_extras(torch, dev))
 
     from types import SimpleNamespace
 
@@ -439,6 +440,70 @@ def falcon_attention_decode_step(torch, _native, dev) -> dict:
     except Exception as e:  # noqa: BLE001 - the eager figure stands on its own
         entry["graph"] = {"error": str(e)[:200]}
     return entry
+
+
+def api_level_extras(torch, dev) -> dict:
+    """Two figures through the package's Python surface (tp.TensorParallel / tp.tensor_parallel), host orchestration
+    included, with BOTH rank shards on this one GPU:
+    c2_tp_module_m4096: the Llama-7B MLP (d 4096, ffn 11008, bf16) split by the Llama rules at W = 2, 4096 tokens per
+        forward: each rank's fused gate/up GEMM and down projection, the second rank's down projection adding the first
+        rank's partial in its epilogue (no reduction launch), and the copy that gives each rank its own result;
+    c1_opt125m: BASELINE config 1, OPT-125m architecture in fp32 with N(0, 0.02) weights, batch 2 x 64 tokens, W = 2
+        through tp.tensor_parallel: tokens/s = 128 / forward latency (for information; the step is launch-bound)."""
+    from types import SimpleNamespace
+
+    from torch import nn
+
+    import tensor_parallel_amd as tp
+    from tensor_parallel_amd.slicing_configs import get_llama_config
+
+    out = {}
+
+    class MLP(nn.Module):
+        def __init__(self, d, f):
+            super().__init__()
+            self.gate_proj, self.up_proj, self.down_proj = nn.Linear(d, f, bias=False), nn.Linear(d, f, bias=False), nn.Linear(f, d, bias=False)
+            self.act_fn = nn.SiLU()
+
+        def forward(self, x):
+            return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+    class Block(nn.Module):
+        def __init__(self, d, f):
+            super().__init__()
+            self.mlp = MLP(d, f)
+
+        def forward(self, x):
+            return self.mlp(x)
+
+    with torch.no_grad():
+        with torch.device(dev):
+            block = Block(D_MODEL, 2 * FFN_SHARD).to(torch.bfloat16)
+        for p in block.parameters():
+            p.normal_(0.0, 0.02)
+        cfg = get_llama_config(SimpleNamespace(model_type="llama", hidden_size=D_MODEL, num_attention_heads=32, num_key_value_heads=32), [dev, dev])
+        model_tp = tp.TensorParallel(block, [dev, dev], tensor_parallel_config=cfg, sharded=False)
+        del block
+        x = torch.randn(4096, D_MODEL, device=dev).to(torch.bfloat16)
+        us = _time_us(torch, lambda i: model_tp(x), 20, 30)
+        flops = 2 * 6.0 * 4096 * D_MODEL * FFN_SHARD
+        out["c2_tp_module_m4096"] = {"us_per_forward": us, "tokens_per_s": 4096 / us * 1e6, "TFLOPs": flops / us / 1e6,
+                                     "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS, "algorithmic_flops": flops,
+                                     "what": "tp.TensorParallel forward, both W=2 rank shards on this GPU (2 rank threads), sum folded into the second rank's down projection"}
+        del model_tp, x
+
+        from transformers import OPTConfig, OPTForCausalLM
+
+        torch.manual_seed(0)
+        model = OPTForCausalLM(OPTConfig()).eval()
+        for p in model.parameters():
+            p.normal_(0.0, 0.02)
+        opt_tp = tp.tensor_parallel(model, [dev, dev])
+        ids = torch.randint(0, 50272, (2, 64), generator=torch.Generator().manual_seed(1)).to(dev)
+        us = _time_us(torch, lambda i: opt_tp(input_ids=ids, use_cache=False).logits, 5, 20)
+        out["c1_opt125m"] = {"us_per_forward": us, "tokens_per_s": 128 / us * 1e6, "dtype": "f32",
+                             "what": "tp.tensor_parallel(OPT-125m, W=2) forward of 2 x 64 tokens, both rank shards on this GPU, host orchestration included"}
+    return out
 
 
 def w8_decode(torch, _native, dev, m=1) -> dict:

@@ -11,6 +11,7 @@ before the reduction by the stream itself; the host-side barrier only makes sure
 """
 from __future__ import annotations
 
+import os
 import threading
 from typing import Any, Callable, List, Optional
 
@@ -31,6 +32,48 @@ _turn = threading.local()
 
 def set_turn_lock(lock: Optional[threading.Lock]) -> None:
     _turn.lock = lock
+
+
+def turn_lock() -> Optional[threading.Lock]:
+    return getattr(_turn, "lock", None)
+
+
+# ---- the sum folded into the last Linear of a row-parallel module -------------------------------------------------
+# A module whose output rule is "sum" usually ends in its row-parallel Linear (attention output projection, MLP down
+# projection). The rank that reaches that Linear while the partials of the other ranks are already waiting in the op
+# can add them in the GEMM's epilogue (`tpamd_linear_add`) instead of leaving a separate M x N pass to the reduction
+# kernel. A wrapper with such a rule publishes a SumContext for its thread while its module runs; shard Linears
+# consult it (shard_modules.linear_in_context); the op learns from it what the value it is handed already contains.
+FUSE_SUM = os.environ.get("TPAMD_FUSE_SUM", "1") != "0"
+_contexts = threading.local()
+
+
+class SumContext:
+    """One call of a wrapped module whose output 0 goes to `op`, on one rank thread."""
+
+    __slots__ = ("op", "rank", "owner", "last_linear", "last_out", "calls", "fused_out", "fused_mask")
+
+    def __init__(self, op: "DeviceAllReduce", rank: int, owner: Any):
+        self.op, self.rank, self.owner = op, rank, owner
+        self.last_linear = self.last_out = self.fused_out = None
+        self.calls: dict = {}
+        self.fused_mask = 0
+
+
+def push_sum_context(ctx: SumContext) -> None:
+    stack = getattr(_contexts, "stack", None)
+    if stack is None:
+        stack = _contexts.stack = []
+    stack.append(ctx)
+
+
+def pop_sum_context() -> None:
+    _contexts.stack.pop()
+
+
+def current_sum_context() -> Optional[SumContext]:
+    stack = getattr(_contexts, "stack", None)
+    return stack[-1] if stack else None
 
 
 def _rendezvous(barrier: threading.Barrier, timeout: float) -> None:
@@ -92,14 +135,66 @@ class CollectiveOperation(CollectiveOpetationBase):
 class DeviceAllReduce(CollectiveOperation):
     """out = p_0 + p_1 + ... + p_{W-1}, delivered to every rank. `accum` picks the arithmetic
     (`_native.ACCUM_STEPWISE`: the running sum is rounded to the tensor dtype after each add, which is what
-    the reference's `sum([...])` of same-dtype tensors does, cross_device_ops.py:49, taken in rank order)."""
+    the reference's `sum([...])` of same-dtype tensors does, cross_device_ops.py:49, taken in rank order).
+
+    A value handed in may already hold the sum over several ranks (see SumContext): rank r's Linear added what
+    `addend_for(r)` gave it. `_masks[r]` records which ranks value r covers; the reduction then adds only what is
+    still missing, in rank order, and launches nothing when one value covers every rank."""
 
     def __init__(self, world_size: int, accum: int = _native.ACCUM_STEPWISE, timeout: float = RENDEZVOUS_TIMEOUT_S):
         super().__init__(world_size, self._reduce, timeout)
         self.accum = accum
+        self._masks: List[int] = [0] * world_size
+
+    @property
+    def fusable(self) -> bool:
+        return FUSE_SUM and self.accum == _native.ACCUM_STEPWISE and self.world_size > 1
+
+    def addend_for(self, rank: int):
+        """(tensor, ranks it covers as a bit mask) that rank `rank`'s last Linear may add to its own partial so that
+        the result is a step of the rank-ordered sum, or None. Two ranks: whatever the other rank has handed in (a sum
+        of two is the same in either order). More ranks: the running sum over ranks 0 .. rank-1, once rank-1 has
+        handed it in. Only for rank threads that take turns on one device (the waiting value is then complete and
+        visible)."""
+        if not self.fusable or turn_lock() is None:
+            return None
+        if self.world_size == 2:
+            other = 1 - rank
+            if self._inputs[other] is not None and self._masks[other] == 1 << other:
+                return self._inputs[other], 1 << other
+            return None
+        below = (1 << rank) - 1
+        if rank > 0 and self._inputs[rank - 1] is not None and self._masks[rank - 1] == below:
+            return self._inputs[rank - 1], below
+        return None
+
+    def __call__(self, x: Any, rank: int):
+        mask = 1 << rank
+        ctx = current_sum_context()
+        if ctx is not None and ctx.op is self and ctx.rank == rank:
+            linear = ctx.last_linear
+            if ctx.fused_out is not None:
+                if x is not ctx.fused_out:
+                    raise RuntimeError(
+                        "tensor_parallel_amd: a row-parallel Linear added the other ranks' partial sums in its epilogue, but the "
+                        "module then returned a different tensor; set TPAMD_FUSE_SUM=0 to keep the sum in its own kernel")
+                mask |= ctx.fused_mask
+            elif linear is not None:
+                # the Linear that produced exactly the value handed in, called once: next time it may add the waiting partials
+                feeds = x is ctx.last_out and ctx.calls.get(id(linear)) == 1
+                linear.__dict__["_tp_feeds_sum"] = ctx.owner if feeds else None
+        self._masks[rank] = mask
+        try:
+            return super().__call__(x, rank)
+        finally:
+            self._masks[rank] = 0
 
     def _reduce(self, *parts: torch.Tensor):
-        out = _native.reduce_partials([p.detach() for p in parts], accum=self.accum)
+        masks = list(self._masks)
+        widest = max(range(self.world_size), key=lambda r: bin(masks[r]).count("1"))
+        todo = [parts[widest]] + [parts[r] for r in range(self.world_size) if not masks[widest] >> r & 1]
+        # the widest value is a running sum from rank 0 on (or covers both of two ranks); what it lacks are higher ranks
+        out = todo[0].detach() if len(todo) == 1 else _native.reduce_partials([p.detach() for p in todo], accum=self.accum)
         # each rank continues with a tensor of its own: later in-place ops on one rank must not leak
         return [_guard(o, *parts) for o in [out] + [out.clone() for _ in range(self.world_size - 1)]]
 

@@ -1254,6 +1254,153 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmParams p) {
     }
 }
 
+// ---- fp32 on the matrix pipe: v_mfma_f32_32x32x2_f32 -------------------------------------------------------------
+// y = act(x . w^T + bias) (+ addend) for fp32 operands whose rows are 16-byte aligned (K, leading dimensions and N
+// multiples of 4). Same staging as gemm_kernel: a K tile is 128 bytes of every row (32 floats here), 16-byte chunks
+// prefetched into registers while the current tile is multiplied, two LDS stages, one barrier per tile. The
+// instruction multiplies a 32 x 2 by a 2 x 32 panel; which two k a step pairs up is free as long as both operands
+// agree, so lane (row r, half h) uses k = 16 h + s in step s: its 16 operands of a K tile are 64 contiguous bytes of
+// the staged row (four 16-byte reads). w is the first operand, so a lane holds 4 consecutive output columns of one
+// row per group of 4 accumulator registers: one 16-byte store. Products and sums are fp32 throughout.
+constexpr int BK32 = 32;  // floats per stage row
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmParams p) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    constexpr int XC = BM * 8 / NT, WC = BN * 8 / NT;
+    constexpr int STAGE = (BM + BN) * LDS_ROW;
+    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile/threads mismatch");
+    extern __shared__ __align__(16) char smem[];
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    const int ld_chunk = tid & 7, ld_row = tid >> 3;
+    const char *xg[XC];
+    const char *wg[WC];
+#pragma unroll
+    for (int i = 0; i < XC; ++i) {
+        int r = m0 + ld_row + i * (NT / 8);
+        r = r < p.M ? r : p.M - 1;  // rows past the end repeat the last one; their outputs are not stored
+        xg[i] = p.x + (static_cast<int64_t>(r) * p.ldx + ld_chunk * 4) * 4;
+    }
+#pragma unroll
+    for (int i = 0; i < WC; ++i) {
+        int r = n0 + ld_row + i * (NT / 8);
+        r = r < p.N ? r : p.N - 1;
+        wg[i] = p.w + (static_cast<int64_t>(r) * p.ldw + ld_chunk * 4) * 4;
+    }
+    const int st_off = ld_row * LDS_ROW + ld_chunk * 16;
+    uint4 xr[XC], wr[WC];
+    auto load_global = [&](int kt) {
+        const bool ok = kt * BK32 + ld_chunk * 4 < p.K;  // K is a multiple of 4: a chunk is entirely inside or outside
+        // past the end of K the row's first chunk is fetched instead (a load, not a branch); x is zeroed when stored
+        const int64_t off = ok ? static_cast<int64_t>(kt) * BK32 * 4 : -static_cast<int64_t>(ld_chunk) * 16;
+#pragma unroll
+        for (int i = 0; i < XC; ++i) xr[i] = *reinterpret_cast<const uint4 *>(xg[i] + off);
+#pragma unroll
+        for (int i = 0; i < WC; ++i) wr[i] = *reinterpret_cast<const uint4 *>(wg[i] + off);
+    };
+    auto store_lds = [&](int stage, int kt) {
+        char *xs = smem + stage * STAGE;
+        char *ws = xs + BM * LDS_ROW;
+        const bool ok = kt * BK32 + ld_chunk * 4 < p.K;
+#pragma unroll
+        for (int i = 0; i < XC; ++i)
+            *reinterpret_cast<uint4 *>(xs + st_off + i * (NT / 8) * LDS_ROW) = make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
+#pragma unroll
+        for (int i = 0; i < WC; ++i)  // w past the end of K may be anything finite or not: it must not meet a NaN-free zero
+            *reinterpret_cast<uint4 *>(ws + st_off + i * (NT / 8) * LDS_ROW) = make_uint4(ok ? wr[i].x : 0u, ok ? wr[i].y : 0u, ok ? wr[i].z : 0u, ok ? wr[i].w : 0u);
+    };
+    int x_rd[TM], w_rd[TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t) x_rd[t] = (wm * (BM / WAVES_M) + t * 32 + l32) * LDS_ROW + lhi * 64;
+#pragma unroll
+    for (int t = 0; t < TN; ++t) w_rd[t] = BM * LDS_ROW + (wn * (BN / WAVES_N) + t * 32 + l32) * LDS_ROW + lhi * 64;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
+
+    const int KT = (p.K + BK32 - 1) / BK32;
+    load_global(0);
+    store_lds(0, 0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_global(kt + 1);
+        const char *stage = smem + (kt & 1) * STAGE;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {  // 4 floats of the lane's 16 at a time
+            f32x4 xf[TM], wf[TN];
+#pragma unroll
+            for (int t = 0; t < TM; ++t) xf[t] = *reinterpret_cast<const f32x4 *>(stage + x_rd[t] + q * 16);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) wf[t] = *reinterpret_cast<const f32x4 *>(stage + w_rd[t] + q * 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int a = 0; a < TM; ++a)
+#pragma unroll
+                    for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[b][j], xf[a][j], acc[a][b], 0, 0, 0);
+        }
+        if (more) store_lds((kt + 1) & 1, kt + 1);
+        __syncthreads();
+    }
+    // D[n_local][m_local]: lane -> m_local = l32, register i -> n_local = 8 * (i / 4) + 4 * lhi + i % 4
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+        const int m = m0 + wm * (BM / WAVES_M) + a * 32 + l32;
+        if (m >= p.M) continue;
+        float *yrow = reinterpret_cast<float *>(p.y) + static_cast<int64_t>(m) * p.ldy;
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = n0 + wn * (BN / WAVES_N) + b * 32 + q * 8 + lhi * 4;
+                if (n >= p.N) continue;  // N is a multiple of 4: the group of 4 is all in or all out
+                f32x4 v = {acc[a][b][q * 4], acc[a][b][q * 4 + 1], acc[a][b][q * 4 + 2], acc[a][b][q * 4 + 3]};
+                if (p.bias) v += *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.bias) + n);
+                if (p.act == TPAMD_ACT_GELU) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
+                }
+                if (p.addend != nullptr) v += *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.addend) + static_cast<int64_t>(m) * p.ldadd + n);
+                *reinterpret_cast<f32x4 *>(yrow + n) = v;
+            }
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_gemm_f32(GemmParams p, hipStream_t s) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int LDS = 2 * (BM + BN) * LDS_ROW;
+    auto kern = gemm_f32_kernel<BM, BN, WAVES_M, WAVES_N>;
+    static thread_local int configured_dev = -1;  // per instantiation and host thread
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        configured_dev = dev;
+    }
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t blocks = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    TPAMD_REQUIRE(blocks < (1ll << 31), "gemm: too many tiles");
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(NT), LDS, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 template <int DT, int MODE, int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_gemm(GemmParams p, hipStream_t s) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -1484,6 +1631,17 @@ int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias
     p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
     p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ldadd = ldadd;
     p.act = act;
+    if (dtype == TPAMD_F32 && !swiglu && K >= 4 && K % 4 == 0 && N % 4 == 0 && ldx % 4 == 0 && ldw % 4 == 0 && ldy % 4 == 0 &&
+        aligned(x, 16) && aligned(w, 16) && aligned(y, 16) && (!bias || aligned(bias, 16)) &&
+        (!addend || (aligned(addend, 16) && ldadd % 4 == 0))) {
+        // fp32 rows that 16-byte accesses can take: the matrix pipe. 128 x 128 tiles once they fill the CUs, else 64 x 64.
+        int dev = 0, cus = 256;
+        TPAMD_HIP(hipGetDevice(&dev));
+        if (int rc = device_cus(dev, &cus); rc != TPAMD_OK) return rc;
+        const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+        if (tiles128 >= cus) return launch_gemm_f32<128, 128, 2, 2>(p, s);
+        return launch_gemm_f32<64, 64, 2, 2>(p, s);
+    }
     if (dtype == TPAMD_F32 || generic) return generic_dispatch(p, dtype, swiglu, s);
     return dtype == TPAMD_BF16 ? gemm_large<TPAMD_BF16>(p, swiglu, s) : gemm_large<TPAMD_F16>(p, swiglu, s);
 }

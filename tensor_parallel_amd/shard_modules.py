@@ -41,12 +41,41 @@ def _guard(out: torch.Tensor, *inputs: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def linear_in_context(module: nn.Module, x: torch.Tensor, w: torch.Tensor, bias) -> torch.Tensor:
+    """`tpamd_linear` for a shard's Linear. Inside a wrapped module whose output goes to a "sum" rule
+    (collectives.SumContext) the Linear that was seen to produce that output adds the partial sums already waiting in
+    the reduction, in its epilogue (`tpamd_linear_add`): the product rounded to the dtype, then one rounded add, which
+    is the same arithmetic as the reduction kernel's step."""
+    from .collectives import current_sum_context
+
+    ctx = current_sum_context()
+    b = None if bias is None else bias.detach()
+    if ctx is None:
+        return _guard(_native.linear(x.detach(), w.detach(), b), x, w, bias)
+    key = id(module)
+    ctx.calls[key] = ctx.calls.get(key, 0) + 1
+    addend = None
+    if module.__dict__.get("_tp_feeds_sum") is ctx.owner and ctx.owner is not None:
+        if ctx.fused_out is not None:
+            raise RuntimeError("tensor_parallel_amd: the Linear that feeds a \"sum\" rule ran twice in one call of its module "
+                               "after adding the waiting partial sums; set TPAMD_FUSE_SUM=0")
+        waiting = ctx.op.addend_for(ctx.rank)
+        if waiting is not None:
+            t, mask = waiting
+            if t.dtype == x.dtype and t.device == x.device and t.shape == (*x.shape[:-1], w.shape[0]):
+                addend, ctx.fused_mask = t.detach(), mask
+    out = _guard(_native.linear(x.detach(), w.detach(), b, addend=addend), x, w, bias)
+    if addend is not None:
+        ctx.fused_out = out
+    ctx.last_linear, ctx.last_out = module, out
+    return out
+
+
 class ShardLinear(nn.Linear):
     """`nn.Linear` whose forward is `tpamd_linear` on the shard's (sliced) weight."""
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:  # noqa: A002
-        out = _native.linear(input.detach(), self.weight.detach(), None if self.bias is None else self.bias.detach())
-        return _guard(out, input, self.weight, self.bias)
+        return linear_in_context(self, input, self.weight, self.bias)
 
 
 def is_conv1d(module: nn.Module) -> bool:
@@ -60,9 +89,7 @@ def _conv1d_forward(self, x: torch.Tensor) -> torch.Tensor:
     if not is_k_major(w):  # a weight assigned after the shard was built: lay it out for the kernel, once
         with torch.no_grad():
             w.data = _native.transpose_regions(w.data.contiguous(), [(0, w.shape[1])]).t()
-    bias = getattr(self, "bias", None)
-    out = _native.linear(x.detach(), w.detach().t(), None if bias is None else bias.detach())
-    return _guard(out, x, w, bias)
+    return linear_in_context(self, x, w.t(), getattr(self, "bias", None))
 
 
 _conv1d_classes: dict = {}

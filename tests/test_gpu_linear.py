@@ -67,6 +67,27 @@ def test_linear_fp32(M, N, K):
     torch.testing.assert_close(got, want, rtol=RTOL_F32, atol=RTOL_F32 * 0.02 * math.sqrt(K))
 
 
+@pytest.mark.parametrize("M,N,K", [(130, 72, 132), (64, 4, 4), (1000, 4100, 72), (2048, 2048, 100), (128, 50272, 384)])
+def test_linear_fp32_on_the_matrix_pipe(M, N, K):
+    """fp32 operands whose rows take 16-byte accesses run on v_mfma_f32_32x32x2_f32: 64 x 64 tiles while those do not
+    fill the CUs, 128 x 128 tiles above (the third and fourth shapes), ragged tiles in M, N and K, a row-parallel
+    slice of x (leading dimension above K), bias, GELU and the addend of the fused partial sum. The last shape is the
+    tied head of BASELINE config 1 (OPT-125m at W = 2: 128 tokens, K = 384 of 768 columns)."""
+    full = rnd((M, K + 8), 1, 1.0, torch.float32)
+    w, b = rnd((N, K), 0, 0.02, torch.float32), rnd((N,), 2, 0.1, torch.float32)
+    other = rnd((M, N), 3, 0.5, torch.float32)
+    xd = full.to(DEV)[:, 4:4 + K]  # rows 16-byte aligned, not contiguous
+    x = full[:, 4:4 + K]
+    atol = RTOL_F32 * 0.02 * math.sqrt(K)
+    want = F.linear(x.double(), w.double(), b.double())
+    got = _native.linear(xd, w.to(DEV), b.to(DEV)).cpu()
+    torch.testing.assert_close(got, want.float(), rtol=RTOL_F32, atol=atol)
+    got = _native.linear(xd, w.to(DEV), b.to(DEV), addend=other.to(DEV)).cpu()
+    torch.testing.assert_close(got, (want + other.double()).float(), rtol=RTOL_F32, atol=atol)
+    got = _native.linear(xd, w.to(DEV), None, act=_native.ACT_GELU).cpu()
+    torch.testing.assert_close(got, F.gelu(F.linear(x.double(), w.double())).float(), rtol=RTOL_F32, atol=atol)
+
+
 def test_gelu_epilogue_and_argument_errors():
     x, w = rnd((40, 64), 1, 1.0, torch.float16), rnd((64, 64), 0, 0.1, torch.float16)
     for M in (8, 40):
