@@ -71,11 +71,18 @@ typedef enum tpamd_act {
 int tpamd_abi_version(void);
 const char *tpamd_last_error(void);
 /* Reads the TPAMD_* environment variables again (they are read once at load time otherwise). For tests and
- * experiments that force a kernel variant; no counterpart in the reference. */
+ * experiments that force a kernel variant; no counterpart in the reference. Not synchronised: call it while no other
+ * thread is inside the library. */
 void tpamd_tuning_reload(void);
 /* The K-split scratch buffer that work on `stream` of the current device uses: *ptr_out = NULL and *bytes_out = 0
  * while the stream has none. Diagnostic; no counterpart in the reference. */
 int tpamd_scratch_query(void *stream, void **ptr_out, uint64_t *bytes_out);
+/* Gives back the scratch buffer of `stream` on the current device (no-op when it has none): call it before destroying a
+ * stream that ran K-split work, with none of that work captured in a graph that will still be replayed. The stream is
+ * synchronised, the buffer freed, and its slot can serve another stream. Without it a buffer lives until the process
+ * ends: at most 33 per device (32 streams and the spare), 64 MiB each on a 256-CU part, i.e. up to 2.1 GiB per device for
+ * a process that keeps creating streams. No counterpart in the reference. */
+int tpamd_scratch_release(void *stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Slicing engine.
@@ -189,9 +196,11 @@ int tpamd_linear_add(const void *x_dev, const void *w_dev, const void *bias_dev,
  * harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, same kernels and the same
  * result, bit for bit, as tpamd_linear; the call allocates nothing (no hipMalloc, no hipFree), also at its first use
  * and under stream capture. Where tpamd_linear would put the fp32 partial tiles of a K split into its stream's
- * scratch buffer, this entry point puts them into a fixed array of tpamd_noalloc_scratch_bytes() = 32 MiB that every
- * GPU the library is loaded on holds until the process ends. A shape whose K split needs more (the message names
- * the size) is refused with TPAMD_ERR_UNSUPPORTED and nothing is launched; tpamd_linear takes such shapes.
+ * scratch buffer, this entry point puts them into a fixed array of tpamd_noalloc_scratch_bytes() = 64 MiB that every
+ * GPU the library is loaded on holds until the process ends: the size of a stream's buffer on a 256-CU part, so every
+ * K split the library picks by itself there fits. A K split that needs more (a part with more CUs, a split forced
+ * through the TPAMD_* variables; the message names the size) is refused with TPAMD_ERR_UNSUPPORTED and nothing is
+ * launched; tpamd_linear takes such shapes.
  * All calls on one GPU share that GPU's array: calls on the same stream are ordered by it, calls that overlap on
  * different streams of one GPU race on the partial tiles and must be ordered by the caller. */
 int tpamd_linear_noalloc(const void *x_dev, const void *w_dev, const void *bias_dev, void *y_dev, int64_t M, int64_t N,

@@ -28,6 +28,7 @@ EXPORTS = (
     "tpamd_reduce_partials",
     "tpamd_tuning_reload",
     "tpamd_scratch_query",
+    "tpamd_scratch_release",
     "tpamd_linear",
     "tpamd_linear_add",
     "tpamd_linear_noalloc",
@@ -112,6 +113,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_tuning_reload.argtypes = []
     lib.tpamd_scratch_query.restype = ci
     lib.tpamd_scratch_query.argtypes = [vp, c.POINTER(vp), c.POINTER(u64)]
+    lib.tpamd_scratch_release.restype = ci
+    lib.tpamd_scratch_release.argtypes = [vp]
     lib.tpamd_swiglu_up.restype = ci
     lib.tpamd_swiglu_up.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
     lib.tpamd_attention.restype = ci
@@ -370,6 +373,14 @@ def scratch_of_stream(device: torch.device, stream_ptr: Optional[int] = None) ->
             stream_ptr = current_stream_ptr(device)
         _check(lib().tpamd_scratch_query(ctypes.c_void_p(stream_ptr), ctypes.byref(ptr), ctypes.byref(nbytes)), "tpamd_scratch_query")
     return ptr.value, int(nbytes.value)
+
+
+def release_scratch(device: torch.device, stream_ptr: Optional[int] = None) -> None:
+    """Free the K-split scratch buffer of a stream that is about to be retired (it is synchronised first)."""
+    with _on_device(device):
+        if stream_ptr is None:
+            stream_ptr = current_stream_ptr(device)
+        _check(lib().tpamd_scratch_release(ctypes.c_void_p(stream_ptr)), "tpamd_scratch_release")
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, act: int = ACT_NONE,

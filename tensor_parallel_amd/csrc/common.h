@@ -67,7 +67,8 @@ std::mutex &splitk_mutex();
 int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out);
 // While one of these lives on a host thread, splitk_scratch() on that thread hands out the library's fixed array and
 // allocates nothing.
-constexpr size_t TPAMD_NOALLOC_SCRATCH_BYTES = static_cast<size_t>(32) << 20;
+// 64 MiB: what a stream's buffer holds on a 256-CU part (4 * CUs * 64 KiB), so every K split the cost models pick there fits.
+constexpr size_t TPAMD_NOALLOC_SCRATCH_BYTES = static_cast<size_t>(64) << 20;
 bool static_scratch_active();
 int static_scratch(int dev, size_t need, void **out);
 struct StaticScratchScope {

@@ -147,6 +147,29 @@ using namespace tpamd;
 
 extern "C" void tpamd_tuning_reload(void) { g_tuning = read_tuning(); }
 
+// Gives back the buffer of `stream` on the current device. The caller says that no work that uses it is in flight or
+// captured: the stream is synchronised here, then the buffer is freed and its slot is free for another stream.
+extern "C" int tpamd_scratch_release(void *stream) {
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    void *ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> hold(splitk_mutex());
+        for (size_t i = 0; i < g_cache.size(); ++i) {
+            const Entry &e = g_cache[i];
+            if (e.dev == dev && !e.spare && e.stream == static_cast<hipStream_t>(stream)) {
+                ptr = e.ptr;
+                g_cache.erase(g_cache.begin() + static_cast<long>(i));
+                break;
+            }
+        }
+    }
+    if (ptr == nullptr) return TPAMD_OK;  // the stream had none
+    TPAMD_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    TPAMD_HIP(hipFree(ptr));
+    return TPAMD_OK;
+}
+
 extern "C" int tpamd_scratch_query(void *stream, void **ptr_out, uint64_t *bytes_out) {
     TPAMD_REQUIRE(ptr_out != nullptr && bytes_out != nullptr, "tpamd_scratch_query: null output pointer");
     int dev = 0;

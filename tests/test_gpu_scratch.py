@@ -70,3 +70,30 @@ def test_a_capturing_stream_takes_the_spare_buffer(tune):
             assert torch.equal(out, eager) and taken[0] != _native.scratch_of_stream(DEV)[0]
         else:  # an earlier capture in this process took the spare: the call ran unsplit
             torch.testing.assert_close(out.float(), eager.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_a_retired_stream_gives_its_buffer_back(tune):
+    """tpamd_scratch_release: the stream's buffer is freed (the device's free memory grows by about its size) and the stream
+    has none afterwards; K-split work on the stream later simply gets a new one."""
+    tune("TPAMD_GEMM_TILE", "128")
+    tune("TPAMD_GEMM_SPLITK", "4")
+    M, N, K = 256, 512, 4096
+    x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
+    want = _native.linear(x, w)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        got = _native.linear(x, w)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    ptr, nbytes = _native.scratch_of_stream(DEV, stream.cuda_stream)
+    assert ptr is not None and nbytes > 0
+    free_before = torch.cuda.mem_get_info(DEV)[0]
+    _native.release_scratch(DEV, stream.cuda_stream)
+    assert _native.scratch_of_stream(DEV, stream.cuda_stream) == (None, 0)
+    assert torch.cuda.mem_get_info(DEV)[0] >= free_before + nbytes // 2  # the driver accounts in its own granules
+    _native.release_scratch(DEV, stream.cuda_stream)  # a stream without a buffer: nothing to do
+    with torch.cuda.stream(stream):
+        again = _native.linear(x, w)
+    torch.cuda.synchronize()
+    assert torch.equal(again, want)
+    assert _native.scratch_of_stream(DEV, stream.cuda_stream)[0] is not None
