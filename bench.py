@@ -314,6 +314,8 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
                              "step": "swiglu_up + down (tiling and K split chosen by the library: 256x256 / 2 and 128x128 / 4)"}
     for m in (1, 16, 32, 64):
         extra[f"w8_decode_m{m}"] = w8_decode(torch, _native, dev, m)
+    extra["w8_prefill_m1024"] = w8_decode(torch, _native, dev, 1024, graph=False)
+    extra["reduce_2partials_m4096"] = reduce_extra(torch, _native, dev, other)
     extra["attention_falcon40b_shard"] = attention_extra(torch, _native, dev)
     extra["c4_decode_step"] = falcon_attention_decode_step(torch, _native, dev)
     extra.update(api_level_extras(torch, dev))
@@ -506,7 +508,17 @@ def api_level_extras(torch, dev) -> dict:
     return out
 
 
-def w8_decode(torch, _native, dev, m=1) -> dict:
+def reduce_extra(torch, _native, dev, other) -> dict:
+    """The "sum" rule on its own: two rank partials [4096 x 4096] bf16 added by tpamd_reduce_partials (what runs when the sum
+    is not folded into the down projection's epilogue). Bytes: two partials read, one result written."""
+    parts = [[torch.randn_like(other), torch.randn_like(other)] for _ in range(4)]
+    out = torch.empty_like(other)
+    us = _time_us(torch, lambda i: _native.reduce_partials(parts[i % 4], out=out), 10, 100)
+    by = 3.0 * other.numel() * 2
+    return {"us_per_call": us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS, "algorithmic_bytes": by}
+
+
+def w8_decode(torch, _native, dev, m=1, graph=True) -> dict:
     """BASELINE config 5 at batch m: int8 weight-only rank-0 shard of a Falcon-40B-shape MLP (up [16384 x 8192] + GELU,
     down [8192 x 16384], per-row scales, 41 / 82 outlier columns in fp16), fp16 activations. HBM-bound."""
     d, f, n_sets = 8192, 16384, 3
@@ -532,6 +544,10 @@ def w8_decode(torch, _native, dev, m=1) -> dict:
     by = 2.0 * f * d + (f * 41 + d * 82) * 2.0 + (f + d) * 4.0
     entry = {"us_per_step": us, "tokens_per_s": m * 1e6 / us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS,
              "algorithmic_bytes": by, "launch": "eager"}
+    if not graph:  # prefill-sized: bound by the matrix pipe, not by the weight bytes
+        flops = 4.0 * m * d * f
+        return {"us_per_step": us, "tokens_per_s": m * 1e6 / us, "TFLOPs": flops / us / 1e6, "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS,
+                "algorithmic_flops": flops, "step": "int8 up + GELU + down of the Falcon-40B MLP shard, weights dequantised on their way into LDS"}
     try:
         gus = _graph_us(torch, fn, per=12)
         entry["graph"] = {"us_per_step": gus, "tokens_per_s": m * 1e6 / gus, "GBps": by / gus / 1e3, "hbm_frac": by / gus / 1e3 / PEAK_HBM_GBS}

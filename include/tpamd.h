@@ -263,6 +263,8 @@ int tpamd_rope_append(const void *q_dev, const void *k_dev, const void *v_dev, c
  * wq is int8 [N,K] (zero in the outlier columns), scale fp32 [N], outlier_idx int32 [n_out] (sorted,
  * distinct, < K), w_out [N,n_out] in `dtype` with leading dimension ld_wout. Not part of the reference
  * (its README points to LLM.int8 notebooks); defined here in closed form.
+ * Up to 64 rows the weights are streamed once (HBM-bound kernels); up to 128-256 rows once per slab of 64 rows; above
+ * that they go through the matrix pipe once, converted to `dtype` (exactly) on their way into LDS.
  * Requirements: dtype is F16 or BF16; K % 16 == 0; ldw (int8 elements) % 16 == 0. */
 int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,
                     const void *w_out_dev, int64_t n_out, const void *bias_dev, void *y_dev, int64_t M, int64_t N,

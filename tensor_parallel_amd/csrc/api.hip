@@ -22,6 +22,10 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
                     int64_t K, int64_t ldx, int64_t ldw, int64_t ldy, int64_t ld_wout, int dtype, int act, bool swiglu, bool w8,
                     hipStream_t s);
 
+int gemm_w8_dispatch(const void *x, const void *wq, const void *scale, const void *outlier_idx, const void *w_out, int64_t n_out,
+                     const void *bias, void *y, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ld_wout,
+                     int64_t ldy, int dtype, int act, hipStream_t s);
+
 int attention_dispatch(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq,
                        int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal, int dtype, hipStream_t s);
 
@@ -51,6 +55,7 @@ int skinny_row_limit(int64_t N, int64_t K, int64_t *rows) {
     return TPAMD_OK;
 }
 constexpr int64_t SKINNY_W8_SLAB = 64;
+constexpr int64_t W8_TILED_ABOVE = 128;  // int8 weights: rows from which the tiled MFMA kernel takes over from the slabs
 
 // What the MFMA kernels need from 16-bit operands: 16-byte aligned rows of x and w, 8-byte aligned groups of 4
 // outputs. Anything else goes to the scalar-load kernel.
@@ -175,6 +180,15 @@ extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void
     TPAMD_REQUIRE(ldx >= K && ldw >= K && ldy >= N, "%s: leading dimension smaller than the row", who);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int esz = 2;
+    // Above two slabs of the weight-streaming kernels the weights go through the matrix pipe once, dequantised on their
+    // way into LDS; the packed stores of that kernel want groups of 4 outputs on 8-byte boundaries.
+    // (measured on 16384 x 8192 / 8192 x 16384: 129-256 rows 131-135 / 225-231 us tiled against 153-204 / 153-203 us in
+    // slabs; 512 rows 263 / 237 against 407 / 406; 1024 rows 309 / 484 us, 0.57-0.89 PFLOP/s). With fewer 128 x 128
+    // tiles than CUs the slabs stay ahead up to 256 rows.
+    const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+    if (M > W8_TILED_ABOVE && (tiles128 >= 256 || M > 2 * W8_TILED_ABOVE) && N % 4 == 0 && ldy % 4 == 0 && aligned(y_dev, 8) && (!bias_dev || aligned(bias_dev, 8)) && n_out <= 256)
+        return gemm_w8_dispatch(x_dev, wq_dev, scale_dev, outlier_idx_dev, w_out_dev, n_out, bias_dev, y_dev, M, N, K, ldx, ldw,
+                                ld_wout, ldy, dtype, act, s);
     for (int64_t m0 = 0; m0 < M; m0 += SKINNY_W8_SLAB) {  // weights are re-streamed once per slab of 64 rows
         const int64_t mm = M - m0 < SKINNY_W8_SLAB ? M - m0 : SKINNY_W8_SLAB;
         int rc = skinny_dispatch(static_cast<const char *>(x_dev) + m0 * ldx * esz, wq_dev, nullptr, bias_dev, nullptr, 0, scale_dev,

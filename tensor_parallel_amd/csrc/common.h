@@ -159,6 +159,29 @@ __device__ __forceinline__ uint32_t add_packed2(uint32_t a, uint32_t b) {
     return pack2_half<DT>(lo_half_to_f32<DT>(a) + lo_half_to_f32<DT>(b), hi_half_to_f32<DT>(a) + hi_half_to_f32<DT>(b));
 }
 
+// Four int8 (one dword) -> four values of the activation dtype, packed as lo = elements 0,1 and
+// hi = elements 2,3. Exact: |q| <= 128 fits both f16 and bf16 significands.
+template <int DT>
+__device__ __forceinline__ void cvt_i8x4(uint32_t q, uint32_t &lo, uint32_t &hi) {
+    const uint32_t u = q ^ 0x80808080u;  // biased to 0..255
+    if constexpr (DT == TPAMD_F16) {
+        // f16 0x6400 | u == 1024 + u; subtracting 1152 gives q
+        const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+        const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+        const tpamd_f16x2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
+        lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(tpamd_f16x2, p0) - bias);
+        hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(tpamd_f16x2, p1) - bias);
+    } else {
+        // f32 0x4B000000 | u == 2^23 + u; subtracting 2^23 + 128 gives q; its high half is the bf16
+        const float f0 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050400u)) - 8388736.0f;
+        const float f1 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050401u)) - 8388736.0f;
+        const float f2 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050402u)) - 8388736.0f;
+        const float f3 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050403u)) - 8388736.0f;
+        lo = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+        hi = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+    }
+}
+
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
 // v_exp_f32 and v_rcp_f32 (1 ulp each) instead of the 10-instruction IEEE division sequence. Every kernel uses this
 // one definition, so a row's result does not depend on which kernel the batch size selects.

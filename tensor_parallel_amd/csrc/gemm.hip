@@ -1254,6 +1254,215 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmParams p) {
     }
 }
 
+// ---- int8 weights at prefill sizes: dequantised on the way into LDS ---------------------------------------------------
+// y = act(scale[n] * (x . wq^T) + x[:, outliers] . w_out^T + bias) for more rows than the weight-streaming kernels
+// take. Same tiling, staging and MFMA as gemm_kernel; a K tile of the weight is 64 bytes of every row (four 16-byte
+// chunks of 16 int8), converted to the activation dtype in registers (exact) and stored as the 128 bytes the MFMA
+// fragments read. After the last K tile the sums are multiplied by the rows' scales, and the outlier columns follow
+// as up to 4 further K tiles of 64 (x gathered through outlier_idx, w_out read as it lies, both element by element:
+// a percent of the work) into the same accumulators.
+struct W8Extra {
+    const float *scale;
+    const int *outlier_idx;
+    const char *w_out;
+    int n_out;
+    int64_t ld_wout;
+};
+
+template <int DT, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_w8_kernel(GemmParams p, W8Extra q) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    constexpr int XC = BM * 8 / NT;   // 16-byte chunks of the x tile per thread (8 elements each)
+    constexpr int WC = BN * 4 / NT;   // 16-byte chunks of the int8 tile per thread (16 elements each)
+    constexpr int WO = BN * 8 / NT;   // 8-element pieces of the w_out tile per thread
+    constexpr int STAGE = (BM + BN) * LDS_ROW;
+    static_assert(BM * 8 % NT == 0 && BN * 4 % NT == 0, "tile/threads mismatch");
+    extern __shared__ __align__(16) char smem[];
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    const int ld_chunk = tid & 7, ld_row = tid >> 3;      // x: 8 chunks per row
+    const int wq_chunk = tid & 3, wq_row = tid >> 2;      // wq: 4 chunks per row
+    const char *xg[XC];
+    const char *wg[WC];
+#pragma unroll
+    for (int i = 0; i < XC; ++i) {
+        int r = m0 + ld_row + i * (NT / 8);
+        r = r < p.M ? r : p.M - 1;
+        xg[i] = p.x + (static_cast<int64_t>(r) * p.ldx + ld_chunk * 8) * 2;
+    }
+#pragma unroll
+    for (int i = 0; i < WC; ++i) {
+        int r = n0 + wq_row + i * (NT / 4);
+        r = r < p.N ? r : p.N - 1;
+        wg[i] = p.w + static_cast<int64_t>(r) * p.ldw + wq_chunk * 16;
+    }
+    const int st_x = ld_row * LDS_ROW + ld_chunk * 16;
+    const int st_w = wq_row * LDS_ROW + wq_chunk * 32;
+
+    uint4 xr[XC], wr[WC];
+    auto load_global = [&](int kt) {
+        // K is a multiple of 16: chunks are entirely inside or outside. Past the end the row's first chunk is fetched
+        // (a load, not a branch around one) and zeros are stored for both operands.
+        const bool okx = kt * BK + ld_chunk * 8 < p.K, okw = kt * BK + wq_chunk * 16 < p.K;
+        const int64_t offx = okx ? static_cast<int64_t>(kt) * BK * 2 : -static_cast<int64_t>(ld_chunk) * 16;
+        const int64_t offw = okw ? static_cast<int64_t>(kt) * BK : -static_cast<int64_t>(wq_chunk) * 16;
+#pragma unroll
+        for (int i = 0; i < XC; ++i) xr[i] = *reinterpret_cast<const uint4 *>(xg[i] + offx);
+#pragma unroll
+        for (int i = 0; i < WC; ++i) wr[i] = *reinterpret_cast<const uint4 *>(wg[i] + offw);
+    };
+    auto store_lds = [&](int stage, int kt) {
+        char *xs = smem + stage * STAGE;
+        char *ws = xs + BM * LDS_ROW;
+        const bool okx = kt * BK + ld_chunk * 8 < p.K, okw = kt * BK + wq_chunk * 16 < p.K;
+#pragma unroll
+        for (int i = 0; i < XC; ++i)
+            *reinterpret_cast<uint4 *>(xs + st_x + i * (NT / 8) * LDS_ROW) = make_uint4(okx ? xr[i].x : 0u, okx ? xr[i].y : 0u, okx ? xr[i].z : 0u, okx ? xr[i].w : 0u);
+#pragma unroll
+        for (int i = 0; i < WC; ++i) {
+            uint4 lo, hi;
+            cvt_i8x4<DT>(wr[i].x, lo.x, lo.y);
+            cvt_i8x4<DT>(wr[i].y, lo.z, lo.w);
+            cvt_i8x4<DT>(wr[i].z, hi.x, hi.y);
+            cvt_i8x4<DT>(wr[i].w, hi.z, hi.w);
+            char *dst = ws + st_w + i * (NT / 4) * LDS_ROW;
+            *reinterpret_cast<uint4 *>(dst) = okw ? lo : make_uint4(0, 0, 0, 0);
+            *reinterpret_cast<uint4 *>(dst + 16) = okw ? hi : make_uint4(0, 0, 0, 0);
+        }
+    };
+    int x_rd[TM], w_rd[TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t) x_rd[t] = (wm * (BM / WAVES_M) + t * 32 + l32) * LDS_ROW + lhi * 16;
+#pragma unroll
+    for (int t = 0; t < TN; ++t) w_rd[t] = BM * LDS_ROW + (wn * (BN / WAVES_N) + t * 32 + l32) * LDS_ROW + lhi * 16;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
+    auto multiply = [&](const char *stage) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            uint4 xf[TM], wf[TN];
+#pragma unroll
+            for (int t = 0; t < TM; ++t) xf[t] = *reinterpret_cast<const uint4 *>(stage + x_rd[t] + ks * 32);
+#pragma unroll
+            for (int t = 0; t < TN; ++t) wf[t] = *reinterpret_cast<const uint4 *>(stage + w_rd[t] + ks * 32);
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b) acc[a][b] = mfma32<DT>(wf[b], xf[a], acc[a][b]);
+        }
+    };
+
+    const int KT = (p.K + BK - 1) / BK;
+    load_global(0);
+    store_lds(0, 0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_global(kt + 1);
+        multiply(smem + (kt & 1) * STAGE);
+        if (more) store_lds((kt + 1) & 1, kt + 1);
+        __syncthreads();
+    }
+    // the int8 sums become real ones: D[n_local][m_local], register i -> n_local = 8 * (i / 4) + 4 * lhi + i % 4
+#pragma unroll
+    for (int b = 0; b < TN; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            int n = n0 + wn * (BN / WAVES_N) + b * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
+            n = n < p.N ? n : p.N - 1;
+            const float sc = q.scale[n];
+#pragma unroll
+            for (int a = 0; a < TM; ++a) acc[a][b][i] *= sc;
+        }
+    // outlier columns, 64 at a time, staged element by element into stage 0 (nobody reads the stages any more)
+    const uint16_t *xe = reinterpret_cast<const uint16_t *>(p.x);
+    const uint16_t *we = reinterpret_cast<const uint16_t *>(q.w_out);
+    for (int o0 = 0; o0 < q.n_out; o0 += BK) {
+        char *xs = smem;
+        char *ws = xs + BM * LDS_ROW;
+        int col[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int o = o0 + ld_chunk * 8 + e;
+            col[e] = q.outlier_idx[o < q.n_out ? o : q.n_out - 1];
+        }
+#pragma unroll
+        for (int i = 0; i < XC; ++i) {
+            int r = m0 + ld_row + i * (NT / 8);
+            r = r < p.M ? r : p.M - 1;
+            uint32_t v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = xe[static_cast<int64_t>(r) * p.ldx + col[e]];
+            uint32_t d[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t lo = o0 + ld_chunk * 8 + 2 * e < q.n_out ? v[2 * e] : 0u;
+                const uint32_t hi = o0 + ld_chunk * 8 + 2 * e + 1 < q.n_out ? v[2 * e + 1] : 0u;
+                d[e] = lo | (hi << 16);
+            }
+            *reinterpret_cast<uint4 *>(xs + st_x + i * (NT / 8) * LDS_ROW) = make_uint4(d[0], d[1], d[2], d[3]);
+        }
+#pragma unroll
+        for (int i = 0; i < WO; ++i) {
+            int r = n0 + ld_row + i * (NT / 8);
+            r = r < p.N ? r : p.N - 1;
+            uint32_t v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int o = o0 + ld_chunk * 8 + e;
+                v[e] = we[static_cast<int64_t>(r) * q.ld_wout + (o < q.n_out ? o : q.n_out - 1)];
+            }
+            uint32_t d[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t lo = o0 + ld_chunk * 8 + 2 * e < q.n_out ? v[2 * e] : 0u;
+                const uint32_t hi = o0 + ld_chunk * 8 + 2 * e + 1 < q.n_out ? v[2 * e + 1] : 0u;
+                d[e] = lo | (hi << 16);
+            }
+            *reinterpret_cast<uint4 *>(ws + st_x + i * (NT / 8) * LDS_ROW) = make_uint4(d[0], d[1], d[2], d[3]);
+        }
+        __syncthreads();
+        multiply(smem);
+        __syncthreads();
+    }
+    epilogue<DT, MODE_LINEAR, BM, BN, WAVES_M, WAVES_N>(p, acc, m0, n0, wm, wn, l32, lhi);
+}
+
+template <int DT, int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_gemm_w8(GemmParams p, const W8Extra &q, hipStream_t s) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int LDS = 2 * (BM + BN) * LDS_ROW;
+    auto kern = gemm_w8_kernel<DT, BM, BN, WAVES_M, WAVES_N>;
+    static thread_local int configured_dev = -1;  // per instantiation and host thread
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        configured_dev = dev;
+    }
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t blocks = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    TPAMD_REQUIRE(blocks < (1ll << 31), "gemm: too many tiles");
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(NT), LDS, s, p, q);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 // ---- fp32 on the matrix pipe: v_mfma_f32_32x32x2_f32 -------------------------------------------------------------
 // y = act(x . w^T + bias) (+ addend) for fp32 operands whose rows are 16-byte aligned (K, leading dimensions and N
 // multiples of 4). Same staging as gemm_kernel: a K tile is 128 bytes of every row (32 floats here), 16-byte chunks
@@ -1644,6 +1853,30 @@ int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias
     }
     if (dtype == TPAMD_F32 || generic) return generic_dispatch(p, dtype, swiglu, s);
     return dtype == TPAMD_BF16 ? gemm_large<TPAMD_BF16>(p, swiglu, s) : gemm_large<TPAMD_F16>(p, swiglu, s);
+}
+
+// int8 weights above the weight-streaming kernels' row count. x, wq 16-byte aligned, K and ldw multiples of 16, ldx of 8
+// (checked by the caller); N and ldy multiples of 4 and y 8-byte aligned for the packed stores.
+int gemm_w8_dispatch(const void *x, const void *wq, const void *scale, const void *outlier_idx, const void *w_out, int64_t n_out,
+                     const void *bias, void *y, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ld_wout,
+                     int64_t ldy, int dtype, int act, hipStream_t s) {
+    GemmParams p{};
+    p.x = static_cast<const char *>(x);
+    p.w = static_cast<const char *>(wq);
+    p.bias = static_cast<const char *>(bias);
+    p.y = static_cast<char *>(y);
+    p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
+    p.ldx = ldx; p.ldw = ldw; p.ldy = ldy;
+    p.act = act;
+    W8Extra q{static_cast<const float *>(scale), static_cast<const int *>(outlier_idx), static_cast<const char *>(w_out),
+              static_cast<int>(n_out), ld_wout};
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (int rc = device_cus(dev, &cus); rc != TPAMD_OK) return rc;
+    const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
+    const bool big = tiles256 * 2 >= cus;
+    if (dtype == TPAMD_BF16) return big ? launch_gemm_w8<TPAMD_BF16, 256, 256, 2, 4>(p, q, s) : launch_gemm_w8<TPAMD_BF16, 128, 128, 2, 2>(p, q, s);
+    return big ? launch_gemm_w8<TPAMD_F16, 256, 256, 2, 4>(p, q, s) : launch_gemm_w8<TPAMD_F16, 128, 128, 2, 2>(p, q, s);
 }
 
 }  // namespace tpamd

@@ -23,7 +23,6 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { SK_LINEAR = 0, SK_SWIGLU = 1 };
@@ -52,29 +51,6 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     else
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-
-// Four int8 (one dword) -> four values of the activation dtype, packed as lo = elements 0,1 and
-// hi = elements 2,3. Exact: |q| <= 128 fits both f16 and bf16 significands.
-template <int DT>
-__device__ __forceinline__ void cvt_i8x4(uint32_t q, uint32_t &lo, uint32_t &hi) {
-    const uint32_t u = q ^ 0x80808080u;  // biased to 0..255
-    if constexpr (DT == TPAMD_F16) {
-        // f16 0x6400 | u == 1024 + u; subtracting 1152 gives q
-        const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
-        const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
-        const f16x2 bias = {static_cast<_Float16>(1152.0f), static_cast<_Float16>(1152.0f)};
-        lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, p0) - bias);
-        hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, p1) - bias);
-    } else {
-        // f32 0x4B000000 | u == 2^23 + u; subtracting 2^23 + 128 gives q; its high half is the bf16
-        const float f0 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050400u)) - 8388736.0f;
-        const float f1 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050401u)) - 8388736.0f;
-        const float f2 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050402u)) - 8388736.0f;
-        const float f3 = __uint_as_float(__builtin_amdgcn_perm(0x4B000000u, u, 0x07050403u)) - 8388736.0f;
-        lo = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
-        hi = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
-    }
 }
 
 // One output element from its fp32 sums (s1 = the up sum of a gated pair): the reference's op chain with its
@@ -1034,6 +1010,7 @@ __global__ __launch_bounds__(WC_NW * 64, MT == 1 ? 4 : 1) void skinny_w8_cols_ke
 // per row are in flight before anything is multiplied, x (at most 4 rows) sits in LDS, products go through
 // v_dot2 with fp32 accumulation, and 64 lane sums meet in a butterfly at the end.
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 
 template <int DT>
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {

@@ -227,3 +227,48 @@ def test_int8_row_streaming_kernel_on_wide_matrices(dtype, M, N, K, n_out):
     got = _native.linear_w8(*args)
     want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
     torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * 0.02 * math.sqrt(K + 400 * n_out))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K,n_out", [
+    (129, 64, 256, 0),       # just above the slabs, one ragged 128 x 128 tile, no outliers
+    (200, 300, 528, 41),     # ragged in M, N and K (K: 8 tiles of 64 and a quarter), outliers in one staged tile
+    (260, 132, 1040, 70),    # outliers over two staged tiles
+    (700, 36, 272, 256),     # the most outlier columns the kernels take
+])
+def test_linear_w8_prefill_sizes_match_definition(dtype, M, N, K, n_out):
+    """More rows than the weight-streaming kernels take in two passes: the weights go through the matrix pipe once,
+    dequantised on their way into LDS; scales, outlier columns, bias and GELU as at every other size."""
+    x, wq, scale, cols, w_out = make_case(M, N, K, n_out, dtype, seed=M)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(5)) * 0.1).to(dtype)
+    args = (x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+            torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None,
+            torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
+    sigma = 0.02 * math.sqrt(K + 400 * n_out)
+    got = _native.linear_w8(*args)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
+    want_b = want + bias.double().numpy()
+    want_b = 0.5 * want_b * (1.0 + np.vectorize(math.erf)(want_b / math.sqrt(2.0)))
+    got = _native.linear_w8(*args, bias=bias.to(DEV), act=_native.ACT_GELU)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want_b), rtol=2e-2, atol=2e-2 * sigma)
+    # the first 64 rows through the weight-streaming kernels: the same sums in another order
+    few = _native.linear_w8(args[0][:64].contiguous(), *args[1:])
+    torch.testing.assert_close(few.float().cpu(), _native.linear_w8(*args)[:64].float().cpu(), rtol=2e-2, atol=2e-2 * sigma)
+
+
+def test_falcon_mlp_shard_full_shape_at_prefill():
+    """BASELINE config 5's matrices at 1024 tokens (256 x 256 tiles fill the part): sampled rows against the definition."""
+    M, d, f = 1024, 8192, 16384
+    x, wq1, s1, c1, o1 = make_case(M, f, d, 41, torch.float16, 0)
+    dev = lambda a, dt=None: (torch.from_numpy(a) if dt is None else torch.from_numpy(a).to(dt)).to(DEV)  # noqa: E731
+    up = _native.linear_w8(x.to(DEV), dev(wq1), dev(s1), dev(c1.astype(np.int32)), dev(o1, torch.float16), act=_native.ACT_GELU)
+    rows = [0, 1, 255, 256, 511, 777, 1023]
+    want_up = torch.nn.functional.gelu(torch.from_numpy(oq.linear_w8_f64(x[rows].float().numpy(), wq1, s1, c1, o1)))
+    torch.testing.assert_close(up[rows].double().cpu(), want_up, rtol=2e-2, atol=2e-2 * 0.02 * math.sqrt(d + 400 * 41))
+    assert torch.isfinite(up.float()).all()
+    del wq1, want_up
+    _, wq2, s2, c2, o2 = make_case(1, d, f, 82, torch.float16, 1)
+    down = _native.linear_w8(up, dev(wq2), dev(s2), dev(c2.astype(np.int32)), dev(o2, torch.float16))
+    want_down = oq.linear_w8_f64(up[rows].cpu().float().numpy(), wq2, s2, c2, o2)
+    torch.testing.assert_close(down[rows].double().cpu(), torch.from_numpy(want_down), rtol=2e-2, atol=2e-2 * float(np.abs(want_down).std()))
