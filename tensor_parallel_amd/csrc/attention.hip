@@ -437,7 +437,7 @@ int launch(AttnParams p, int cus, hipStream_t s) {
         return TPAMD_OK;
     }
     const size_t need = static_cast<size_t>(nsplit) * p.B * p.Hkv * p.rows_pad * (D + 4) * sizeof(float);
-    std::lock_guard<std::mutex> hold(splitk_mutex());
+    std::lock_guard<std::mutex> hold(splitk_mutex(dev));
     void *ws = nullptr;
     int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
     if (rc != TPAMD_OK) return rc;

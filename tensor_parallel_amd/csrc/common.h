@@ -61,9 +61,10 @@ const Tuning &tuning();
 int device_cus(int dev, int *cus_out);
 
 // fp32 scratch memory of the K-split kernels (split-K partial tiles, split-key attention partials): defined in
-// runtime.hip. Callers hold splitk_mutex() from the lookup until their launches that use the buffer are enqueued
-// and pass reserve = 4 * CUs * 64 KiB, so that a stream's buffer is allocated with the size every shape can live with.
-std::mutex &splitk_mutex();
+// runtime.hip. Callers hold splitk_mutex(dev), the lock of their device, from the lookup until their launches that use
+// the buffer are enqueued (two host threads that share a stream must not interleave a K-split launch and its finishing
+// pass), and pass reserve = 4 * CUs * 64 KiB, so that a stream's buffer is allocated with the size every shape can live with.
+std::mutex &splitk_mutex(int dev);
 int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, void **out);
 // While one of these lives on a host thread, splitk_scratch() on that thread hands out the library's fixed array and
 // allocates nothing.

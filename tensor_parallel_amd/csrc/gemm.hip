@@ -1672,7 +1672,7 @@ int launch_direct(GemmParams p, int cus, int splits, hipStream_t s) {
             f.tiles_n = (p.N + BN_OUT / 2 - 1) / (BN_OUT / 2);
             const int64_t tiles128 = static_cast<int64_t>(f.tiles_m) * f.tiles_n;
             const size_t ws_bytes = static_cast<size_t>(p.splits) * tiles128 * 128 * 128 * sizeof(float);
-            std::lock_guard<std::mutex> hold(splitk_mutex());
+            std::lock_guard<std::mutex> hold(splitk_mutex(dev));
             void *ws = nullptr;
             const int rc = splitk_scratch(dev, s, ws_bytes, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
             if (rc != TPAMD_OK) return rc;
@@ -1750,7 +1750,7 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
         if (rc != TPAMD_OK) return rc;
         const size_t ws_bytes = static_cast<size_t>(splits) * tiles * 128 * 128 * sizeof(float);
         // the scratch buffer is ours until both launches are enqueued
-        std::lock_guard<std::mutex> hold(splitk_mutex());
+        std::lock_guard<std::mutex> hold(splitk_mutex(dev));
         void *ws = nullptr;
         rc = splitk_scratch(dev, s, ws_bytes, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
         if (rc != TPAMD_OK) return rc;

@@ -12,7 +12,7 @@ static __device__ __align__(256) char scratch[TPAMD_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 constexpr int MAX_DEV = 64;
-void *g_static_ptr[MAX_DEV];  // guarded by splitk_mutex()
+void *g_static_ptr[MAX_DEV];  // entry d guarded by splitk_mutex(d)
 thread_local bool g_static_mode = false;
 }  // namespace
 
@@ -20,7 +20,7 @@ StaticScratchScope::StaticScratchScope() { g_static_mode = true; }
 StaticScratchScope::~StaticScratchScope() { g_static_mode = false; }
 bool static_scratch_active() { return g_static_mode; }
 
-// Called by splitk_scratch() with splitk_mutex() held and `dev` current.
+// Called by splitk_scratch() with splitk_mutex(dev) held and `dev` current.
 int static_scratch(int dev, size_t need, void **out) {
     *out = nullptr;
     if (need > TPAMD_NOALLOC_SCRATCH_BYTES) {

@@ -72,17 +72,20 @@ struct Entry {
     void *ptr;
     size_t bytes;
 };
-std::vector<Entry> g_cache;  // guarded by splitk_mutex()
+constexpr int LOCKS = 64;  // one lock and one list per device (devices 64 apart would share them)
+std::vector<Entry> g_caches[LOCKS];  // list d guarded by splitk_mutex(d)
 constexpr int MAX_BUFFERS_PER_DEVICE = 33;  // 32 streams (a framework's stream pool) and the spare
+
+int slot_of(int dev) { return dev >= 0 ? dev % LOCKS : 0; }
 
 }  // namespace
 
-std::mutex &splitk_mutex() {
-    static std::mutex m;
-    return m;
+std::mutex &splitk_mutex(int dev) {
+    static std::mutex m[LOCKS];
+    return m[slot_of(dev)];
 }
 
-// The caller holds splitk_mutex() from this call until its launches that use the buffer are enqueued.
+// The caller holds splitk_mutex(dev) from this call until its launches that use the buffer are enqueued.
 // *out = a buffer of at least `need` bytes for work on `stream` of device `dev` (the current device), or NULL: then the
 // caller runs its unsplit form. A stream's buffer is allocated at its first use with max(need, reserve) bytes and kept
 // until the process ends; streams of one device never share one, so K-split work on different streams cannot meet in
@@ -99,7 +102,7 @@ static int allocate_entry(int dev, hipStream_t stream, bool spare, size_t bytes,
         set_error("hipMalloc of %zu bytes of K-split scratch memory failed: %s", bytes, hipGetErrorString(e));
         return TPAMD_ERR_NOMEM;
     }
-    g_cache.push_back(Entry{dev, stream, spare, ptr, bytes});
+    g_caches[slot_of(dev)].push_back(Entry{dev, stream, spare, ptr, bytes});
     if (out != nullptr) *out = ptr;
     return TPAMD_OK;
 }
@@ -109,7 +112,7 @@ int splitk_scratch(int dev, hipStream_t stream, size_t need, size_t reserve, voi
     if (static_scratch_active()) return static_scratch(dev, need, out);
     int on_device = 0;
     Entry *spare = nullptr;
-    for (Entry &e : g_cache) {
+    for (Entry &e : g_caches[slot_of(dev)]) {
         if (e.dev != dev) continue;
         ++on_device;
         if (e.spare) {
@@ -154,7 +157,8 @@ extern "C" int tpamd_scratch_release(void *stream) {
     TPAMD_HIP(hipGetDevice(&dev));
     void *ptr = nullptr;
     {
-        std::lock_guard<std::mutex> hold(splitk_mutex());
+        std::lock_guard<std::mutex> hold(splitk_mutex(dev));
+        std::vector<Entry> &g_cache = g_caches[slot_of(dev)];
         for (size_t i = 0; i < g_cache.size(); ++i) {
             const Entry &e = g_cache[i];
             if (e.dev == dev && !e.spare && e.stream == static_cast<hipStream_t>(stream)) {
@@ -176,8 +180,8 @@ extern "C" int tpamd_scratch_query(void *stream, void **ptr_out, uint64_t *bytes
     TPAMD_HIP(hipGetDevice(&dev));
     *ptr_out = nullptr;
     *bytes_out = 0;
-    std::lock_guard<std::mutex> hold(splitk_mutex());
-    for (const Entry &e : g_cache)
+    std::lock_guard<std::mutex> hold(splitk_mutex(dev));
+    for (const Entry &e : g_caches[slot_of(dev)])
         if (e.dev == dev && !e.spare && e.stream == static_cast<hipStream_t>(stream)) {
             *ptr_out = e.ptr;
             *bytes_out = e.bytes;

@@ -1446,7 +1446,7 @@ int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
         return TPAMD_OK;
     }
     const size_t need = static_cast<size_t>(splits) * p.M * p.N * sizeof(float);
-    std::lock_guard<std::mutex> hold(splitk_mutex());
+    std::lock_guard<std::mutex> hold(splitk_mutex(dev));
     void *ws = nullptr;
     const int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
     if (rc != TPAMD_OK) return rc;
@@ -1497,7 +1497,7 @@ int launch_w8_cols_mt(const SkinnyParams &p, int dev, int cus, hipStream_t s, bo
     }
     if (int rc = configure_w8_cols<DT, MT, false>(dev, lds); rc != TPAMD_OK) return rc;
     const size_t need = static_cast<size_t>(planes) * p.M * p.N * sizeof(float);
-    std::lock_guard<std::mutex> hold(splitk_mutex());
+    std::lock_guard<std::mutex> hold(splitk_mutex(dev));
     void *ws = nullptr;
     const int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
     if (rc != TPAMD_OK) return rc;
