@@ -318,6 +318,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     extra["reduce_2partials_m4096"] = reduce_extra(torch, _native, dev, other)
     extra["attention_falcon40b_shard"] = attention_extra(torch, _native, dev)
     extra["c4_decode_step"] = falcon_attention_decode_step(torch, _native, dev)
+    extra["c4_prefill_step"] = falcon_attention_prefill_step(torch, _native, dev)
     extra.update(api_level_extras(torch, dev))
 
     from types import SimpleNamespace
@@ -442,6 +443,35 @@ def falcon_attention_decode_step(torch, _native, dev) -> dict:
     except Exception as e:  # noqa: BLE001 - the eager figure stands on its own
         entry["graph"] = {"error": str(e)[:200]}
     return entry
+
+
+def falcon_attention_prefill_step(torch, _native, dev) -> dict:
+    """BASELINE config 4, prefill: the same shard on 1024 new tokens of one sequence (empty cache): QKV projection, rotary +
+    cache fill, causal attention over the 1024 positions, dense projection. FLOPs: both projections and the visible half
+    of the score and value products."""
+    S, Hq, Hkv, D, d_model = 1024, 64, 4, 64, 8192
+    per = Hq // Hkv
+    g = torch.Generator(device=dev).manual_seed(0)
+    wqkv = (torch.randn((Hq + 2 * Hkv) * D, d_model, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    wdense = (torch.randn(d_model, Hq * D, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    kc = torch.zeros(1, Hkv, S, D, device=dev, dtype=torch.bfloat16)
+    vc = torch.zeros(1, Hkv, S, D, device=dev, dtype=torch.bfloat16)
+    x = torch.randn(1, S, d_model, device=dev, generator=g).to(torch.bfloat16)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
+    ang = torch.arange(S, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
+    ang = torch.cat([ang, ang], dim=-1)[None]
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+
+    def fn(i):
+        fused = _native.linear(x, wqkv).view(1, S, Hkv, per + 2, D)
+        q_rot = _native.rope_append(fused[:, :, :, :per], fused[:, :, :, per], fused[:, :, :, per + 1], cos, sin, kc, vc, 0)
+        attn = _native.attention(q_rot, kc, vc, causal=True)
+        return _native.linear(attn.view(S, Hq * D), wdense)
+
+    us = _time_us(torch, fn, 10, 50)
+    flops = 2.0 * S * d_model * (Hq + 2 * Hkv) * D + 2.0 * S * Hq * D * d_model + 4.0 * Hq * S * S * D * 0.5
+    return {"us_per_step": us, "tokens_per_s": S / us * 1e6, "TFLOPs": flops / us / 1e6, "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS,
+            "algorithmic_flops": flops, "step": "qkv projection + rotary/cache fill + causal attention core + dense projection, eager"}
 
 
 def api_level_extras(torch, dev) -> dict:
