@@ -75,11 +75,14 @@ def test_a_split_whose_partial_tiles_do_not_fit_is_refused(tune):
 
 def test_nothing_is_allocated():
     """A first call on a fresh stream, with a K-split shape: the device's free memory does not move and the stream gets
-    no scratch buffer of its own (the allocating entry point would give it one)."""
+    no scratch buffer of its own (the allocating entry point would give it 64 MiB). The stream has run one unrelated
+    kernel before, so that what the HIP runtime itself sets up for a stream's first launch (2 MiB here) is not counted."""
     M, N, K = 384, 2048, 4096
     x, w = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV)
     y = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
     fresh = torch.cuda.Stream()
+    with torch.cuda.stream(fresh):
+        y.zero_()
     torch.cuda.synchronize()
     free_before = torch.cuda.mem_get_info(DEV)[0]
     with torch.cuda.stream(fresh):
