@@ -1471,14 +1471,17 @@ int launch_gemm_w8(GemmParams p, const W8Extra &q, hipStream_t s) {
 // agree, so lane (row r, half h) uses k = 16 h + s in step s: its 16 operands of a K tile are 64 contiguous bytes of
 // the staged row (four 16-byte reads). w is the first operand, so a lane holds 4 consecutive output columns of one
 // row per group of 4 accumulator registers: one 16-byte store. Products and sums are fp32 throughout.
-constexpr int BK32 = 32;  // floats per stage row
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+// BKF = floats of K per stage and row: 32 (128 bytes, two blocks per CU) for problems with many tiles; 128 for few tiles,
+// where a block has its CU to itself and a loop of many short stages would wait for memory once per stage.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKF>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmParams p) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
-    constexpr int XC = BM * 8 / NT, WC = BN * 8 / NT;
-    constexpr int STAGE = (BM + BN) * LDS_ROW;
-    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile/threads mismatch");
+    constexpr int CPR = BKF / 4;             // 16-byte chunks per staged row
+    constexpr int ROW = BKF * 4 + 16;        // staged row pitch in bytes: conflict-free 16-byte reads
+    constexpr int XC = BM * CPR / NT, WC = BN * CPR / NT;
+    constexpr int STAGE = (BM + BN) * ROW;
+    static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0 && NT % CPR == 0, "tile/threads mismatch");
     extern __shared__ __align__(16) char smem[];
 
     int tile_m, tile_n;
@@ -1489,27 +1492,27 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmPar
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    const int ld_chunk = tid & 7, ld_row = tid >> 3;
+    const int ld_chunk = tid % CPR, ld_row = tid / CPR;
     const char *xg[XC];
     const char *wg[WC];
 #pragma unroll
     for (int i = 0; i < XC; ++i) {
-        int r = m0 + ld_row + i * (NT / 8);
+        int r = m0 + ld_row + i * (NT / CPR);
         r = r < p.M ? r : p.M - 1;  // rows past the end repeat the last one; their outputs are not stored
         xg[i] = p.x + (static_cast<int64_t>(r) * p.ldx + ld_chunk * 4) * 4;
     }
 #pragma unroll
     for (int i = 0; i < WC; ++i) {
-        int r = n0 + ld_row + i * (NT / 8);
+        int r = n0 + ld_row + i * (NT / CPR);
         r = r < p.N ? r : p.N - 1;
         wg[i] = p.w + (static_cast<int64_t>(r) * p.ldw + ld_chunk * 4) * 4;
     }
-    const int st_off = ld_row * LDS_ROW + ld_chunk * 16;
+    const int st_off = ld_row * ROW + ld_chunk * 16;
     uint4 xr[XC], wr[WC];
     auto load_global = [&](int kt) {
-        const bool ok = kt * BK32 + ld_chunk * 4 < p.K;  // K is a multiple of 4: a chunk is entirely inside or outside
-        // past the end of K the row's first chunk is fetched instead (a load, not a branch); x is zeroed when stored
-        const int64_t off = ok ? static_cast<int64_t>(kt) * BK32 * 4 : -static_cast<int64_t>(ld_chunk) * 16;
+        const bool ok = kt * BKF + ld_chunk * 4 < p.K;  // K is a multiple of 4: a chunk is entirely inside or outside
+        // past the end of K the row's first chunk is fetched instead (a load, not a branch); zeros are stored for it
+        const int64_t off = ok ? static_cast<int64_t>(kt) * BKF * 4 : -static_cast<int64_t>(ld_chunk) * 16;
 #pragma unroll
         for (int i = 0; i < XC; ++i) xr[i] = *reinterpret_cast<const uint4 *>(xg[i] + off);
 #pragma unroll
@@ -1517,20 +1520,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmPar
     };
     auto store_lds = [&](int stage, int kt) {
         char *xs = smem + stage * STAGE;
-        char *ws = xs + BM * LDS_ROW;
-        const bool ok = kt * BK32 + ld_chunk * 4 < p.K;
+        char *ws = xs + BM * ROW;
+        const bool ok = kt * BKF + ld_chunk * 4 < p.K;
 #pragma unroll
         for (int i = 0; i < XC; ++i)
-            *reinterpret_cast<uint4 *>(xs + st_off + i * (NT / 8) * LDS_ROW) = make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
+            *reinterpret_cast<uint4 *>(xs + st_off + i * (NT / CPR) * ROW) = make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
 #pragma unroll
-        for (int i = 0; i < WC; ++i)  // w past the end of K may be anything finite or not: it must not meet a NaN-free zero
-            *reinterpret_cast<uint4 *>(ws + st_off + i * (NT / 8) * LDS_ROW) = make_uint4(ok ? wr[i].x : 0u, ok ? wr[i].y : 0u, ok ? wr[i].z : 0u, ok ? wr[i].w : 0u);
+        for (int i = 0; i < WC; ++i)  // both operands are zeroed: whatever the other one holds there must not meet a NaN
+            *reinterpret_cast<uint4 *>(ws + st_off + i * (NT / CPR) * ROW) = make_uint4(ok ? wr[i].x : 0u, ok ? wr[i].y : 0u, ok ? wr[i].z : 0u, ok ? wr[i].w : 0u);
     };
     int x_rd[TM], w_rd[TN];
 #pragma unroll
-    for (int t = 0; t < TM; ++t) x_rd[t] = (wm * (BM / WAVES_M) + t * 32 + l32) * LDS_ROW + lhi * 64;
+    for (int t = 0; t < TM; ++t) x_rd[t] = (wm * (BM / WAVES_M) + t * 32 + l32) * ROW + lhi * (BKF * 2);
 #pragma unroll
-    for (int t = 0; t < TN; ++t) w_rd[t] = BM * LDS_ROW + (wn * (BN / WAVES_N) + t * 32 + l32) * LDS_ROW + lhi * 64;
+    for (int t = 0; t < TN; ++t) w_rd[t] = BM * ROW + (wn * (BN / WAVES_N) + t * 32 + l32) * ROW + lhi * (BKF * 2);
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -1540,7 +1543,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmPar
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.0f;
 
-    const int KT = (p.K + BK32 - 1) / BK32;
+    const int KT = (p.K + BKF - 1) / BKF;
     load_global(0);
     store_lds(0, 0);
     __syncthreads();
@@ -1549,7 +1552,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmPar
         if (more) load_global(kt + 1);
         const char *stage = smem + (kt & 1) * STAGE;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {  // 4 floats of the lane's 16 at a time
+        for (int q = 0; q < BKF / 8; ++q) {  // 4 floats of the lane's BKF / 2 at a time
             f32x4 xf[TM], wf[TN];
 #pragma unroll
             for (int t = 0; t < TM; ++t) xf[t] = *reinterpret_cast<const f32x4 *>(stage + x_rd[t] + q * 16);
@@ -1589,11 +1592,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmPar
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BKF>
 int launch_gemm_f32(GemmParams p, hipStream_t s) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
-    constexpr int LDS = 2 * (BM + BN) * LDS_ROW;
-    auto kern = gemm_f32_kernel<BM, BN, WAVES_M, WAVES_N>;
+    constexpr int LDS = 2 * (BM + BN) * (BKF * 4 + 16);
+    auto kern = gemm_f32_kernel<BM, BN, WAVES_M, WAVES_N, BKF>;
     static thread_local int configured_dev = -1;  // per instantiation and host thread
     int dev = 0;
     TPAMD_HIP(hipGetDevice(&dev));
@@ -1848,8 +1851,10 @@ int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias
         TPAMD_HIP(hipGetDevice(&dev));
         if (int rc = device_cus(dev, &cus); rc != TPAMD_OK) return rc;
         const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
-        if (tiles128 >= cus) return launch_gemm_f32<128, 128, 2, 2>(p, s);
-        return launch_gemm_f32<64, 64, 2, 2>(p, s);
+        if (tiles128 >= cus) return launch_gemm_f32<128, 128, 2, 2, 32>(p, s);
+        const int64_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+        if (tiles64 >= 2 * cus) return launch_gemm_f32<64, 64, 2, 2, 32>(p, s);
+        return launch_gemm_f32<64, 64, 2, 2, 128>(p, s);  // few tiles: long stages, a block per CU
     }
     if (dtype == TPAMD_F32 || generic) return generic_dispatch(p, dtype, swiglu, s);
     return dtype == TPAMD_BF16 ? gemm_large<TPAMD_BF16>(p, swiglu, s) : gemm_large<TPAMD_F16>(p, swiglu, s);

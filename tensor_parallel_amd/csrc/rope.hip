@@ -3,8 +3,8 @@
 //
 // Every (batch, position, head) row of D contiguous elements is handled by D / 16 lanes. A lane owns 8 elements of the
 // first half of the row and the 8 elements of the second half that rotate with them, so one 16-byte load per half
-// gives it both members of its 8 pairs, and both 16-byte stores are whole. Rows are numbered q rows first, then k,
-// then v (v rows are copied); the launch is bound by its latency at decode and by HBM at prefill, where it moves
+// gives it both members of its 8 pairs, and both 16-byte stores are whole. A block takes 256 lanes of one (batch,
+// position): its q rows first, then k, then v (v rows are copied); the launch is bound by its latency at decode and by HBM at prefill, where it moves
 // every byte once.
 #include "common.h"
 
@@ -23,7 +23,7 @@ struct RopeParams {
     int64_t qo_b, qo_h, qo_s;      // q_out [B, Hq, S, D]
     int64_t kc_b, kc_h, kc_s;      // key cache [B, Hkv, S_max, D]
     int64_t vc_b, vc_h, vc_s;
-    int64_t n_lanes;               // B * S * (Hq + 2 Hkv) * (D / 16)
+    int lanes_per_pos;             // (Hq + 2 Hkv) * (D / 16): lanes of one (batch, position)
 };
 
 // out = round(round(a * c) + round(b * s)) per 16-bit element: the three torch ops of
@@ -45,23 +45,21 @@ __device__ __forceinline__ uint4 rot8(uint4 a, uint4 c, uint4 b, uint4 s, float 
 
 template <int DT>
 __global__ __launch_bounds__(256) void rope_append_kernel(RopeParams p) {
-    const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (t >= p.n_lanes) return;
-    const int lanes_per_row = p.D >> 4;
-    const int chunk = static_cast<int>(t % lanes_per_row);
-    int64_t row = t / lanes_per_row;
-    const int heads = p.Hq + 2 * p.Hkv;
-    const int head = static_cast<int>(row % heads);
-    row /= heads;
-    const int s = static_cast<int>(row % p.S);
-    const int b = static_cast<int>(row / p.S);
+    // grid: x = (batch, position), y = blocks of 256 lanes over that position's heads; 32-bit index arithmetic throughout
+    const int t = blockIdx.y * 256 + threadIdx.x;
+    if (t >= p.lanes_per_pos) return;
+    const int shift = p.D == 64 ? 2 : 3;  // D / 16 lanes per head row
+    const int chunk = t & ((1 << shift) - 1);
+    const int head = t >> shift;
+    const int b = static_cast<int>(blockIdx.x) / p.S;
+    const int s = static_cast<int>(blockIdx.x) - b * p.S;
     const int half_bytes = p.D;  // D / 2 elements of 2 bytes
     const int at = chunk * 16;   // byte offset of the lane's 8 elements inside a half
 
     if (head >= p.Hq + p.Hkv) {  // value row: copied into the cache
         const int h = head - p.Hq - p.Hkv;
-        const char *src = p.v + (b * p.v_b + s * p.v_s + h * p.v_h) * 2 + at;
-        char *dst = p.v_cache + (b * p.vc_b + h * p.vc_h + (p.pos0 + s) * p.vc_s) * 2 + at;
+        const char *src = p.v + (static_cast<int64_t>(b) * p.v_b + s * p.v_s + h * p.v_h) * 2 + at;
+        char *dst = p.v_cache + (static_cast<int64_t>(b) * p.vc_b + h * p.vc_h + (p.pos0 + s) * p.vc_s) * 2 + at;
         const uint4 lo = *reinterpret_cast<const uint4 *>(src), hi = *reinterpret_cast<const uint4 *>(src + half_bytes);
         *reinterpret_cast<uint4 *>(dst) = lo;
         *reinterpret_cast<uint4 *>(dst + half_bytes) = hi;
@@ -122,12 +120,12 @@ extern "C" int tpamd_rope_append(const void *q_dev, const void *k_dev, const voi
     p.vc_b = strides[17]; p.vc_h = strides[18]; p.vc_s = strides[19];
     p.q_g = strides[20];
     p.per = static_cast<int>(Hq / Hkv);
-    p.n_lanes = B * S * (Hq + 2 * Hkv) * (D / 16);
-    const int64_t blocks = (p.n_lanes + 255) / 256;
-    TPAMD_REQUIRE(blocks < (1ll << 31), "%s: too many rows for one launch", who);
+    p.lanes_per_pos = static_cast<int>((Hq + 2 * Hkv) * (D / 16));
+    TPAMD_REQUIRE(B * S < (1ll << 31), "%s: too many positions for one launch", who);
+    const dim3 grid(static_cast<unsigned>(B * S), static_cast<unsigned>((p.lanes_per_pos + 255) / 256));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == TPAMD_BF16) hipLaunchKernelGGL(rope_append_kernel<TPAMD_BF16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL(rope_append_kernel<TPAMD_F16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, p);
+    if (dtype == TPAMD_BF16) hipLaunchKernelGGL(rope_append_kernel<TPAMD_BF16>, grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(rope_append_kernel<TPAMD_F16>, grid, dim3(256), 0, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }
