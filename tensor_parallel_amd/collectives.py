@@ -24,14 +24,36 @@ from .slicing import concat_dim
 RENDEZVOUS_TIMEOUT_S = 600.0
 
 # Rank threads that share ONE device take turns on the host: a rank holds the "turn" lock while it runs module
-# code and gives it up only while it waits in a rendezvous. All ranks enqueue onto the same device anyway, so
+# code and gives it up only while it waits in a collective. All ranks enqueue onto the same device anyway, so
 # nothing is lost, and host-side lazy initialisation inside torch (attention backends, BLAS handles) is never
-# entered by two rank threads at once. The lock of the running forward is published per thread here.
+# entered by two rank threads at once. The turn of the running forward is published per thread here.
 _turn = threading.local()
 
 
-def set_turn_lock(lock: Optional[threading.Lock]) -> None:
-    _turn.lock = lock
+class Turn:
+    """What the rank threads of one forward on one device share: the lock that says whose turn it is, a condition on that
+    lock on which ranks wait inside a collective, and a flag that a rank has failed (its peers stop waiting)."""
+
+    __slots__ = ("lock", "cond", "failed")
+
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.cond = threading.Condition(self.lock)
+        self.failed = False
+
+    def fail(self) -> None:
+        """Called by a failing rank while it holds the lock: wakes every waiting peer."""
+        self.failed = True
+        self.cond.notify_all()
+
+
+def set_turn_lock(turn: Optional[Turn]) -> None:
+    _turn.turn = turn
+    _turn.lock = turn.lock if turn is not None else None
+
+
+def current_turn() -> Optional[Turn]:
+    return getattr(_turn, "turn", None)
 
 
 def turn_lock() -> Optional[threading.Lock]:
@@ -105,8 +127,48 @@ class CollectiveOperation(CollectiveOpetationBase):
         self._inputs: List[Any] = [None] * world_size
         self._outputs: List[Any] = [None] * world_size
         self._error: Optional[BaseException] = None
+        self._arrived = 0  # turn-taking ranks: how many have handed in their value this round
+        self._round = 0
+
+    def _call_in_turns(self, x: Any, rank: int, turn: Turn):
+        """The same exchange for rank threads that take turns on one device (the caller holds the turn lock): a rank
+        hands in its value and waits on the turn's condition, which gives the turn away; the rank that arrives last
+        runs `func` and wakes the others. One wake-up per waiting rank and collective instead of three barrier rounds.
+        The results of a round stay in place until the next round of this op completes, which needs every rank to have
+        come back, so nobody can miss its result."""
+        self._inputs[rank] = x
+        self._arrived += 1
+        if self._arrived == self.world_size:
+            try:
+                result = self.func(*self._inputs)
+                self._outputs = [result[i] for i in range(self.world_size)]
+                self._error = None
+            except BaseException as e:  # fan the failure out to every rank
+                self._outputs = [None] * self.world_size
+                self._error = e
+            self._inputs = [None] * self.world_size
+            self._arrived = 0
+            self._round += 1
+            turn.cond.notify_all()
+        else:
+            started = self._round
+            while self._round == started:
+                if turn.failed:
+                    self._inputs[rank] = None
+                    self._arrived -= 1
+                    raise threading.BrokenBarrierError
+                if not turn.cond.wait(self.timeout):
+                    self._inputs[rank] = None
+                    self._arrived -= 1
+                    raise threading.BrokenBarrierError
+        if self._error is not None:
+            raise self._error
+        return self._outputs[rank]
 
     def __call__(self, x: Any, rank: int):
+        turn = current_turn()
+        if turn is not None:
+            return self._call_in_turns(x, rank, turn)
         try:
             self._inputs[rank] = x
             _rendezvous(self._barrier, self.timeout)

@@ -17,7 +17,7 @@ import torch
 from torch import nn
 
 from .autoconfig import get_default_config
-from .collectives import set_turn_lock
+from .collectives import Turn, set_turn_lock
 from .config import Config, add_lora_rules
 from .kv_cache import is_kv_cache, rank_caches
 from .shard import make_shard
@@ -249,19 +249,19 @@ def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devi
     grad_enabled = torch.is_grad_enabled()
     # ranks that share one device take turns on the host (see collectives.set_turn_lock)
     shared = len(modules) > 1 and all(d.type == "cuda" and d == devices[0] for d in devices)
-    turn = threading.Lock() if shared else None
+    turn = Turn() if shared else None
 
     def worker(i, module, args, kwargs, device):
         torch.set_grad_enabled(grad_enabled)
         if turn is not None:
-            turn.acquire()
+            turn.lock.acquire()
             set_turn_lock(turn)
         try:
             _run(i, module, args, kwargs, device)
         finally:
             if turn is not None:
                 set_turn_lock(None)
-                turn.release()
+                turn.lock.release()
 
     def _run(i, module, args, kwargs, device):
         try:
@@ -276,6 +276,8 @@ def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devi
             with lock:
                 results[i] = (False, e)
             # a rank that fails must not leave its peers waiting in a collective
+            if turn is not None:
+                turn.fail()
             for m in module.modules():
                 for rules in (getattr(m, "input_actions", {}), getattr(m, "output_actions", {})):
                     for op in rules.values():

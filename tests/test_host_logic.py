@@ -318,16 +318,16 @@ def test_rendezvous_timeout_does_not_hang():
 
 
 def test_rank_threads_take_turns_between_rendezvous():
-    """With a turn lock published, only one rank runs host code at a time; the lock is given up inside a
-    rendezvous (otherwise the second rank could never arrive) and is free again afterwards."""
+    """With a turn published, only one rank runs host code at a time; the turn is given up while a rank waits inside a
+    collective (otherwise the next rank could never arrive) and is free again afterwards."""
     import threading
     import time
 
-    from tensor_parallel_amd.collectives import CollectiveOperation, set_turn_lock
+    from tensor_parallel_amd.collectives import CollectiveOperation, Turn, set_turn_lock
 
     world = 3
     op = CollectiveOperation(world, lambda *xs: [sum(xs)] * world, timeout=20.0)
-    turn = threading.Lock()
+    turn = Turn()
     running, overlaps, results = [0], [0], {}
 
     def critical():
@@ -338,7 +338,7 @@ def test_rank_threads_take_turns_between_rendezvous():
         running[0] -= 1
 
     def worker(rank):
-        turn.acquire()
+        turn.lock.acquire()
         set_turn_lock(turn)
         try:
             total = 0
@@ -348,7 +348,7 @@ def test_rank_threads_take_turns_between_rendezvous():
             results[rank] = total
         finally:
             set_turn_lock(None)
-            turn.release()
+            turn.lock.release()
 
     threads = [threading.Thread(target=worker, args=(r,)) for r in range(world)]
     for t in threads:
@@ -359,7 +359,76 @@ def test_rank_threads_take_turns_between_rendezvous():
     assert overlaps[0] == 0
     want = sum(sum(r + step for r in range(world)) for step in range(5))
     assert results == {r: want for r in range(world)}
-    assert turn.acquire(blocking=False)
+    assert turn.lock.acquire(blocking=False)
+
+
+def test_a_failing_rank_wakes_the_ranks_that_wait_in_turns():
+    """Two ranks wait inside a collective; the third fails before it arrives and says so on the turn: the waiting ranks
+    leave with BrokenBarrierError, and the op is usable for the next forward (a fresh turn)."""
+    import threading
+
+    from tensor_parallel_amd.collectives import CollectiveOperation, Turn, set_turn_lock
+
+    world = 3
+    op = CollectiveOperation(world, lambda *xs: [sum(xs)] * world, timeout=20.0)
+
+    def run(fail_rank):
+        turn, outcome = Turn(), {}
+
+        def worker(rank):
+            turn.lock.acquire()
+            set_turn_lock(turn)
+            try:
+                if rank == fail_rank:
+                    turn.fail()
+                    outcome[rank] = "failed"
+                    return
+                outcome[rank] = op(rank, rank)
+            except threading.BrokenBarrierError:
+                outcome[rank] = "broken"
+            finally:
+                set_turn_lock(None)
+                turn.lock.release()
+
+        threads = [threading.Thread(target=worker, args=(r,)) for r in range(world)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(10)
+        assert not any(t.is_alive() for t in threads)
+        return outcome
+
+    assert run(fail_rank=2) == {0: "broken", 1: "broken", 2: "failed"}
+    assert run(fail_rank=None) == {0: 3, 1: 3, 2: 3}
+
+
+def test_a_collective_whose_function_raises_raises_on_every_rank_in_turns():
+    import threading
+
+    from tensor_parallel_amd.collectives import CollectiveOperation, Turn, set_turn_lock
+
+    def boom(*xs):
+        raise ValueError("bad values")
+
+    op, turn, seen = CollectiveOperation(2, boom, timeout=5.0), Turn(), {}
+
+    def worker(rank):
+        turn.lock.acquire()
+        set_turn_lock(turn)
+        try:
+            op(rank, rank)
+        except ValueError as e:
+            seen[rank] = str(e)
+        finally:
+            set_turn_lock(None)
+            turn.lock.release()
+
+    threads = [threading.Thread(target=worker, args=(r,)) for r in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(10)
+    assert seen == {0: "bad values", 1: "bad values"}
 
 
 # ---------------------------------------------------------------------------------------- wrapper protocol
