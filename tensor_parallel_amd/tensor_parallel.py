@@ -250,6 +250,9 @@ def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devi
     # ranks that share one device take turns on the host (see collectives.set_turn_lock)
     shared = len(modules) > 1 and all(d.type == "cuda" and d == devices[0] for d in devices)
     turn = Turn() if shared else None
+    # a thread starts on its device's default stream: the rank threads work on the stream the caller is on instead, so that
+    # what the caller enqueued before the forward is ordered before it and what it enqueues afterwards behind it
+    streams = [torch.cuda.current_stream(d) if d.type == "cuda" else None for d in devices]
 
     def worker(i, module, args, kwargs, device):
         torch.set_grad_enabled(grad_enabled)
@@ -257,7 +260,11 @@ def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devi
             turn.lock.acquire()
             set_turn_lock(turn)
         try:
-            _run(i, module, args, kwargs, device)
+            if streams[i] is not None:
+                with torch.cuda.stream(streams[i]):
+                    _run(i, module, args, kwargs, device)
+            else:
+                _run(i, module, args, kwargs, device)
         finally:
             if turn is not None:
                 set_turn_lock(None)

@@ -43,6 +43,33 @@ def test_embeds_and_linear_forward_parity(world):
             assert torch.equal(sd[k].cpu(), v), k
 
 
+def test_forward_runs_on_the_callers_stream():
+    """The rank threads enqueue on the stream the caller is on: an input produced on a side stream just before the forward
+    (behind a long chain of kernels) is complete when the shards read it, and the result is ready for what the caller
+    enqueues next on that stream."""
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(512, 1024), nn.ReLU(), nn.Linear(1024, 256)).to(torch.bfloat16)
+    model_tp = tp.TensorParallel(deepcopy(model), [DEV] * 2, sharded=False)
+    a = torch.randn(2048, 2048, device=DEV, dtype=torch.bfloat16) * 0.02
+    seed = torch.randn(2048, 512, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        want_x = seed
+        for _ in range(30):
+            want_x = (a @ want_x.repeat(1, 4))[:, :512] * 0.5
+        want = model_tp(want_x).clone()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            x = seed
+            for _ in range(30):  # tens of microseconds each: still running when the forward is enqueued
+                x = (a @ x.repeat(1, 4))[:, :512] * 0.5
+            out = model_tp(x)
+            doubled = out * 2
+        side.synchronize()
+    assert torch.equal(out, want)
+    assert torch.equal(doubled, want * 2)
+
+
 def test_backward_is_refused():
     model_tp = tp.TensorParallel(toy(), [DEV] * 2, sharded=False)
     out = model_tp(torch.randint(1, 1000, size=(1, 10), device=DEV))
