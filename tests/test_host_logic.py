@@ -615,3 +615,68 @@ def test_convolution_layers_get_no_rule_and_a_warning(caplog):
     assert any("convolution" in r.getMessage() for r in caplog.records)
     patterns = [p.pattern for p in cfg.state_rules]
     assert any(p.startswith("^2.") for p in patterns) and not any(p.startswith("^0.") for p in patterns)
+
+
+# ---------------------------------------------------------------------------------------- the sum folded into a Linear
+def test_sum_op_hands_out_only_running_sums_in_rank_order(monkeypatch):
+    """What a rank's last Linear may add in its epilogue: with two ranks whatever the other rank has handed in; with more,
+    the running sum over ranks 0 .. r-1 and nothing else, so that the result stays the rank-ordered stepwise sum. The
+    reduction then adds only what the widest value lacks."""
+    from tensor_parallel_amd import _native, collectives
+    from tensor_parallel_amd.collectives import DeviceAllReduce, Turn, set_turn_lock
+
+    summed = []
+
+    def host_sum(parts, accum=0, out=None):
+        summed.append([float(p[0]) for p in parts])
+        total = parts[0].clone()
+        for p in parts[1:]:
+            total = total + p
+        return total
+
+    monkeypatch.setattr(_native, "reduce_partials", host_sum)
+    monkeypatch.setattr(collectives, "FUSE_SUM", True)
+    t = [torch.full((2,), float(10 ** r)) for r in range(4)]  # 1, 10, 100, 1000: a sum shows which ranks it covers
+    op = DeviceAllReduce(3)
+    assert op.addend_for(1) is None  # no turn: ranks are not taking turns on one device
+    set_turn_lock(Turn())
+    try:
+        assert op.addend_for(1) is None  # nothing has been handed in
+        op._inputs, op._masks = [t[0], None, None], [0b001, 0, 0]
+        got = op.addend_for(1)
+        assert got is not None and got[0] is t[0] and got[1] == 0b001
+        assert op.addend_for(2) is None  # rank 1 has not arrived
+        s01 = t[0] + t[1]
+        op._inputs, op._masks = [t[0], s01, None], [0b001, 0b011, 0]
+        got = op.addend_for(2)
+        assert got[0] is s01 and got[1] == 0b011
+        # rank 1 arrived first: neither rank 0 (nothing below it) nor rank 2 (rank 1's value is not a sum from rank 0 on)
+        op._inputs, op._masks = [None, t[1], None], [0, 0b010, 0]
+        assert op.addend_for(0) is None and op.addend_for(2) is None
+        # the reduction: a value that covers ranks 0 and 1 and rank 2's own partial -> only those two are added, in order
+        op._masks = [0b001, 0b011, 0b100]
+        out = op._reduce(t[0], s01, t[2])
+        assert summed[-1] == [11.0, 100.0] and float(out[0][0]) == 111.0 and len(out) == 3
+        # a value that covers every rank: nothing is launched
+        s012 = s01 + t[2]
+        op._masks = [0b001, 0b011, 0b111]
+        n = len(summed)
+        out = op._reduce(t[0], s01, s012)
+        assert len(summed) == n and float(out[1][0]) == 111.0
+        # nobody folded anything: the plain rank-ordered sum
+        op._masks = [0b001, 0b010, 0b100]
+        op._reduce(t[0], t[1], t[2])
+        assert summed[-1] == [1.0, 10.0, 100.0]
+        # two ranks: either order
+        two = DeviceAllReduce(2)
+        two._inputs, two._masks = [None, t[1]], [0, 0b10]
+        got = two.addend_for(0)
+        assert got[0] is t[1] and got[1] == 0b10
+        two._masks = [0b11, 0b10]
+        n = len(summed)
+        out = two._reduce(t[0] + t[1], t[1])
+        assert len(summed) == n and float(out[0][0]) == 11.0
+        # F32 accumulation is another arithmetic: never folded
+        assert DeviceAllReduce(2, accum=_native.ACCUM_F32).fusable is False
+    finally:
+        set_turn_lock(None)
