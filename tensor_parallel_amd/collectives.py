@@ -81,8 +81,21 @@ class SumContext:
         self.calls: dict = {}
         self.fused_mask = 0
 
+    def settle(self, value: Any) -> None:
+        """Called by the wrapper with the value its module returned for the summed output, before the rules run. If a
+        Linear folded the waiting partials in, that value must be the Linear's output itself. Otherwise this call
+        teaches the Linear that produced exactly this value (and ran once) that it feeds the sum: next time it may fold."""
+        if self.fused_out is not None:
+            if value is not self.fused_out:
+                raise RuntimeError(
+                    "tensor_parallel_amd: a row-parallel Linear added the other ranks' partial sums in its epilogue, but its "
+                    "module then returned a different tensor; set TPAMD_FUSE_SUM=0 to keep the sum in its own kernel")
+        elif self.last_linear is not None:
+            feeds = value is self.last_out and self.calls.get(id(self.last_linear)) == 1
+            self.last_linear.__dict__["_tp_feeds_sum"] = self.owner if feeds else None
 
-def push_sum_context(ctx: SumContext) -> None:
+
+def push_sum_context(ctx: Optional[SumContext]) -> None:
     stack = getattr(_contexts, "stack", None)
     if stack is None:
         stack = _contexts.stack = []
@@ -233,18 +246,8 @@ class DeviceAllReduce(CollectiveOperation):
     def __call__(self, x: Any, rank: int):
         mask = 1 << rank
         ctx = current_sum_context()
-        if ctx is not None and ctx.op is self and ctx.rank == rank:
-            linear = ctx.last_linear
-            if ctx.fused_out is not None:
-                if x is not ctx.fused_out:
-                    raise RuntimeError(
-                        "tensor_parallel_amd: a row-parallel Linear added the other ranks' partial sums in its epilogue, but the "
-                        "module then returned a different tensor; set TPAMD_FUSE_SUM=0 to keep the sum in its own kernel")
-                mask |= ctx.fused_mask
-            elif linear is not None:
-                # the Linear that produced exactly the value handed in, called once: next time it may add the waiting partials
-                feeds = x is ctx.last_out and ctx.calls.get(id(linear)) == 1
-                linear.__dict__["_tp_feeds_sum"] = ctx.owner if feeds else None
+        if ctx is not None and ctx.op is self and ctx.fused_out is not None and x is ctx.fused_out:
+            mask |= ctx.fused_mask  # this value already holds what the rank's Linear was given by addend_for()
         self._masks[rank] = mask
         try:
             return super().__call__(x, rank)

@@ -151,3 +151,39 @@ def test_fp32_linear_with_bias_under_a_sum_rule(monkeypatch):
     for out in outs:
         assert torch.equal(out, want)
     torch.testing.assert_close(outs[-1].cpu(), model(x), rtol=1e-5, atol=1e-5)
+
+
+def test_two_summed_outputs_of_one_module_share_the_op(monkeypatch):
+    """A module that returns two row-parallel products, both under a "sum" rule (one op object serves both): the Linear
+    behind output 0 folds its sum, output 1 goes through the reduction kernel, and neither is taken for the other."""
+    class Pair(nn.Module):
+        def __init__(self, d):
+            super().__init__()
+            self.a, self.b = nn.Linear(d, d, bias=False), nn.Linear(d, 2 * d, bias=False)
+
+        def forward(self, x):
+            second = self.a(x)
+            first = self.b(x)
+            return first, second
+
+    torch.manual_seed(0)
+    d, world = 128, 2
+    model = nn.Sequential(Pair(d)).to(torch.bfloat16)
+    cfg = tp.Config(state_rules={r"^0\.a\.weight$": tp.Split(world, 1), r"^0\.b\.weight$": tp.Split(world, 1)},
+                    input_rules={r"^0$": {0: "split -1"}}, output_rules={r"^0$": {0: "sum", 1: "sum"}}, attr_rules={})
+    model_tp = tp.TensorParallel(deepcopy(model), [DEV] * world, tensor_parallel_config=cfg, sharded=False)
+    x = torch.randn(33, d).to(torch.bfloat16).to(DEV)
+    monkeypatch.setattr(collectives, "FUSE_SUM", False)
+    with torch.no_grad():
+        want = model_tp(x)
+    monkeypatch.setattr(collectives, "FUSE_SUM", True)
+    count = Counter(monkeypatch)
+    with torch.no_grad():
+        outs = [model_tp(x) for _ in range(3)]
+    # first forward: two reductions; then output 0 is folded into b's epilogue and only output 1 is reduced
+    assert count.reductions == 2 + 1 + 1 and count.fused == 2
+    for out in outs:
+        assert torch.equal(out[0], want[0]) and torch.equal(out[1], want[1])
+    ref = model.float()(x.float().cpu())
+    for got, r in zip(outs[-1], ref):
+        torch.testing.assert_close(got.float().cpu(), r, rtol=2e-2, atol=2e-2 * r.std().item())
