@@ -78,3 +78,88 @@ def test_int8_linear_random_shape(seed):
     want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
     sigma = 0.02 * math.sqrt(K + 400 * n_out)
     torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL * sigma, msg=lambda m: f"M={M} N={N} K={K} n_out={n_out} {dtype}: {m}")
+
+
+@pytest.mark.parametrize("seed", range(300, 330))
+def test_fp32_linear_random_shape(seed):
+    """fp32 operands, mostly with rows that 16-byte accesses can take (the matrix-pipe kernel in its three tilings), some
+    without (the scalar kernel); bias, GELU and the addend of the folded partial sum in turn. rtol 1e-5."""
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    aligned = seed % 5 != 0
+    M = pick(1, 700)
+    K = 4 * pick(1, 400) if aligned else pick(1, 900)
+    N = 4 * pick(1, 700) if aligned else pick(1, 900)
+    if seed % 7 == 0:  # enough 128 x 128 tiles for the large tiling
+        M, N = 128 * pick(9, 14), 128 * pick(20, 24) + 4 * pick(0, 8)
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(N, K, generator=g) * 0.02
+    b = torch.randn(N, generator=g) * 0.1 if seed % 2 else None
+    add = torch.randn(M, N, generator=g) if seed % 3 == 1 else None
+    act = _native.ACT_GELU if seed % 3 == 0 else _native.ACT_NONE
+    got = _native.linear(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), act=act, addend=None if add is None else add.to(DEV))
+    want = F.linear(x.double(), w.double(), None if b is None else b.double())
+    if act == _native.ACT_GELU:
+        want = F.gelu(want)
+    if add is not None:
+        want = want + add.double()
+    torch.testing.assert_close(got.cpu(), want.float(), rtol=1e-5, atol=1e-5 * 0.02 * math.sqrt(K) + 1e-6,
+                               msg=lambda m: f"M={M} N={N} K={K} aligned={aligned}: {m}")
+
+
+@pytest.mark.parametrize("seed", range(400, 416))
+def test_int8_linear_random_shape_at_prefill_sizes(seed):
+    """More rows than the weight-streaming kernels take: the tiled kernel that converts the weights on their way into LDS
+    (both tilings), and the slabs of 64 rows where the matrix has too few tiles."""
+    import numpy as np
+
+    from oracle import quant as oq
+
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    M = pick(129, 900)
+    N, K = 4 * pick(8, 1100), 16 * pick(2, 260)
+    if seed % 4 == 0:
+        M, N = 256 * pick(4, 6) + pick(0, 40), 256 * pick(16, 20) + 4 * pick(0, 20)  # fills the 256 x 256 tiling
+    n_out = [0, 7, 41, 130, 256][pick(0, 4)]
+    n_out = min(n_out, K // 2)
+    dtype = [torch.bfloat16, torch.float16][pick(0, 1)]
+    w = (torch.randn(N, K, generator=g) * 0.02).to(dtype).float().numpy()
+    x = torch.randn(M, K, generator=g)
+    cols = np.sort(torch.randperm(K, generator=g)[:n_out].numpy())
+    x[:, cols] *= 20
+    x = x.to(dtype)
+    wq, scale, w_out = oq.quantize_rows(w, cols)
+    got = _native.linear_w8(x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+                            torch.from_numpy(cols.astype(np.int32)).to(DEV) if n_out else None,
+                            torch.from_numpy(w_out).to(dtype).to(DEV) if n_out else None)
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
+    sigma = 0.02 * math.sqrt(K + 400 * n_out)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=RTOL, atol=RTOL * sigma,
+                               msg=lambda m: f"M={M} N={N} K={K} n_out={n_out} {dtype}: {m}")
+
+
+@pytest.mark.parametrize("seed", range(500, 520))
+def test_rope_append_random_shape(seed):
+    """Random batch, positions, head counts and cache offsets, q / k / v as strided views of one fused buffer: bit for bit
+    against the oracle."""
+    from oracle import rope as orp
+
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    B, S, Hkv, per = pick(1, 5), pick(1, 40), pick(1, 5), pick(1, 9)
+    D = [64, 128][pick(0, 1)]
+    dtype = [torch.bfloat16, torch.float16][pick(0, 1)]
+    pos0 = pick(0, 50)
+    L = pos0 + S + pick(0, 7)
+    fused = torch.randn(B, S, Hkv, per + 2, D, generator=g).to(dtype)
+    cos, sin = orp.angles(torch.arange(pos0, pos0 + S), D, dtype=dtype)
+    kc = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
+    vc = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
+    want_q, want_kc, want_vc = orp.rope_append(fused[:, :, :, :per].reshape(B, S, Hkv * per, D), fused[:, :, :, per], fused[:, :, :, per + 1],
+                                               cos[None], sin[None], kc, vc, pos0)
+    fd, kcd, vcd = fused.to(DEV), kc.to(DEV), vc.to(DEV)
+    got_q = _native.rope_append(fd[:, :, :, :per], fd[:, :, :, per], fd[:, :, :, per + 1], cos.to(DEV), sin.to(DEV), kcd, vcd, pos0)
+    as_bits = lambda t: t.detach().cpu().contiguous().view(torch.int16)  # noqa: E731
+    assert torch.equal(as_bits(got_q), as_bits(want_q)), f"B={B} S={S} Hkv={Hkv} per={per} D={D} pos0={pos0}"
+    assert torch.equal(as_bits(kcd), as_bits(want_kc)) and torch.equal(as_bits(vcd), as_bits(want_vc))
