@@ -1592,6 +1592,117 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_f32_kernel(GemmPar
     }
 }
 
+// Few output tiles (the Linears of a small model on a short sequence): 32 x 32 tiles, and the four wavefronts of a block
+// share a tile's K instead of its outputs. Wavefront w multiplies floats [32 w, 32 w + 32) of every 128-float stage, so a
+// tile's chain of dependent MFMAs is a quarter as long and four times as many blocks are in flight; the four partial
+// tiles meet in LDS and wavefront w finishes output columns 8 w .. 8 w + 7 of the tile.
+__global__ __launch_bounds__(256) void gemm_f32_small_kernel(GemmParams p) {
+    constexpr int T = 32, BKF = 128, CPR = BKF / 4, ROW = BKF * 4 + 16, NT = 256;
+    constexpr int XC = T * CPR / NT;  // 16-byte chunks per thread and operand
+    constexpr int STAGE = 2 * T * ROW;
+    extern __shared__ __align__(16) char smem[];
+    const int tile_n = blockIdx.x % p.tiles_n, tile_m = blockIdx.x / p.tiles_n;
+    const int m0 = tile_m * T, n0 = tile_n * T;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int ld_chunk = tid % CPR, ld_row = tid / CPR;
+    const char *xg[XC];
+    const char *wg[XC];
+#pragma unroll
+    for (int i = 0; i < XC; ++i) {
+        int r = m0 + ld_row + i * (NT / CPR);
+        r = r < p.M ? r : p.M - 1;
+        xg[i] = p.x + (static_cast<int64_t>(r) * p.ldx + ld_chunk * 4) * 4;
+        r = n0 + ld_row + i * (NT / CPR);
+        r = r < p.N ? r : p.N - 1;
+        wg[i] = p.w + (static_cast<int64_t>(r) * p.ldw + ld_chunk * 4) * 4;
+    }
+    const int st_off = ld_row * ROW + ld_chunk * 16;
+    uint4 xr[XC], wr[XC];
+    auto load_global = [&](int kt) {
+        const bool ok = kt * BKF + ld_chunk * 4 < p.K;
+        const int64_t off = ok ? static_cast<int64_t>(kt) * BKF * 4 : -static_cast<int64_t>(ld_chunk) * 16;
+#pragma unroll
+        for (int i = 0; i < XC; ++i) {
+            xr[i] = *reinterpret_cast<const uint4 *>(xg[i] + off);
+            wr[i] = *reinterpret_cast<const uint4 *>(wg[i] + off);
+        }
+    };
+    auto store_lds = [&](int stage, int kt) {
+        char *xs = smem + stage * STAGE;
+        char *ws = xs + T * ROW;
+        const bool ok = kt * BKF + ld_chunk * 4 < p.K;
+#pragma unroll
+        for (int i = 0; i < XC; ++i) {
+            *reinterpret_cast<uint4 *>(xs + st_off + i * (NT / CPR) * ROW) = make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
+            *reinterpret_cast<uint4 *>(ws + st_off + i * (NT / CPR) * ROW) = make_uint4(ok ? wr[i].x : 0u, ok ? wr[i].y : 0u, ok ? wr[i].z : 0u, ok ? wr[i].w : 0u);
+        }
+    };
+    // lane (row l32, half lhi) of wavefront w: floats 32 w + 16 lhi + s of the stage in step s
+    const int x_rd = l32 * ROW + wave * 128 + lhi * 64;
+    const int w_rd = T * ROW + x_rd;
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    const int KT = (p.K + BKF - 1) / BKF;
+    load_global(0);
+    store_lds(0, 0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_global(kt + 1);
+        const char *stage = smem + (kt & 1) * STAGE;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const f32x4 xf = *reinterpret_cast<const f32x4 *>(stage + x_rd + q * 16);
+            const f32x4 wf = *reinterpret_cast<const f32x4 *>(stage + w_rd + q * 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[j], xf[j], acc, 0, 0, 0);
+        }
+        if (more) store_lds((kt + 1) & 1, kt + 1);
+        __syncthreads();
+    }
+    // the four partial tiles meet: red[wave][register][lane]
+    float *red = reinterpret_cast<float *>(smem);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[(wave * 16 + i) * 64 + lane] = acc[i];
+    __syncthreads();
+    f32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int i = wave * 4 + e;
+        v[e] = (red[(0 * 16 + i) * 64 + lane] + red[(1 * 16 + i) * 64 + lane]) + (red[(2 * 16 + i) * 64 + lane] + red[(3 * 16 + i) * 64 + lane]);
+    }
+    // D[n_local][m_local]: lane -> m_local = l32, register i -> n_local = 8 * (i / 4) + 4 * lhi + i % 4; here i / 4 = wave
+    const int m = m0 + l32, n = n0 + 8 * wave + 4 * lhi;
+    if (m >= p.M || n >= p.N) return;  // N is a multiple of 4: the group of 4 is all in or all out
+    if (p.bias) v += *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.bias) + n);
+    if (p.act == TPAMD_ACT_GELU) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = gelu_erf(v[j]);
+    }
+    if (p.addend != nullptr) v += *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.addend) + static_cast<int64_t>(m) * p.ldadd + n);
+    *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.y) + static_cast<int64_t>(m) * p.ldy + n) = v;
+}
+
+int launch_gemm_f32_small(GemmParams p, hipStream_t s) {
+    constexpr int LDS = 2 * 2 * 32 * (128 * 4 + 16);
+    static thread_local int configured_dev = -1;
+    int dev = 0;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (configured_dev != dev) {
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_f32_small_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        configured_dev = dev;
+    }
+    p.tiles_m = (p.M + 31) / 32;
+    p.tiles_n = (p.N + 31) / 32;
+    const int64_t blocks = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    TPAMD_REQUIRE(blocks < (1ll << 31), "gemm: too many tiles");
+    hipLaunchKernelGGL(gemm_f32_small_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), LDS, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BKF>
 int launch_gemm_f32(GemmParams p, hipStream_t s) {
     constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -1854,7 +1965,8 @@ int gemm_dispatch(const void *x, const void *w, const void *w2, const void *bias
         if (tiles128 >= cus) return launch_gemm_f32<128, 128, 2, 2, 32>(p, s);
         const int64_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
         if (tiles64 >= 2 * cus) return launch_gemm_f32<64, 64, 2, 2, 32>(p, s);
-        return launch_gemm_f32<64, 64, 2, 2, 128>(p, s);  // few tiles: long stages, a block per CU
+        if (tiles64 * 2 >= cus) return launch_gemm_f32<64, 64, 2, 2, 128>(p, s);  // few tiles: long stages, a block per CU
+        return launch_gemm_f32_small(p, s);  // fewer still: 32 x 32 tiles whose K is shared by the block's wavefronts
     }
     if (dtype == TPAMD_F32 || generic) return generic_dispatch(p, dtype, swiglu, s);
     return dtype == TPAMD_BF16 ? gemm_large<TPAMD_BF16>(p, swiglu, s) : gemm_large<TPAMD_F16>(p, swiglu, s);
