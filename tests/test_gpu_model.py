@@ -90,6 +90,33 @@ def test_worker_failure_is_raised_not_hung():
         model_tp.to("cpu")(torch.randn(2, 8))
 
 
+def test_one_failing_rank_frees_its_peers_and_the_next_forward_works():
+    """Only one rank fails, between two collectives, while its peer may already wait in the next one: the forward raises
+    the rank's error (not a timeout), and the collective ops are usable again afterwards."""
+    class Flaky(nn.Module):
+        calls, armed = 0, False
+
+        def forward(self, x):
+            Flaky.calls += 1
+            if Flaky.armed and Flaky.calls % 2 == 0:
+                raise RuntimeError("one rank failed")
+            return x
+
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(16, 32), Flaky(), nn.Linear(32, 8))
+    model_tp = tp.TensorParallel(deepcopy(model), [DEV] * 2, sharded=False)
+    x = torch.randn(5, 16)
+    with torch.no_grad():
+        want = model(x)
+        torch.testing.assert_close(model_tp(x.to(DEV)).cpu(), want, rtol=1e-5, atol=1e-5)
+        Flaky.armed = True
+        with pytest.raises(RuntimeError, match="one rank failed"):
+            model_tp(x.to(DEV))
+        Flaky.armed = False
+        for _ in range(2):
+            torch.testing.assert_close(model_tp(x.to(DEV)).cpu(), want, rtol=1e-5, atol=1e-5)
+
+
 class LlamaMLP(nn.Module):
     def __init__(self, d, f):
         super().__init__()
