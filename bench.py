@@ -356,41 +356,46 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
 
 
 def attention_extra(torch, _native, dev) -> dict:
-    """Rank-local attention core at the Falcon-40B shard shape of BASELINE config 4 (W = 2: 64 query heads, 4 key/value
-    heads, head_dim 64): decode batch 8 on 2048 cached keys (bound by reading K and V once) and causal prefill of 1024
-    positions at batch 8 (bound by the matrix pipe; flops counted for the visible half of the score matrix)."""
+    """Rank-local attention core at the shape of a Falcon-40B rank shard at W = 2 (64 query heads, 4 key/value heads,
+    head_dim 64): decode batch 8 on 2048 and on 8192 cached keys (bound by reading K and V once) and causal prefill of
+    1024 positions at batch 8 (bound by the matrix pipe; flops counted for the visible half of the score matrix)."""
     g = torch.Generator(device=dev).manual_seed(0)
     out = {}
     q = torch.randn(8, 64, 1, 64, device=dev, generator=g).to(torch.bfloat16)
-    caches = [(torch.randn(8, 4, 2048, 64, device=dev, generator=g).to(torch.bfloat16),
-               torch.randn(8, 4, 2048, 64, device=dev, generator=g).to(torch.bfloat16)) for _ in range(8)]
 
-    def dec(i):
-        k, v = caches[i % len(caches)]
-        return _native.attention(q, k, v, causal=True)
+    def decode(keys, n_caches):
+        # more caches than the 256 MB of last-level cache hold, taken in turn
+        caches = [(torch.randn(8, 4, keys, 64, device=dev, generator=g).to(torch.bfloat16),
+                   torch.randn(8, 4, keys, 64, device=dev, generator=g).to(torch.bfloat16)) for _ in range(n_caches)]
 
-    by = 2.0 * 8 * 4 * 2048 * 64 * 2
-    us = _time_us(torch, dec, 10, 100)
-    entry = {"us_per_call": us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS, "algorithmic_bytes": by, "launch": "eager"}
-    try:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for i in range(3):
-                dec(i)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph, per = torch.cuda.CUDAGraph(), 32
-        with torch.cuda.graph(graph, stream=side):  # the stream that ran the warm-up calls
-            for i in range(per):
-                dec(i)
-        gus = _time_us(torch, lambda i: graph.replay(), 3, 10) / per
-        entry["graph"] = {"us_per_call": gus, "GBps": by / gus / 1e3, "hbm_frac": by / gus / 1e3 / PEAK_HBM_GBS}
-        del graph
-    except Exception as e:  # noqa: BLE001
-        entry["graph"] = {"error": str(e)[:200]}
-    out["decode_b8_kv2048"] = entry
-    del caches
+        def dec(i):
+            k, v = caches[i % len(caches)]
+            return _native.attention(q, k, v, causal=True)
+
+        by = 2.0 * 8 * 4 * keys * 64 * 2
+        us = _time_us(torch, dec, 10, 100)
+        entry = {"us_per_call": us, "GBps": by / us / 1e3, "hbm_frac": by / us / 1e3 / PEAK_HBM_GBS, "algorithmic_bytes": by, "launch": "eager"}
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for i in range(3):
+                    dec(i)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph, per = torch.cuda.CUDAGraph(), 32
+            with torch.cuda.graph(graph, stream=side):  # the stream that ran the warm-up calls
+                for i in range(per):
+                    dec(i)
+            gus = _time_us(torch, lambda i: graph.replay(), 3, 10) / per
+            entry["graph"] = {"us_per_call": gus, "GBps": by / gus / 1e3, "hbm_frac": by / gus / 1e3 / PEAK_HBM_GBS}
+            del graph
+        except Exception as e:  # noqa: BLE001
+            entry["graph"] = {"error": str(e)[:200]}
+        return entry
+
+    out["decode_b8_kv2048"] = decode(2048, 8)
+    out["decode_b8_kv8192"] = decode(8192, 6)
     q = torch.randn(8, 64, 1024, 64, device=dev, generator=g).to(torch.bfloat16)
     k = torch.randn(8, 4, 1024, 64, device=dev, generator=g).to(torch.bfloat16)
     v = torch.randn(8, 4, 1024, 64, device=dev, generator=g).to(torch.bfloat16)

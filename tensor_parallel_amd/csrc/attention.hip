@@ -35,6 +35,21 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
 }
 
 typedef __attribute__((ext_vector_type(4))) short i16x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;  // 16 bytes on their way from global memory to LDS
+
+// A loop whose counter is a constant expression inside the body (f gets Const<0>, Const<1>, ...): arrays indexed with it
+// are split into registers from the start, not only if a later pass unrolls the loop.
+template <int I>
+struct Const {
+    static constexpr int value = I;
+};
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(Const<I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 // ds_read_b64_tr_b16: every lane gives the LDS address of four 16-bit elements; within each group of 16 lanes,
 // lane i receives element i % 4 of lanes i / 4, 4 + i / 4, 8 + i / 4 and 12 + i / 4 (in that order).
@@ -61,7 +76,8 @@ constexpr int AT_KEYS = 64;   // keys per tile
 // A block owns 64 * RT consecutive rows.
 // At least two wavefronts per SIMD are asked for: that caps a wavefront at 256 registers, and with no need for
 // AGPRs the compiler keeps MFMA results in ordinary VGPRs, where the softmax can use them without copies.
-template <int DT, int D, int RT>
+// P = K / V tiles a thread keeps requested ahead of the one being multiplied (see the two loops below).
+template <int DT, int D, int RT, int P>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) void attention_kernel(AttnParams p) {
     constexpr int KP = D * 2 + 16;   // K tile row pitch (bytes): conflict-free 16-byte reads
     constexpr int VP = D * 2 + 32;   // V tile row pitch (bytes): 8 consecutive keys' 32-byte pieces cover all banks
@@ -139,13 +155,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     const char *kbase = p.k + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh) * 2;
     const char *vbase = p.v + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh) * 2;
 
-    // K / V tiles travel global -> registers -> LDS (row-major, both). The registers of tile i+2 are requested right after
-    // tile i+1 has been written to the other LDS buffer, so the loads fly during a whole tile's MFMAs and softmax, and a
-    // tile costs one barrier. A full tile's addresses are a loop-invariant per-thread pointer plus a uniform offset.
+    // K / V tiles travel global -> registers -> LDS (row-major, both), and a tile costs one barrier. A full tile's
+    // addresses are a loop-invariant per-thread pointer plus a uniform offset.
     constexpr int CH = D / 8;                    // 16-byte chunks per key
     constexpr int LPT = AT_KEYS * CH / 256;      // chunks per thread per tile (2 for head_dim 64, 4 for 128)
     constexpr int KSTEP = 256 / CH;              // keys between a thread's chunks
-    uint4 kreg[LPT], vreg[LPT];
+    u32x4 kreg[P][LPT], vreg[P][LPT];
     const int key_j0 = tid / CH, chunk = tid % CH;  // thread's key inside a tile for j = 0
     const int64_t k_pitch = p.k_ss * 2, v_pitch = p.v_ss * 2;
     const char *kthr = kbase + chunk * 16 + key_j0 * k_pitch, *vthr = vbase + chunk * 16 + key_j0 * v_pitch;
@@ -153,8 +168,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         if (k0 + AT_KEYS <= k_end) {  // uniform
 #pragma unroll
             for (int j = 0; j < LPT; ++j) {
-                kreg[j] = *reinterpret_cast<const uint4 *>(kthr + static_cast<int64_t>(k0 + j * KSTEP) * k_pitch);
-                vreg[j] = *reinterpret_cast<const uint4 *>(vthr + static_cast<int64_t>(k0 + j * KSTEP) * v_pitch);
+                kreg[0][j] = *reinterpret_cast<const u32x4 *>(kthr + static_cast<int64_t>(k0 + j * KSTEP) * k_pitch);
+                vreg[0][j] = *reinterpret_cast<const u32x4 *>(vthr + static_cast<int64_t>(k0 + j * KSTEP) * v_pitch);
             }
         } else {
 #pragma unroll
@@ -164,10 +179,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
                 // unconditional loads (first key of the range when out of it) keep all of them in flight together;
                 // keys past the end are zero (and masked below)
                 const int64_t kr = ok ? key : k_begin;
-                const uint4 kv4 = *reinterpret_cast<const uint4 *>(kbase + chunk * 16 + kr * k_pitch);
-                const uint4 vv4 = *reinterpret_cast<const uint4 *>(vbase + chunk * 16 + kr * v_pitch);
-                kreg[j] = ok ? kv4 : make_uint4(0, 0, 0, 0);
-                vreg[j] = ok ? vv4 : make_uint4(0, 0, 0, 0);
+                const u32x4 kv4 = *reinterpret_cast<const u32x4 *>(kbase + chunk * 16 + kr * k_pitch);
+                const u32x4 vv4 = *reinterpret_cast<const u32x4 *>(vbase + chunk * 16 + kr * v_pitch);
+                kreg[0][j] = ok ? kv4 : u32x4{0, 0, 0, 0};
+                vreg[0][j] = ok ? vv4 : u32x4{0, 0, 0, 0};
             }
         }
     };
@@ -175,22 +190,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
             const int key = key_j0 + j * KSTEP;
-            *reinterpret_cast<uint4 *>(ks[buf] + key * KP + chunk * 16) = kreg[j];
-            *reinterpret_cast<uint4 *>(vs[buf] + key * VP + chunk * 16) = vreg[j];
+            *reinterpret_cast<u32x4 *>(ks[buf] + key * KP + chunk * 16) = kreg[0][j];
+            *reinterpret_cast<u32x4 *>(vs[buf] + key * VP + chunk * 16) = vreg[0][j];
         }
+    };
+    // The same two steps for the ring of P register sets (slot = tile % P, a constant once the loops are unrolled). The
+    // loads are unconditional and sit on no branch, so the compiler can count, per slot, how many younger loads may still
+    // be in flight when a slot is written to LDS, instead of waiting for all of them. A key past the end of the range reads
+    // the first key of the range instead: finite numbers, whose scores are masked and whose probabilities are 0.
+    const int64_t k_safe = k_begin < p.Skv ? k_begin : 0;
+    auto fetch_slot = [&](auto slot, int tile) {
+        static_for<LPT>([&](auto jc) {
+            constexpr int S = decltype(slot)::value, j = decltype(jc)::value;
+            const int key = k_begin + tile * AT_KEYS + key_j0 + j * KSTEP;
+            const int64_t kr = key < k_end ? key : k_safe;
+            kreg[S][j] = *reinterpret_cast<const u32x4 *>(kbase + chunk * 16 + kr * k_pitch);
+            vreg[S][j] = *reinterpret_cast<const u32x4 *>(vbase + chunk * 16 + kr * v_pitch);
+        });
+    };
+    auto stage_slot = [&](auto slot, int buf) {
+        static_for<LPT>([&](auto jc) {
+            constexpr int S = decltype(slot)::value, j = decltype(jc)::value;
+            const int key = key_j0 + j * KSTEP;
+            *reinterpret_cast<u32x4 *>(ks[buf] + key * KP + chunk * 16) = kreg[S][j];
+            *reinterpret_cast<u32x4 *>(vs[buf] + key * VP + chunk * 16) = vreg[S][j];
+        });
     };
     // The transposed V fragments come from the LDS transpose load: the 16 lanes of a group point at 4 keys x 16 head-dim
     // elements (lane j: key j / 4, elements 4 (j % 4) ...) and lane i gets back, for head-dim element i, its 4 keys.
     // This lane's address inside a V tile: key 4 lq + l16 / 4, element 4 (l16 % 4); (u, half, dt) add (32 u + 16 half)
     // keys and 16 dt elements.
     const int v_lane = (4 * lq + (l16 >> 2)) * VP + (l16 & 3) * 8;
-    if (k_begin < k_end) {
-        fetch(k_begin);
-        stage(0);
-        if (k_begin + AT_KEYS < k_end) fetch(k_begin + AT_KEYS);
-    }
-    __syncthreads();
-    int buf = 0;
     // A wavefront multiplies only the tiles some row of its own can see (causal: the block's range ends with the last row
     // of the block); for the tiles behind them it only takes part in the staging and the barriers.
     int wave_lim = my_lim[0];
@@ -204,10 +234,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 #pragma unroll
     for (int r = 0; r < RT; ++r) any_row = any_row || row_ok[r];
     const int k_stop = __any(any_row) ? min(k_end, wave_lim + 1) : k_begin;
-    int k0 = k_begin;
-    for (; k0 < k_stop; k0 += AT_KEYS, buf ^= 1) {
-        const char *kt = ks[buf], *vtile = vs[buf];
-
+    // One tile of 64 keys starting at k0, read from the LDS tiles kt (K) and vtile (V).
+    auto tile_math = [&](const int k0, const char *kt, const char *vtile) {
         // ---- S^T = K Q^T: s[r][t][i] = score of key k0 + 16 t + 4 lq + i against query row r of this lane
         f32x4 s[RT][4];
 #pragma unroll
@@ -311,19 +339,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 #pragma unroll
             for (int r = 0; r < RT; ++r) l_acc[r] = mfma16<DT>(ones, pf[r][u], l_acc[r]);
         }
-        // the next tile into the other buffer (last read one tile ago, before the previous barrier)
-        if (k0 + AT_KEYS < k_end) {
-            stage(buf ^ 1);
-            if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
+    };
+
+    if constexpr (P == 1) {
+        // One register set: the loads of tile i+2 are requested right after tile i+1 went into LDS, and fly during one
+        // tile's MFMAs and softmax. Enough where a CU holds several blocks with long tiles (prefill).
+        if (k_begin < k_end) {
+            fetch(k_begin);
+            stage(0);
+            if (k_begin + AT_KEYS < k_end) fetch(k_begin + AT_KEYS);
         }
         __syncthreads();
-    }
-    for (; k0 < k_end; k0 += AT_KEYS, buf ^= 1) {
-        if (k0 + AT_KEYS < k_end) {
-            stage(buf ^ 1);
-            if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
+        int buf = 0;
+        int k0 = k_begin;
+        for (; k0 < k_stop; k0 += AT_KEYS, buf ^= 1) {
+            tile_math(k0, ks[buf], vs[buf]);
+            // the next tile into the other buffer (last read one tile ago, before the previous barrier)
+            if (k0 + AT_KEYS < k_end) {
+                stage(buf ^ 1);
+                if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
+            }
+            __syncthreads();
         }
+        for (; k0 < k_end; k0 += AT_KEYS, buf ^= 1) {
+            if (k0 + AT_KEYS < k_end) {
+                stage(buf ^ 1);
+                if (k0 + 2 * AT_KEYS < k_end) fetch(k0 + 2 * AT_KEYS);
+            }
+            __syncthreads();
+        }
+    } else {
+        // Few rows (decode): a tile's arithmetic is short, and with one register set a block would wait out one memory
+        // round trip per tile. P sets keep P tiles requested: tile t + 1 goes from its slot into LDS after tile t was
+        // multiplied, and the slot is asked for tile t + 1 + P at once. The loop body is repeated P times so that slots are
+        // compile-time registers; the iterations past the last tile only stage and load harmless repeats.
+        const int n_tiles = k_begin < k_end ? (k_end - k_begin + AT_KEYS - 1) / AT_KEYS : 0;
+        const int n_math = k_begin < k_stop ? (k_stop - k_begin + AT_KEYS - 1) / AT_KEYS : 0;
+        // (also for an empty range, where they read the fallback key: one path into the loop lets the compiler know that
+        // the Q fragments have arrived by then, instead of waiting for every load in flight at the top of each round)
+        static_for<P>([&](auto sl) { fetch_slot(sl, decltype(sl)::value); });
+        stage_slot(Const<0>{}, 0);
+        fetch_slot(Const<0>{}, P);
         __syncthreads();
+        for (int g = 0; g < n_tiles; g += P) {
+            static_for<P>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const int t = g + j;
+                if (t < n_math) tile_math(k_begin + t * AT_KEYS, ks[t & 1], vs[t & 1]);
+                stage_slot(Const<(j + 1) % P>{}, (t + 1) & 1);
+                fetch_slot(Const<(j + 1) % P>{}, t + 1 + P);
+                __syncthreads();
+            });
+        }
     }
 
     // ---- acc[r][dt][i] = O[row r of this lane][d = 16 dt + 4 lq + i]
@@ -407,33 +474,53 @@ int launch(AttnParams p, int cus, hipStream_t s) {
     int dev = 0;
     TPAMD_HIP(hipGetDevice(&dev));
     const int nrows = p.G * p.Sq;
+    constexpr int RING = D == 64 ? 4 : 2;  // tiles requested ahead by the ring kernel: 64 registers either way
+    constexpr int RING_MIN_TILES = 8;      // shorter key ranges: the ring's extra loads and idle rounds cost more than it hides
     // 128 rows per block (two 16-row tiles per wavefront) once that still leaves every CU a few blocks
     const bool wide = nrows >= 128 && static_cast<int64_t>((nrows + 127) / 128) * p.B * p.Hkv >= 2 * cus;
     const int block_rows = wide ? 128 : 64;
     const int row_tiles = (nrows + block_rows - 1) / block_rows;
     const int64_t blocks = static_cast<int64_t>(row_tiles) * p.B * p.Hkv;
-    // split the keys when the rows alone leave CUs idle and there are enough keys to share out
+    // Split the keys when the rows alone leave CUs idle and there are enough keys to share out. Where every CU can get a
+    // block with a long key range (RING_MIN_TILES tiles or more), one block per CU and the ring kernel streams them
+    // (batch 8 on 8192 keys: 20.0 us); otherwise two blocks per CU with at least 128 keys each, for the kernel with one
+    // tile in flight per block (that shape: 23.4 us; batch 8 on 2048 keys: 9.4 us against 11.4 us for 4 ring blocks
+    // of 8 tiles per head).
     int nsplit = 1;
+    bool ring = false;
     if (blocks < 2 * cus) {
-        // two blocks per CU, at least 128 keys per split (four per CU, with half the keys each, was the slower choice
-        // wherever the two differ: batch 8 on 8192 keys 24.2 against 21.1 us)
-        nsplit = static_cast<int>((2 * cus + blocks - 1) / blocks);
-        const int max_by_keys = (p.Skv + 127) / 128;
-        if (nsplit > max_by_keys) nsplit = max_by_keys;
+        const int by_cu = blocks < cus ? static_cast<int>(cus / blocks) : 1;
+        const int by_keys = p.Skv / (RING_MIN_TILES * AT_KEYS);
+        if (by_keys >= by_cu) {
+            ring = true;
+            nsplit = by_cu;
+        } else {
+            nsplit = static_cast<int>((2 * cus + blocks - 1) / blocks);
+            const int max_by_keys = (p.Skv + 127) / 128;
+            if (nsplit > max_by_keys) nsplit = max_by_keys;
+            if (nsplit < 1) nsplit = 1;
+        }
         if (nsplit > 64) nsplit = 64;
-        if (nsplit < 1) nsplit = 1;
     }
-    if (tuning().attn_splits != TUNE_UNSET) nsplit = tuning().attn_splits > 0 ? tuning().attn_splits : 1;
+    if (tuning().attn_splits != TUNE_UNSET) {
+        nsplit = tuning().attn_splits > 0 ? tuning().attn_splits : 1;
+        ring = !wide && p.Skv / nsplit >= RING_MIN_TILES * AT_KEYS;
+    }
+    if (tuning().attn_ring != TUNE_UNSET) ring = !wide && tuning().attn_ring > 0;
     p.keys_per_split = ((p.Skv + nsplit - 1) / nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
     nsplit = (p.Skv + p.keys_per_split - 1) / p.keys_per_split;
     p.nsplit = nsplit;
     p.rows_pad = row_tiles * block_rows;
     TPAMD_REQUIRE(p.B * p.Hkv < 65536 && nsplit < 65536, "attention: batch * kv heads too large for one launch");
     const dim3 grid(row_tiles, p.B * p.Hkv, nsplit);
+    auto run = [&](const AttnParams &prm, dim3 g, bool with_ring) {
+        if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2, 1>), g, dim3(256), 0, s, prm);
+        else if (with_ring) hipLaunchKernelGGL((attention_kernel<DT, D, 1, RING>), g, dim3(256), 0, s, prm);
+        else hipLaunchKernelGGL((attention_kernel<DT, D, 1, 1>), g, dim3(256), 0, s, prm);
+        return hipGetLastError();
+    };
     if (nsplit == 1) {
-        if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2>), grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL((attention_kernel<DT, D, 1>), grid, dim3(256), 0, s, p);
-        TPAMD_HIP(hipGetLastError());
+        TPAMD_HIP(run(p, grid, ring));
         return TPAMD_OK;
     }
     const size_t need = static_cast<size_t>(nsplit) * p.B * p.Hkv * p.rows_pad * (D + 4) * sizeof(float);
@@ -444,15 +531,11 @@ int launch(AttnParams p, int cus, hipStream_t s) {
     if (ws == nullptr) {  // no scratch (first use under stream capture, or more than it holds): one split
         p.nsplit = 1;
         p.keys_per_split = (p.Skv + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
-        if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2>), dim3(row_tiles, p.B * p.Hkv, 1), dim3(256), 0, s, p);
-        else hipLaunchKernelGGL((attention_kernel<DT, D, 1>), dim3(row_tiles, p.B * p.Hkv, 1), dim3(256), 0, s, p);
-        TPAMD_HIP(hipGetLastError());
+        TPAMD_HIP(run(p, dim3(row_tiles, p.B * p.Hkv, 1), p.Skv >= RING_MIN_TILES * AT_KEYS));
         return TPAMD_OK;
     }
     p.part = static_cast<float *>(ws);
-    if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2>), grid, dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((attention_kernel<DT, D, 1>), grid, dim3(256), 0, s, p);
-    TPAMD_HIP(hipGetLastError());
+    TPAMD_HIP(run(p, grid, ring));
     const unsigned cblocks = static_cast<unsigned>((static_cast<int64_t>(nrows) * (D / 4) + 255) / 256);
     hipLaunchKernelGGL((attention_combine_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
     TPAMD_HIP(hipGetLastError());

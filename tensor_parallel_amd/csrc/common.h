@@ -50,6 +50,7 @@ struct Tuning {
     int skinny_xlds;         // TPAMD_SKINNY_XLDS: 0 = gated pair at 4-16 rows through the older kernels
     int gemv_rows;           // TPAMD_GEMV_ROWS: wavefronts per block of the unrolled M <= 3 kernel (2, 4, 8, 16); 0 = the general kernel
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel
+    int attn_ring;           // TPAMD_ATTN_RING: 1 / 0 = the few-row attention kernel with / without several K / V tiles in flight
     int copy_tile_units;     // TPAMD_COPY_TILE_UNITS: 16-byte units per copy tile
     int copy_blocks_per_cu;  // TPAMD_COPY_BLOCKS_PER_CU
     int copy_sort;           // TPAMD_COPY_SORT: 0 = tiles stay in the order of the jobs instead of the order of their source addresses

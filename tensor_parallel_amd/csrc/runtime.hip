@@ -33,6 +33,7 @@ Tuning read_tuning() {
     t.skinny_max_m = env_int("TPAMD_SKINNY_MAX_M");
     t.gemv_rows = env_int("TPAMD_GEMV_ROWS");
     t.attn_splits = env_int("TPAMD_ATTN_SPLITS");
+    t.attn_ring = env_int("TPAMD_ATTN_RING");
     t.copy_tile_units = env_int("TPAMD_COPY_TILE_UNITS");
     t.copy_blocks_per_cu = env_int("TPAMD_COPY_BLOCKS_PER_CU");
     t.copy_sort = env_int("TPAMD_COPY_SORT");

@@ -62,6 +62,30 @@ def test_key_counts_around_the_tile_size(Sq, Skv, causal):
     check(*make(2, 4, 2, Sq, Skv, 64, torch.bfloat16, seed=Sq * 1000 + Skv), causal)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("Skv", [1, 63, 64, 65, 128, 200, 256, 257, 320, 449, 512, 577, 640, 1100])
+@pytest.mark.parametrize("Sq", [1, 40])
+def test_key_counts_with_several_tiles_in_flight(tune, Sq, Skv, D, causal):
+    """The kernel that keeps 4 (head_dim 64) or 2 (128) key tiles requested per block, forced onto short ranges too: 1 to
+    18 tiles, so that the rounds of 4 / 2 end after every possible number of tiles, with full and ragged last tiles."""
+    if causal and Sq > Skv:
+        pytest.skip("more new positions than keys")
+    tune("TPAMD_ATTN_RING", 1)
+    check(*make(2, 4, 2, Sq, Skv, D, torch.float16 if Skv % 2 else torch.bfloat16, seed=Sq * 1000 + Skv), causal)
+
+
+@pytest.mark.parametrize("ring", [0, 1])
+@pytest.mark.parametrize("splits", [1, 3, 8])
+def test_both_few_row_kernels_on_split_key_ranges(tune, ring, splits):
+    """Decode on 2100 keys cut into 1, 3 and 8 ranges (the last one ragged), by the kernel with one tile in flight and by
+    the one with several: the default choice between them depends on the range length, here both take every length."""
+    tune("TPAMD_ATTN_SPLITS", splits)
+    tune("TPAMD_ATTN_RING", ring)
+    check(*make(2, 16, 2, 1, 2100, 64, torch.bfloat16, seed=11), True)
+    check(*make(1, 8, 2, 3, 2100, 128, torch.float16, seed=12), True)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("Sq,causal", [(1, False), (96, False), (96, True)])
 def test_reference_maximum_moves_along_the_keys(dtype, Sq, causal):
