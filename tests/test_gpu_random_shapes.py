@@ -163,3 +163,33 @@ def test_rope_append_random_shape(seed):
     as_bits = lambda t: t.detach().cpu().contiguous().view(torch.int16)  # noqa: E731
     assert torch.equal(as_bits(got_q), as_bits(want_q)), f"B={B} S={S} Hkv={Hkv} per={per} D={D} pos0={pos0}"
     assert torch.equal(as_bits(kcd), as_bits(want_kc)) and torch.equal(as_bits(vcd), as_bits(want_vc))
+
+
+@pytest.mark.parametrize("seed", range(600, 650))
+def test_attention_random_shape(seed):
+    """Random batch, head grouping, new positions, key counts (up to 5000: one block per range, split ranges, and ranges
+    long enough for the kernel that keeps several tiles in flight), head_dim and mask through the default dispatch, q / k /
+    v as strided views of wider buffers, against the float64 oracle."""
+    from oracle import attention as oat
+
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    B, Hkv, G = pick(1, 4), pick(1, 4), [1, 2, 4, 8, 16][pick(0, 4)]
+    D = [64, 128][pick(0, 1)]
+    decode = pick(0, 2) > 0
+    Sq = 1 if decode else pick(2, 150)
+    Skv = pick(max(Sq, 1), 5000 if decode else 700)
+    causal = bool(pick(0, 1))
+    dtype = [torch.bfloat16, torch.float16][pick(0, 1)]
+    Hq = Hkv * G
+    pad = 8 * pick(0, 2)
+    q_wide = torch.randn(B, Hq, Sq, D + pad, generator=g).to(dtype)
+    k_wide = torch.randn(B, Hkv, Skv + pick(0, 5), D, generator=g).to(dtype)
+    v_wide = torch.randn(B, Hkv, Skv, D + pad, generator=g).to(dtype)
+    views = lambda qw, kw, vw: (qw[..., :D], kw[:, :, :Skv], vw[..., pad:])  # noqa: E731
+    q, k, v = views(q_wide, k_wide, v_wide)
+    scale = D ** -0.5 * [1.0, 0.5, 3.0][pick(0, 2)]
+    got = _native.attention(*views(q_wide.to(DEV), k_wide.to(DEV), v_wide.to(DEV)), scale=scale, causal=causal)
+    want = torch.from_numpy(oat.attention_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale, causal))
+    torch.testing.assert_close(got.double().cpu(), want, rtol=RTOL, atol=RTOL * want.std().item(),
+                               msg=lambda m: f"B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Skv={Skv} D={D} causal={causal} {dtype}: {m}")
