@@ -526,7 +526,7 @@ def api_level_extras(torch, dev) -> dict:
         flops = 2 * 6.0 * 4096 * D_MODEL * FFN_SHARD
         out["c2_tp_module_m4096"] = {"us_per_forward": us, "tokens_per_s": 4096 / us * 1e6, "TFLOPs": flops / us / 1e6,
                                      "mfma_frac": flops / us / 1e6 / PEAK_BF16_TFLOPS, "algorithmic_flops": flops,
-                                     "what": "tp.TensorParallel forward, both W=2 rank shards on this GPU (2 rank threads), sum folded into the second rank's down projection"}
+                                     "what": "tp.TensorParallel forward, both W=2 rank shards on this GPU (the ranks take turns on the host), sum folded into the second rank's down projection"}
         del model_tp, x
 
         from transformers import OPTConfig, OPTForCausalLM

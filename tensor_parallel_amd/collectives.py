@@ -11,6 +11,7 @@ before the reduction by the stream itself; the host-side barrier only makes sure
 """
 from __future__ import annotations
 
+import contextvars
 import os
 import threading
 from typing import Any, Callable, List, Optional
@@ -23,11 +24,13 @@ from .slicing import concat_dim
 
 RENDEZVOUS_TIMEOUT_S = 600.0
 
-# Rank threads that share ONE device take turns on the host: a rank holds the "turn" lock while it runs module
-# code and gives it up only while it waits in a collective. All ranks enqueue onto the same device anyway, so
-# nothing is lost, and host-side lazy initialisation inside torch (attention backends, BLAS handles) is never
-# entered by two rank threads at once. The turn of the running forward is published per thread here.
-_turn = threading.local()
+# Ranks that share ONE device take turns on the host: a rank holds the turn while it runs module code and gives it up
+# only while it waits in a collective. All ranks enqueue onto the same device anyway, so nothing is lost, and host-side
+# lazy initialisation inside torch (attention backends, BLAS handles) is never entered by two ranks at once. The ranks
+# are greenlets of the calling thread where the greenlet package is there (a switch costs about a microsecond), else
+# threads (a hand-over through a condition variable costs tens of microseconds, twice per collective). The turn of the
+# running forward is published per rank here: context variables are per thread and per greenlet.
+_turn: contextvars.ContextVar = contextvars.ContextVar("tpamd_turn", default=None)
 
 
 class Turn:
@@ -41,23 +44,49 @@ class Turn:
         self.cond = threading.Condition(self.lock)
         self.failed = False
 
+    def wait(self, timeout: float) -> bool:
+        """Gives the turn away until a peer wakes this rank; False after `timeout` seconds without that."""
+        return self.cond.wait(timeout)
+
+    def wake(self) -> None:
+        """A round of a collective is complete: its waiting ranks may go on when they get the turn."""
+        self.cond.notify_all()
+
     def fail(self) -> None:
         """Called by a failing rank while it holds the lock: wakes every waiting peer."""
         self.failed = True
         self.cond.notify_all()
 
 
-def set_turn_lock(turn: Optional[Turn]) -> None:
-    _turn.turn = turn
-    _turn.lock = turn.lock if turn is not None else None
+class GreenTurn:
+    """The same for ranks that are greenlets of one thread: the turn is whichever greenlet runs. A rank that waits
+    switches to `hub`, the greenlet that started the ranks and hands the turn round (tensor_parallel.parallel_apply_simple);
+    `events` counts completed rounds and finished ranks, which is how the hub sees that the ranks still get anywhere."""
+
+    __slots__ = ("hub", "events", "failed")
+
+    def __init__(self, hub):
+        self.hub = hub
+        self.events = 0
+        self.failed = False
+
+    def wait(self, timeout: float) -> bool:
+        self.hub.switch()
+        return True
+
+    def wake(self) -> None:
+        self.events += 1
+
+    def fail(self) -> None:
+        self.failed = True
 
 
-def current_turn() -> Optional[Turn]:
-    return getattr(_turn, "turn", None)
+def set_turn_lock(turn) -> None:
+    _turn.set(turn)
 
 
-def turn_lock() -> Optional[threading.Lock]:
-    return getattr(_turn, "lock", None)
+def current_turn():
+    return _turn.get()
 
 
 # ---- the sum folded into the last Linear of a row-parallel module -------------------------------------------------
@@ -67,7 +96,7 @@ def turn_lock() -> Optional[threading.Lock]:
 # kernel. A wrapper with such a rule publishes a SumContext for its thread while its module runs; shard Linears
 # consult it (shard_modules.linear_in_context); the op learns from it what the value it is handed already contains.
 FUSE_SUM = os.environ.get("TPAMD_FUSE_SUM", "1") != "0"
-_contexts = threading.local()
+_contexts: contextvars.ContextVar = contextvars.ContextVar("tpamd_sum_contexts", default=None)
 
 
 class SumContext:
@@ -96,31 +125,24 @@ class SumContext:
 
 
 def push_sum_context(ctx: Optional[SumContext]) -> None:
-    stack = getattr(_contexts, "stack", None)
+    stack = _contexts.get()
     if stack is None:
-        stack = _contexts.stack = []
+        stack = []
+        _contexts.set(stack)
     stack.append(ctx)
 
 
 def pop_sum_context() -> None:
-    _contexts.stack.pop()
+    _contexts.get().pop()
 
 
 def current_sum_context() -> Optional[SumContext]:
-    stack = getattr(_contexts, "stack", None)
+    stack = _contexts.get()
     return stack[-1] if stack else None
 
 
 def _rendezvous(barrier: threading.Barrier, timeout: float) -> None:
-    lock = getattr(_turn, "lock", None)
-    if lock is None:
-        barrier.wait(timeout)
-        return
-    lock.release()
-    try:
-        barrier.wait(timeout)
-    finally:
-        lock.acquire()
+    barrier.wait(timeout)
 
 
 class CollectiveOpetationBase:
@@ -143,7 +165,7 @@ class CollectiveOperation(CollectiveOpetationBase):
         self._arrived = 0  # turn-taking ranks: how many have handed in their value this round
         self._round = 0
 
-    def _call_in_turns(self, x: Any, rank: int, turn: Turn):
+    def _call_in_turns(self, x: Any, rank: int, turn):
         """The same exchange for rank threads that take turns on one device (the caller holds the turn lock): a rank
         hands in its value and waits on the turn's condition, which gives the turn away; the rank that arrives last
         runs `func` and wakes the others. One wake-up per waiting rank and collective instead of three barrier rounds.
@@ -162,7 +184,7 @@ class CollectiveOperation(CollectiveOpetationBase):
             self._inputs = [None] * self.world_size
             self._arrived = 0
             self._round += 1
-            turn.cond.notify_all()
+            turn.wake()
         else:
             started = self._round
             while self._round == started:
@@ -170,7 +192,7 @@ class CollectiveOperation(CollectiveOpetationBase):
                     self._inputs[rank] = None
                     self._arrived -= 1
                     raise threading.BrokenBarrierError
-                if not turn.cond.wait(self.timeout):
+                if not turn.wait(self.timeout):
                     self._inputs[rank] = None
                     self._arrived -= 1
                     raise threading.BrokenBarrierError
@@ -231,7 +253,7 @@ class DeviceAllReduce(CollectiveOperation):
         of two is the same in either order). More ranks: the running sum over ranks 0 .. rank-1, once rank-1 has
         handed it in. Only for rank threads that take turns on one device (the waiting value is then complete and
         visible)."""
-        if not self.fusable or turn_lock() is None:
+        if not self.fusable or current_turn() is None:
             return None
         if self.world_size == 2:
             other = 1 - rank

@@ -2,13 +2,17 @@
 (reference: src/tensor_parallel/tensor_parallel.py:26-315).
 
 Construction slices the whole state for all ranks with one launch of the region mover. A forward runs the
-W shards on W host threads, as the reference does (tensor_parallel.py:237-287); the threads meet in the
+W shards side by side on the host, as the reference does with W threads (tensor_parallel.py:237-287): here as W
+greenlets of the calling thread, or W threads where the greenlet package is missing; they meet in the
 "sum" / "gather" ops, which are single-device kernels here. `sharded=True` keeps the parameters the rule table
 leaves replicated as flat per-rank shards (`sharding.Sharded`) and recombines them on the device before a forward.
 """
 from __future__ import annotations
 
+import contextlib
+import functools
 import logging
+import os
 import threading
 from operator import attrgetter
 from typing import Any, Collection, Optional, Sequence, Union
@@ -17,7 +21,7 @@ import torch
 from torch import nn
 
 from .autoconfig import get_default_config
-from .collectives import Turn, set_turn_lock
+from .collectives import GreenTurn, Turn, set_turn_lock
 from .config import Config, add_lora_rules
 from .kv_cache import is_kv_cache, rank_caches
 from .shard import make_shard
@@ -238,6 +242,57 @@ class TensorParallel(nn.Module):
         return destination
 
 
+try:
+    import greenlet as _greenlet
+except ImportError:  # the ranks of a shared device are threads then
+    _greenlet = None
+RANK_GREENLETS = _greenlet is not None and os.environ.get("TPAMD_RANK_GREENLETS", "1") != "0"
+
+
+def _apply_in_greenlets(modules: Sequence[nn.Module], inputs, kwargs_tup, device: torch.device):
+    """The ranks of one device as greenlets of the calling thread. They run on the caller's stream, device and grad mode
+    because they are the caller's thread. A rank runs until it has to wait in a collective, which switches back here;
+    the ranks get the turn in rotation until all have returned. When a whole rotation passes in which no collective
+    completed and no rank finished, the live ranks wait for one that will not come (it has returned or failed): they
+    are told to give up."""
+    hub = _greenlet.getcurrent()
+    turn = GreenTurn(hub)
+    results: dict = {}
+
+    def body(i, module, args, kwargs):
+        set_turn_lock(turn)  # a greenlet starts with an empty context of its own
+        try:
+            if not isinstance(args, (list, tuple)):
+                args = (args,)
+            results[i] = (True, module(*args, **kwargs))
+        except BaseException as e:  # noqa: BLE001 - handed to the caller below
+            results[i] = (False, e)
+            turn.fail()  # its peers must not wait for it
+
+    ranks = [_greenlet.greenlet(functools.partial(body, i, m, a, k), parent=hub)
+             for i, (m, a, k) in enumerate(zip(modules, inputs, kwargs_tup))]
+    alive = list(range(len(ranks)))
+    with torch.cuda.device(device) if device.type == "cuda" else contextlib.nullcontext():
+        position = idle = 0
+        while alive:
+            r = alive[position % len(alive)]
+            before = turn.events
+            ranks[r].switch()
+            if ranks[r].dead:
+                alive.remove(r)
+                turn.events += 1
+            else:
+                position += 1
+            idle = 0 if turn.events != before else idle + 1
+            if idle > len(alive):
+                turn.fail()
+    failures = [results[i] for i in range(len(ranks)) if not results[i][0]]
+    if failures:
+        real = [e for ok, e in failures if not isinstance(e, threading.BrokenBarrierError)]
+        raise (real[0] if real else failures[0][1])
+    return [results[i][1] for i in range(len(ranks))]
+
+
 def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devices: Sequence[torch.device]):
     """Run shard i on (inputs[i], kwargs_tup[i]) in its own thread; re-raise the first failure
     (tensor_parallel.py:237-287)."""
@@ -249,6 +304,8 @@ def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devi
     grad_enabled = torch.is_grad_enabled()
     # ranks that share one device take turns on the host (see collectives.set_turn_lock)
     shared = len(modules) > 1 and all(d.type == "cuda" and d == devices[0] for d in devices)
+    if shared and RANK_GREENLETS:
+        return _apply_in_greenlets(modules, inputs, kwargs_tup, devices[0])
     turn = Turn() if shared else None
     # a thread starts on its device's default stream: the rank threads work on the stream the caller is on instead, so that
     # what the caller enqueued before the forward is ordered before it and what it enqueues afterwards behind it

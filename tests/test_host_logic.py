@@ -402,6 +402,88 @@ def test_a_failing_rank_wakes_the_ranks_that_wait_in_turns():
     assert run(fail_rank=None) == {0: 3, 1: 3, 2: 3}
 
 
+class _Steps(torch.nn.Module):
+    """A rank's module for the greenlet tests: `steps` collectives, host work between them recorded in `log`."""
+
+    def __init__(self, op, rank, steps, log, fail_at=None, leave_at=None):
+        super().__init__()
+        self.op, self.rank, self.steps, self.log, self.fail_at, self.leave_at = op, rank, steps, log, fail_at, leave_at
+
+    def forward(self, x):
+        from tensor_parallel_amd.collectives import current_sum_context, pop_sum_context, push_sum_context
+
+        push_sum_context(("ctx", self.rank))  # the stack of contexts is a rank's own
+        try:
+            for step in range(self.steps):
+                self.log.append((self.rank, step))
+                if step == self.fail_at:
+                    raise ValueError(f"rank {self.rank} fails")
+                if step == self.leave_at:
+                    return x
+                x = x + self.op(self.rank + step, self.rank)
+                assert current_sum_context() == ("ctx", self.rank)
+            return x
+        finally:
+            pop_sum_context()
+
+
+greenlets = pytest.mark.skipif(not __import__("tensor_parallel_amd.tensor_parallel", fromlist=["x"]).RANK_GREENLETS,
+                               reason="the greenlet package is not there: the ranks of a device are threads")
+
+
+@greenlets
+def test_ranks_as_greenlets_take_turns_and_meet_in_collectives():
+    from tensor_parallel_amd.collectives import CollectiveOperation, current_turn
+    from tensor_parallel_amd.tensor_parallel import _apply_in_greenlets
+
+    world, steps, log = 3, 4, []
+    op = CollectiveOperation(world, lambda *xs: [sum(xs)] * world, timeout=5.0)
+    mods = [_Steps(op, r, steps, log) for r in range(world)]
+    for _ in range(2):  # the op is ready for the next forward
+        out = _apply_in_greenlets(mods, [(10 * r,) for r in range(world)], [{}] * world, torch.device("cpu"))
+        want = sum(sum(r + step for r in range(world)) for step in range(steps))
+        assert out == [10 * r + want for r in range(world)]
+    # a rank runs until its next collective, then the next one gets the turn: every step is entered by all ranks before
+    # any rank enters the step after it
+    first = log[:world * steps]
+    assert [step for _, step in first] == sorted(step for _, step in first)
+    assert current_turn() is None  # nothing leaks into the caller's context
+
+
+@greenlets
+def test_a_failing_greenlet_rank_frees_its_peers_and_the_next_forward_works():
+    import threading
+
+    from tensor_parallel_amd.collectives import CollectiveOperation
+    from tensor_parallel_amd.tensor_parallel import _apply_in_greenlets
+
+    world, log = 3, []
+    op = CollectiveOperation(world, lambda *xs: [sum(xs)] * world, timeout=5.0)
+    bad = [_Steps(op, r, 3, log, fail_at=1 if r == 1 else None) for r in range(world)]
+    with pytest.raises(ValueError, match="rank 1 fails"):
+        _apply_in_greenlets(bad, [(0,)] * world, [{}] * world, torch.device("cpu"))
+    good = [_Steps(op, r, 3, log) for r in range(world)]
+    assert _apply_in_greenlets(good, [(0,)] * world, [{}] * world, torch.device("cpu")) == [18] * world
+    # a rank that returns without taking part in a collective its peers wait in: they are told to give up at once
+    early = [_Steps(op, r, 3, log, leave_at=2 if r == 0 else None) for r in range(world)]
+    with pytest.raises(threading.BrokenBarrierError):
+        _apply_in_greenlets(early, [(0,)] * world, [{}] * world, torch.device("cpu"))
+    assert _apply_in_greenlets(good, [(0,)] * world, [{}] * world, torch.device("cpu")) == [18] * world
+
+
+@greenlets
+def test_a_collective_whose_function_raises_raises_on_every_greenlet_rank():
+    from tensor_parallel_amd.collectives import CollectiveOperation
+    from tensor_parallel_amd.tensor_parallel import _apply_in_greenlets
+
+    def boom(*xs):
+        raise KeyError("bad values")
+
+    op = CollectiveOperation(2, boom, timeout=5.0)
+    with pytest.raises(KeyError, match="bad values"):
+        _apply_in_greenlets([_Steps(op, r, 1, []) for r in range(2)], [(0,)] * 2, [{}] * 2, torch.device("cpu"))
+
+
 def test_a_collective_whose_function_raises_raises_on_every_rank_in_turns():
     import threading
 
