@@ -222,10 +222,37 @@ def main() -> int:
     }
     if not args.no_extra:
         out["extra"] = extra_measurements(torch, _native, dev, sets, other)
+        out["extra"]["copy_bandwidth"] = copy_bandwidth(torch, _native, dev)
+        add_copy_fractions(out["extra"], out["extra"]["copy_bandwidth"]["GBps"])
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(M)
     print(json.dumps(out), flush=True)
     return 0
+
+
+def copy_bandwidth(torch, _native, dev) -> dict:
+    """What a plain copy reaches on this part, as the second yardstick beside the published 8 TB/s: 1 GiB moved to another
+    1 GiB buffer (bytes read + written per second) by torch's `copy_` and by the library's region mover as one job of
+    8192 rows; `GBps` is the better of the two."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).random_()
+    dst = torch.empty_like(src)
+    t_torch = _time_us(torch, lambda i: dst.copy_(src), 3, 10)
+    job = [(src.data_ptr(), dst.data_ptr(), 8192, n // 8192, n // 8192, n // 8192)]
+    t_lib = _time_us(torch, lambda i: _native.run_copy_jobs(job, dev), 3, 10)
+    torch.cuda.synchronize()
+    assert torch.equal(src[-4096:], dst[-4096:])
+    both = {"torch_copy_GBps": 2.0 * n / t_torch / 1e3, "region_mover_GBps": 2.0 * n / t_lib / 1e3}
+    return {**both, "GBps": max(both.values()), "bytes_each_way": n}
+
+
+def add_copy_fractions(tree, copy_gbps: float) -> None:
+    """Beside every `hbm_frac` (of the published 8 TB/s) the same figure as a fraction of the measured copy bandwidth."""
+    if isinstance(tree, dict):
+        if "hbm_frac" in tree and "GBps" in tree:
+            tree["copy_frac"] = tree["GBps"] / copy_gbps
+        for value in tree.values():
+            add_copy_fractions(value, copy_gbps)
 
 
 def _graph_us(torch, fn, per=30, reps=10):
