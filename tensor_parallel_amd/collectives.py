@@ -296,5 +296,6 @@ class DeviceAllGather(CollectiveOperation):
     def _gather(self, *parts: torch.Tensor):
         for p in parts:
             _native.require_device(p, "gather")
-        out = concat_dim([p.detach() for p in parts], self.dim)
-        return [_guard(o, *parts) for o in [out] + [out.clone() for _ in range(self.world_size - 1)]]
+        # each rank continues with a tensor of its own, all written by the same launch where their jobs fit one
+        outs = concat_dim([p.detach() for p in parts], self.dim, copies=self.world_size)
+        return [_guard(o, *parts) for o in (outs if self.world_size > 1 else [outs])]

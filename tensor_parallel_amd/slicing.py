@@ -141,30 +141,42 @@ def apply_spec(t: torch.Tensor, spec: SliceSpec, device: Optional[torch.device] 
     return out
 
 
-def concat_specs(parts: Sequence[torch.Tensor], specs: Sequence[SliceSpec]) -> torch.Tensor:
-    """Inverse of slicing: scatter every part back to the ranges its spec names, giving the full tensor."""
+def concat_specs(parts: Sequence[torch.Tensor], specs: Sequence[SliceSpec], copies: int = 1):
+    """Inverse of slicing: scatter every part back to the ranges its spec names, giving the full tensor. With
+    `copies` > 1: a list of that many separate full tensors (one per rank of a gather), written by as few launches as
+    their jobs fit into."""
     if len(parts) != len(specs) or not parts:
         raise ValueError("concat_specs: need one spec per part")
     full_shape = specs[0].shape
     first = parts[0]
     if first.device.type == "meta":
-        return torch.empty(full_shape, dtype=first.dtype, device="meta")
+        outs = [torch.empty(full_shape, dtype=first.dtype, device="meta") for _ in range(copies)]
+        return outs[0] if copies == 1 else outs
     dev_parts = [_device_source(p, None if first.device.type != "cuda" else first.device) for p in parts]
     device = dev_parts[0].device
-    out = torch.empty(full_shape, dtype=first.dtype, device=device)
-    jobs: List[tuple] = []
     for p, spec in zip(dev_parts, specs):
         if tuple(p.shape) != spec.out_shape:
             raise ValueError(f"part has shape {tuple(p.shape)}, its spec expects {spec.out_shape}")
         if p.device != device or p.dtype != first.dtype:
             raise ValueError("concat_specs: parts must share device and dtype")
-        jobs += copy_jobs(spec, p.element_size(), out.data_ptr(), p.data_ptr(), scatter=True)
+    outs = [torch.empty(full_shape, dtype=first.dtype, device=device) for _ in range(copies)]
+    jobs: List[tuple] = []
+    for out in outs:
+        mine: List[tuple] = []
+        for p, spec in zip(dev_parts, specs):
+            mine += copy_jobs(spec, p.element_size(), out.data_ptr(), p.data_ptr(), scatter=True)
+        # the jobs of several copies share a launch while they fit the kernel's argument list
+        if jobs and len(jobs) + len(mine) > _native.SMALL_COPY_MAX_JOBS:
+            _native.run_copy_jobs(jobs, device)
+            jobs = []
+        jobs += mine
     _native.run_copy_jobs(jobs, device)
-    return out
+    return outs[0] if copies == 1 else outs
 
 
-def concat_dim(parts: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
-    """torch.cat(parts, dim) through the region mover (parts may have different lengths on `dim`)."""
+def concat_dim(parts: Sequence[torch.Tensor], dim: int, copies: int = 1):
+    """torch.cat(parts, dim) through the region mover (parts may have different lengths on `dim`); `copies` as in
+    concat_specs."""
     first = parts[0]
     d = normalize_dim(dim, first.dim())
     total = sum(p.shape[d] for p in parts)
@@ -174,7 +186,7 @@ def concat_dim(parts: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
     for p in parts:
         specs.append(SliceSpec(tuple(full_shape), d, ((at, p.shape[d]),)))
         at += p.shape[d]
-    return concat_specs(parts, specs)
+    return concat_specs(parts, specs, copies)
 
 
 class BatchSlicer:
