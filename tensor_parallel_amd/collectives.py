@@ -2,7 +2,7 @@
 
 The reference rendezvouses W rank threads and moves data between devices
 (src/tensor_parallel/communications.py:21-171, cross_device_ops.py:30-50). Here the W partials are already
-on the same GPU: the threads still rendezvous (an op object is called as `op(x, rank)` from W threads, as
+on the same GPU: the ranks still rendezvous (an op object is called as `op(x, rank)` by each of the W ranks, as
 in the reference, communications.py:16-18), but the work is one kernel launch: a W-way elementwise sum
 (`tpamd_reduce_partials`) or a concatenation done by the region mover. No inter-GPU collective exists.
 
@@ -93,14 +93,14 @@ def current_turn():
 # A module whose output rule is "sum" usually ends in its row-parallel Linear (attention output projection, MLP down
 # projection). The rank that reaches that Linear while the partials of the other ranks are already waiting in the op
 # can add them in the GEMM's epilogue (`tpamd_linear_add`) instead of leaving a separate M x N pass to the reduction
-# kernel. A wrapper with such a rule publishes a SumContext for its thread while its module runs; shard Linears
+# kernel. A wrapper with such a rule publishes a SumContext for its rank while its module runs; shard Linears
 # consult it (shard_modules.linear_in_context); the op learns from it what the value it is handed already contains.
 FUSE_SUM = os.environ.get("TPAMD_FUSE_SUM", "1") != "0"
 _contexts: contextvars.ContextVar = contextvars.ContextVar("tpamd_sum_contexts", default=None)
 
 
 class SumContext:
-    """One call of a wrapped module whose output 0 goes to `op`, on one rank thread."""
+    """One call of a wrapped module whose output 0 goes to `op`, on one rank."""
 
     __slots__ = ("op", "rank", "owner", "last_linear", "last_out", "calls", "fused_out", "fused_mask")
 
@@ -166,8 +166,8 @@ class CollectiveOperation(CollectiveOpetationBase):
         self._round = 0
 
     def _call_in_turns(self, x: Any, rank: int, turn):
-        """The same exchange for rank threads that take turns on one device (the caller holds the turn lock): a rank
-        hands in its value and waits on the turn's condition, which gives the turn away; the rank that arrives last
+        """The same exchange for ranks that take turns on one device (the caller holds the turn): a rank
+        hands in its value and waits on the turn, which gives it away; the rank that arrives last
         runs `func` and wakes the others. One wake-up per waiting rank and collective instead of three barrier rounds.
         The results of a round stay in place until the next round of this op completes, which needs every rank to have
         come back, so nobody can miss its result."""
@@ -251,7 +251,7 @@ class DeviceAllReduce(CollectiveOperation):
         """(tensor, ranks it covers as a bit mask) that rank `rank`'s last Linear may add to its own partial so that
         the result is a step of the rank-ordered sum, or None. Two ranks: whatever the other rank has handed in (a sum
         of two is the same in either order). More ranks: the running sum over ranks 0 .. rank-1, once rank-1 has
-        handed it in. Only for rank threads that take turns on one device (the waiting value is then complete and
+        handed it in. Only for ranks that take turns on one device (the waiting value is then complete and
         visible)."""
         if not self.fusable or current_turn() is None:
             return None

@@ -294,8 +294,8 @@ def _apply_in_greenlets(modules: Sequence[nn.Module], inputs, kwargs_tup, device
 
 
 def parallel_apply_simple(modules: Sequence[nn.Module], inputs, kwargs_tup, devices: Sequence[torch.device]):
-    """Run shard i on (inputs[i], kwargs_tup[i]) in its own thread; re-raise the first failure
-    (tensor_parallel.py:237-287)."""
+    """Run shard i on (inputs[i], kwargs_tup[i]), all shards side by side (greenlets of this thread when they share a
+    device and the greenlet package is there, else a thread each); re-raise the first failure (tensor_parallel.py:237-287)."""
     assert len(modules) == len(inputs)
     kwargs_tup = kwargs_tup if kwargs_tup is not None else ({},) * len(modules)
     assert len(modules) == len(kwargs_tup)
