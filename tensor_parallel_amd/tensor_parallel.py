@@ -23,6 +23,7 @@ from torch import nn
 from .autoconfig import get_default_config
 from .collectives import GreenTurn, Turn, set_turn_lock
 from .config import Config, add_lora_rules
+from .int8 import ShardLinearW8
 from .kv_cache import is_kv_cache, rank_caches
 from .shard import make_shard
 from .sharding import Sharded
@@ -209,6 +210,9 @@ class TensorParallel(nn.Module):
         if self.preserve_shards_when_saving or len(self.module_shards) <= 1:
             return state_dict
         world_size = len(self.module_shards)
+        if any(isinstance(m, ShardLinearW8) for m in self.module_shards[0].modules()):
+            raise RuntimeError("tensor_parallel_amd: full weights cannot be rebuilt from int8 Linears (int8.quantize_linears_); "
+                               "save the shards as they are (outside save_tensor_parallel)")
         for name in [n for n in state_dict if "_sanity_check_params." in n]:
             del state_dict[name]
         for name in [n for n in state_dict if "tp_wrapped_module." in n]:

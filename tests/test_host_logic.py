@@ -762,3 +762,18 @@ def test_sum_op_hands_out_only_running_sums_in_rank_order(monkeypatch):
         assert DeviceAllReduce(2, accum=_native.ACCUM_F32).fusable is False
     finally:
         set_turn_lock(None)
+
+
+def test_int8_step_refuses_host_tensors_and_leaves_host_modules_alone():
+    """The quantiser computes on the device only; Linears whose weights live on the host are not touched."""
+    from tensor_parallel_amd import _native
+    from tensor_parallel_amd.int8 import ShardLinearW8, quantize_linears_, quantize_rows
+
+    with pytest.raises(_native.NativeLibraryError):
+        quantize_rows(torch.randn(4, 16, dtype=torch.float16))
+    block = nn.Sequential(nn.Linear(16, 8), nn.ReLU(), nn.Linear(8, 4)).to(torch.float16)
+    assert quantize_linears_(block) == 0
+    assert not any(isinstance(m, ShardLinearW8) for m in block.modules())
+    with pytest.raises(TypeError):
+        ShardLinearW8(torch.zeros(4, 16, dtype=torch.int8), torch.ones(4), torch.zeros(0, dtype=torch.int32),
+                      torch.zeros(4, 0), None, torch.float32)
