@@ -777,3 +777,15 @@ def test_int8_step_refuses_host_tensors_and_leaves_host_modules_alone():
     with pytest.raises(TypeError):
         ShardLinearW8(torch.zeros(4, 16, dtype=torch.int8), torch.ones(4), torch.zeros(0, dtype=torch.int32),
                       torch.zeros(4, 0), None, torch.float32)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU's share: asking for more exits with a message that says so, before anything is
+    imported or measured."""
+    import subprocess
+    import sys
+
+    root = Path(__file__).resolve().parents[1]
+    res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 2 and res.stdout == ""
+    assert "--gpus above 1 is not supported" in res.stderr
