@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TPAMD_ABI_VERSION 3
+#define TPAMD_ABI_VERSION 4
 
 typedef enum tpamd_status {
     TPAMD_OK = 0,
@@ -257,6 +257,28 @@ int tpamd_attention(const void *q_dev, const void *k_dev, const void *v_dev, voi
 int tpamd_rope_append(const void *q_dev, const void *k_dev, const void *v_dev, const void *cos_dev, const void *sin_dev,
                       void *q_out_dev, void *k_cache_dev, void *v_cache_dev, int64_t B, int64_t S, int64_t Hq, int64_t Hkv,
                       int64_t D, int64_t pos0, int64_t cache_len, const int64_t *strides, int dtype, void *stream);
+
+/* Decode step of the same call site with tpamd_rope_append and tpamd_attention in one: one new position per sequence
+ * on a rank-local cache that holds pos0 positions (reference: the wrapped attention module's torch ops, as for the two
+ * entry points above; src/tensor_parallel/wrapper.py:69-72, aux_actions.py:7-15, slicing_configs.py:430-461).
+ *   q [B, Hq, D], k / v [B, Hkv, D]: the new position's raw rows, views of the projection output (query head h at
+ *   (h / g) * "q group" + (h % g) * "q head", g = Hq / Hkv); cos / sin [B or 1, D];
+ *   k_cache / v_cache [B, Hkv, cache_len, D]: positions 0 .. pos0 - 1 are read, position pos0 receives the rotated key
+ *   and the value (the same bits tpamd_rope_append writes);
+ *   out [B, Hq, D] = softmax(scale * rot(q) . [cache keys, rot(k)]^T) [cache values, v].
+ * Two launches instead of three: the attention kernel rotates its query fragments itself and leaves one partial result
+ * per key range of the cache; the merge adds the new position (its score in fp32 from the rotated rows) and writes the
+ * cache rows. Rounding differs from the two-call sequence only in that the new position's probability is not rounded to
+ * `dtype` before it weighs its value.
+ *   strides: 16 element strides, {q batch, q head, q group, k batch, k head, v batch, v head, cos/sin batch (0 when
+ *   shared), k_cache batch, k_cache head, k_cache position, v_cache batch, v_cache head, v_cache position, out batch,
+ *   out head}; the first 14 multiples of 8, the last two of 4; pointers 16-byte aligned (out: 8).
+ * Needs the stream's scratch buffer for the partial results: TPAMD_ERR_UNSUPPORTED when there is none (the stream's
+ * first use of it under capture, or a batch too large for it); callers then use the two entry points above. */
+int tpamd_attention_decode_rope(const void *q_dev, const void *k_dev, const void *v_dev, const void *cos_dev,
+                                const void *sin_dev, void *k_cache_dev, void *v_cache_dev, void *out_dev, int64_t B,
+                                int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0, int64_t cache_len, const int64_t *strides,
+                                float scale, int dtype, void *stream);
 
 /* Weight-only int8 shard Linear with fp16/bf16 outlier columns:
  *   y[m,n] = act( scale[n] * sum_k x[m,k]*wq[n,k]  +  sum_j x[m,outlier_idx[j]] * w_out[n,j]  + bias[n] )

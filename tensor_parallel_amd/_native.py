@@ -37,9 +37,10 @@ EXPORTS = (
     "tpamd_linear_w8",
     "tpamd_attention",
     "tpamd_rope_append",
+    "tpamd_attention_decode_rope",
 )
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 BF16, F16, F32 = 0, 1, 2
 ACCUM_STEPWISE, ACCUM_F32 = 0, 1
@@ -119,6 +120,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_swiglu_up.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
     lib.tpamd_attention.restype = ci
     lib.tpamd_attention.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, c.POINTER(i64), c.c_float, ci, ci, vp]
+    lib.tpamd_attention_decode_rope.restype = ci
+    lib.tpamd_attention_decode_rope.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, c.POINTER(i64), c.c_float, ci, vp]
     lib.tpamd_rope_append.restype = ci
     lib.tpamd_rope_append.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, c.POINTER(i64), ci, vp]
     lib.tpamd_linear_w8.restype = ci
@@ -536,6 +539,56 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
             "tpamd_rope_append",
         )
     return q_out
+
+
+def attention_decode_rope(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                          k_cache: torch.Tensor, v_cache: torch.Tensor, pos0: int, scale: Optional[float] = None,
+                          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`rope_append` and `attention` for one new position per sequence, in two launches instead of three.
+    q [B, 1, Hq, D] or [B, 1, Hkv, Hq / Hkv, D], k / v [B, 1, Hkv, D] (views of the projection output), cos / sin [B or 1, 1, D]
+    (or [1, D] / [D]); the caches [B, Hkv, L, D] hold pos0 positions and receive the new one at pos0. Returns [B, 1, Hq, D].
+    Where the library has no scratch buffer for the stream (first use under graph capture) the two calls are made instead."""
+    require_device(q, "attention_decode_rope")
+    if not (q.dtype == k.dtype == v.dtype == cos.dtype == sin.dtype == k_cache.dtype == v_cache.dtype) or q.dtype not in (
+            torch.bfloat16, torch.float16):
+        raise TypeError("attention_decode_rope: every tensor must share bfloat16 or float16")
+    if q.dim() not in (4, 5) or k.dim() != 4 or v.shape != k.shape or q.shape[:2] != k.shape[:2] or k.shape[1] != 1 or \
+            q.shape[-1] != k.shape[3] or (q.dim() == 5 and q.shape[2] != k.shape[2]):
+        raise ValueError(f"attention_decode_rope: shapes q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} do not fit one new position")
+    B, _, Hkv, D = k.shape
+    Hq = q.shape[2] if q.dim() == 4 else q.shape[2] * q.shape[3]
+    if Hq % Hkv:
+        raise ValueError(f"attention_decode_rope: {Hq} query heads over {Hkv} key/value heads")
+    q_head, q_group = (q.stride(2), q.stride(2) * (Hq // Hkv)) if q.dim() == 4 else (q.stride(3), q.stride(2))
+    cos, sin = cos.reshape(-1, D), sin.reshape(-1, D)
+    if cos.shape != sin.shape or cos.shape[0] not in (1, B):
+        raise ValueError(f"attention_decode_rope: cos / sin must hold [{B} or 1] rows of {D}, got {tuple(cos.shape)} / {tuple(sin.shape)}")
+    if k_cache.dim() != 4 or v_cache.shape != k_cache.shape or k_cache.shape[0] != B or k_cache.shape[1] != Hkv or k_cache.shape[3] != D:
+        raise ValueError(f"attention_decode_rope: caches must be [{B}, {Hkv}, L, {D}], got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    for name, t in (("q", q), ("k", k), ("v", v), ("cos", cos), ("sin", sin), ("k_cache", k_cache), ("v_cache", v_cache)):
+        if t.device != q.device:
+            raise ValueError(f"attention_decode_rope: q is on {q.device}, {name} on {t.device}")
+        if t.stride(-1) != 1:
+            raise ValueError(f"attention_decode_rope: {name} must have contiguous rows")
+    if sin.stride() != cos.stride():
+        sin, cos = sin.contiguous(), cos.contiguous()
+    if out is None:
+        out = torch.empty((B, 1, Hq, D), dtype=q.dtype, device=q.device)
+    elif out.shape != (B, 1, Hq, D) or out.dtype != q.dtype or out.device != q.device or out.stride(3) != 1:
+        raise ValueError(f"attention_decode_rope: out must be a [{B}, 1, {Hq}, {D}] {q.dtype} tensor on {q.device} with contiguous rows")
+    strides = (ctypes.c_int64 * 16)(q.stride(0), q_head, q_group, k.stride(0), k.stride(2), v.stride(0), v.stride(2),
+                                    cos.stride(0) if cos.shape[0] > 1 else 0, k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+                                    v_cache.stride(0), v_cache.stride(1), v_cache.stride(2), out.stride(0), out.stride(2))
+    with _on_device(q.device):
+        rc = lib().tpamd_attention_decode_rope(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                               k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, int(pos0),
+                                               k_cache.shape[2], strides, float(scale if scale is not None else D ** -0.5),
+                                               dtype_code(q.dtype), ctypes.c_void_p(current_stream_ptr(q.device)))
+    if rc == -2 and B > 0 and D in (64, 128):  # no scratch buffer for this stream: the two-call sequence needs none
+        q_rot = rope_append(q, k, v, cos.unsqueeze(1), sin.unsqueeze(1), k_cache, v_cache, pos0)
+        return attention(q_rot, k_cache[:, :, :pos0 + 1], v_cache[:, :, :pos0 + 1], scale=scale, causal=True, out=out)
+    _check(rc, "tpamd_attention_decode_rope")
+    return out
 
 
 def linear_w8(x: torch.Tensor, wq: torch.Tensor, scale_: torch.Tensor, outlier_idx: Optional[torch.Tensor],

@@ -28,6 +28,9 @@ int gemm_w8_dispatch(const void *x, const void *wq, const void *scale, const voi
 
 int attention_dispatch(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq,
                        int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal, int dtype, hipStream_t s);
+int attention_decode_rope_dispatch(const void *q, const void *k, const void *v, const void *cos, const void *sin, void *k_cache,
+                                   void *v_cache, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0,
+                                   const int64_t *strides, float scale, int dtype, hipStream_t s);
 
 namespace {
 
@@ -160,6 +163,32 @@ extern "C" int tpamd_attention(const void *q_dev, const void *k_dev, const void 
     }
     return attention_dispatch(q_dev, k_dev, v_dev, out_dev, B, Hq, Hkv, Sq, Skv, D, strides, scale, causal, dtype,
                               static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tpamd_attention_decode_rope(const void *q_dev, const void *k_dev, const void *v_dev, const void *cos_dev,
+                                           const void *sin_dev, void *k_cache_dev, void *v_cache_dev, void *out_dev, int64_t B,
+                                           int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0, int64_t cache_len,
+                                           const int64_t *strides, float scale, int dtype, void *stream) {
+    const char *who = "tpamd_attention_decode_rope";
+    TPAMD_REQUIRE(dtype == TPAMD_BF16 || dtype == TPAMD_F16, "%s: dtype must be BF16 or F16", who);
+    TPAMD_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0, "%s: bad dimension", who);
+    TPAMD_REQUIRE(Hq % Hkv == 0, "%s: %lld query heads are not a multiple of %lld key/value heads", who, (long long)Hq, (long long)Hkv);
+    TPAMD_REQUIRE(pos0 >= 0 && pos0 < cache_len, "%s: position %lld does not fit a cache of %lld positions", who, (long long)pos0,
+                  (long long)cache_len);
+    TPAMD_REQUIRE(strides != nullptr, "%s: strides is NULL", who);
+    if (B == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(q_dev && k_dev && v_dev && cos_dev && sin_dev && k_cache_dev && v_cache_dev && out_dev, "%s: null pointer", who);
+    TPAMD_REQUIRE(Hq / Hkv < (1ll << 20) && pos0 < (1ll << 30), "%s: sequence too long", who);
+    bool ok = (D == 64 || D == 128) && aligned(q_dev, 16) && aligned(k_dev, 16) && aligned(v_dev, 16) && aligned(cos_dev, 16) &&
+              aligned(sin_dev, 16) && aligned(k_cache_dev, 16) && aligned(v_cache_dev, 16) && aligned(out_dev, 8);
+    for (int i = 0; i < 14; ++i) ok = ok && strides[i] % 8 == 0;   // 16-byte loads of every row
+    for (int i = 14; i < 16; ++i) ok = ok && strides[i] % 4 == 0;  // 8-byte stores
+    if (!ok) {
+        set_error("%s: head_dim must be 64 or 128 and rows 16-byte aligned", who);
+        return TPAMD_ERR_UNSUPPORTED;
+    }
+    return attention_decode_rope_dispatch(q_dev, k_dev, v_dev, cos_dev, sin_dev, k_cache_dev, v_cache_dev, out_dev, B, Hq, Hkv, D,
+                                          pos0, strides, scale, dtype, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,

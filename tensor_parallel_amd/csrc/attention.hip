@@ -67,6 +67,14 @@ struct AttnParams {
     float scale_log2;  // scale * log2(e)
     int causal;        // query position sq sees keys j <= sq + (Skv - Sq)
     int nsplit, keys_per_split, rows_pad;
+    int64_t q_sg;  // elements between the first query heads of consecutive key/value heads (G * q_sh for a plain [B, Hq, Sq, D])
+    // Decode with the rotary embedding folded in (Sq = 1; tpamd_attention_decode_rope): q, new_k, new_v are the raw rows of
+    // the projection output, cos / sin [B or 1, D]; the kernel rotates its Q fragments, always leaves partials, and the merge
+    // adds the new position's key and value and writes them to the caches (k, v above) at position Skv.
+    const char *cos, *sin, *new_k, *new_v;
+    char *k_cache_w, *v_cache_w;  // k and v above, writable
+    int64_t cs_b, nk_sb, nk_sh, nv_sb, nv_sh;
+    int force_partials;
 };
 
 constexpr int AT_KEYS = 64;   // keys per tile
@@ -123,10 +131,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         sq[r] = row_ok[r] ? row[r] % p.Sq : 0;
         head[r] = hkv * p.G + g;
         my_lim[r] = p.causal ? sq[r] + shift : p.Skv - 1;  // last key this row may see
-        const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(head[r]) * p.q_sh + static_cast<int64_t>(sq[r]) * p.q_ss) * 2;
+        const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(hkv) * p.q_sg + static_cast<int64_t>(g) * p.q_sh + static_cast<int64_t>(sq[r]) * p.q_ss) * 2;
 #pragma unroll
         for (int kk = 0; kk < DK; ++kk)
             qf[r][kk] = *reinterpret_cast<const uint4 *>(qrow + (32 * kk + 8 * lq) * 2);  // rows past the end: row 0 of the group, never stored
+        if (p.cos != nullptr) {
+            // rotary embedding of the row, as rope_append_kernel does it: element d of the first half pairs with d + D / 2,
+            // which is fragment kk + DK / 2 of the same lane
+            const char *cs = p.cos + static_cast<int64_t>(b) * p.cs_b * 2, *sn = p.sin + static_cast<int64_t>(b) * p.cs_b * 2;
+#pragma unroll
+            for (int kk = 0; kk < DK / 2; ++kk) {
+                const int at = (32 * kk + 8 * lq) * 2;
+                const uint4 x1 = qf[r][kk], x2 = qf[r][kk + DK / 2];
+                const uint4 c1 = *reinterpret_cast<const uint4 *>(cs + at), c2 = *reinterpret_cast<const uint4 *>(cs + at + D);
+                const uint4 s1 = *reinterpret_cast<const uint4 *>(sn + at), s2 = *reinterpret_cast<const uint4 *>(sn + at + D);
+                qf[r][kk] = rot8<DT>(x1, c1, x2, s1, -1.0f);
+                qf[r][kk + DK / 2] = rot8<DT>(x2, c2, x1, s2, 1.0f);
+            }
+        }
     }
 
     // ---- key range of this block
@@ -397,7 +419,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
         if (!row_ok[r]) continue;
-        if (p.nsplit == 1) {
+        if (p.nsplit == 1 && !p.force_partials) {
             const float l_row = l_acc[r][0];
             const float inv = l_row > 0.f ? 1.0f / l_row : 0.f;
             char *orow = p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(sq[r]) * p.o_ss + static_cast<int64_t>(head[r]) * p.o_sh) * 2;
@@ -469,6 +491,84 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(AttnParams p) {
     *reinterpret_cast<uint2 *>(p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(sq) * p.o_ss + static_cast<int64_t>(head) * p.o_sh + d4) * 2) = o2;
 }
 
+// The merge for decode with the rotary embedding folded in (Sq = 1): the splits over the cached keys (none when the
+// cache is empty), plus the new position. A row's D / 4 threads (consecutive lanes of one wavefront) rotate their 4
+// elements of the raw query and key rows exactly as rope_append_kernel does, meet for the dot product, and merge
+// (score, 1, v) as one more partial in fp32; the threads of a group's first head also write the rotated key and the
+// value into the caches at position Skv.
+template <int DT, int D>
+__global__ __launch_bounds__(256) void attention_combine_newkey_kernel(AttnParams p) {
+    constexpr int per_row = D / 4;
+    const int nrows = p.G;  // Sq = 1: a row is a query head of the group
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / p.Hkv, hkv = bh % p.Hkv;
+    // threads past the last row work on row 0 (they take part in the shuffles) and store nothing
+    const bool live = e < nrows * per_row;
+    const int row = live ? e / per_row : 0, d4 = (e % per_row) * 4;
+    const bool lower = d4 < D / 2;
+    const int partner = lower ? d4 + D / 2 : d4 - D / 2;
+    const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(hkv) * p.q_sg + static_cast<int64_t>(row) * p.q_sh) * 2;
+    const char *krow = p.new_k + (static_cast<int64_t>(b) * p.nk_sb + static_cast<int64_t>(hkv) * p.nk_sh) * 2;
+    const char *vrow = p.new_v + (static_cast<int64_t>(b) * p.nv_sb + static_cast<int64_t>(hkv) * p.nv_sh) * 2;
+    const char *cs = p.cos + static_cast<int64_t>(b) * p.cs_b * 2, *sn = p.sin + static_cast<int64_t>(b) * p.cs_b * 2;
+    const uint2 c = *reinterpret_cast<const uint2 *>(cs + d4 * 2), sv = *reinterpret_cast<const uint2 *>(sn + d4 * 2);
+    const float sign = lower ? -1.0f : 1.0f;  // rotate_half(x) = cat(-x[D/2:], x[:D/2])
+    auto rotated = [&](const char *r) {
+        const uint2 own = *reinterpret_cast<const uint2 *>(r + d4 * 2), oth = *reinterpret_cast<const uint2 *>(r + partner * 2);
+        return make_uint2(rot2<DT>(own.x, c.x, oth.x, sv.x, sign), rot2<DT>(own.y, c.y, oth.y, sv.y, sign));
+    };
+    const uint2 qr = rotated(qrow), kr = rotated(krow);
+    const uint2 vn = *reinterpret_cast<const uint2 *>(vrow + d4 * 2);
+    float dot = lo_half_to_f32<DT>(qr.x) * lo_half_to_f32<DT>(kr.x) + hi_half_to_f32<DT>(qr.x) * hi_half_to_f32<DT>(kr.x) +
+                lo_half_to_f32<DT>(qr.y) * lo_half_to_f32<DT>(kr.y) + hi_half_to_f32<DT>(qr.y) * hi_half_to_f32<DT>(kr.y);
+#pragma unroll
+    for (int d = 1; d < per_row; d *= 2) dot += __shfl_xor(dot, d);
+    const float x_new = dot * p.scale_log2;
+    if (live && row == 0) {  // the new position's cache rows
+        *reinterpret_cast<uint2 *>(p.k_cache_w + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh + static_cast<int64_t>(p.Skv) * p.k_ss + d4) * 2) = kr;
+        *reinterpret_cast<uint2 *>(p.v_cache_w + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh + static_cast<int64_t>(p.Skv) * p.v_ss + d4) * 2) = vn;
+    }
+    if (!live) return;
+
+    const int64_t split_pitch = static_cast<int64_t>(gridDim.y) * p.rows_pad * (D + 4);
+    const float *pr0 = p.part + (static_cast<int64_t>(bh) * p.rows_pad + row) * (D + 4);
+    float M = x_new;
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float ms[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ms[j] = pr0[(s0 + j < p.nsplit ? s0 + j : s0) * split_pitch + D];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) M = fmaxf(M, ms[j]);
+    }
+    const float w_new = exp2f(x_new - M);
+    float o[4] = {w_new * lo_half_to_f32<DT>(vn.x), w_new * hi_half_to_f32<DT>(vn.x), w_new * lo_half_to_f32<DT>(vn.y), w_new * hi_half_to_f32<DT>(vn.y)};
+    float l = w_new;
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        float2 ml[8];
+        f32x4 ov[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float *pr = pr0 + (s0 + j < p.nsplit ? s0 + j : s0) * split_pitch;
+            ml[j] = *reinterpret_cast<const float2 *>(pr + D);
+            ov[j] = *reinterpret_cast<const f32x4 *>(pr + d4);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float w = s0 + j < p.nsplit ? exp2f(ml[j].x - M) : 0.f;
+            l += w * ml[j].y;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] += w * ov[j][i];
+        }
+    }
+    const float inv = 1.0f / l;  // l >= the new position's weight, which is 1 when it holds the maximum
+    uint2 o2;
+    o2.x = pack2_half<DT>(o[0] * inv, o[1] * inv);
+    o2.y = pack2_half<DT>(o[2] * inv, o[3] * inv);
+    const int head = hkv * p.G + row;
+    *reinterpret_cast<uint2 *>(p.o + (static_cast<int64_t>(b) * p.o_sb + static_cast<int64_t>(head) * p.o_sh + d4) * 2) = o2;
+}
+
 template <int DT, int D>
 int launch(AttnParams p, int cus, hipStream_t s) {
     int dev = 0;
@@ -507,37 +607,59 @@ int launch(AttnParams p, int cus, hipStream_t s) {
         ring = !wide && p.Skv / nsplit >= RING_MIN_TILES * AT_KEYS;
     }
     if (tuning().attn_ring != TUNE_UNSET) ring = !wide && tuning().attn_ring > 0;
-    p.keys_per_split = ((p.Skv + nsplit - 1) / nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
-    nsplit = (p.Skv + p.keys_per_split - 1) / p.keys_per_split;
+    const bool newkey = p.cos != nullptr;  // decode with the new position merged in by the second launch
+    if (p.Skv > 0) {
+        p.keys_per_split = ((p.Skv + nsplit - 1) / nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
+        nsplit = (p.Skv + p.keys_per_split - 1) / p.keys_per_split;
+    } else {
+        nsplit = 0;  // an empty cache (newkey only): no partials, the merge sees the new position alone
+        p.keys_per_split = AT_KEYS;
+    }
     p.nsplit = nsplit;
     p.rows_pad = row_tiles * block_rows;
+    p.force_partials = newkey ? 1 : 0;
     TPAMD_REQUIRE(p.B * p.Hkv < 65536 && nsplit < 65536, "attention: batch * kv heads too large for one launch");
-    const dim3 grid(row_tiles, p.B * p.Hkv, nsplit);
+    const dim3 grid(row_tiles, p.B * p.Hkv, nsplit > 0 ? nsplit : 1);
     auto run = [&](const AttnParams &prm, dim3 g, bool with_ring) {
         if (wide) hipLaunchKernelGGL((attention_kernel<DT, D, 2, 1>), g, dim3(256), 0, s, prm);
         else if (with_ring) hipLaunchKernelGGL((attention_kernel<DT, D, 1, RING>), g, dim3(256), 0, s, prm);
         else hipLaunchKernelGGL((attention_kernel<DT, D, 1, 1>), g, dim3(256), 0, s, prm);
         return hipGetLastError();
     };
-    if (nsplit == 1) {
+    if (nsplit == 1 && !newkey) {
         TPAMD_HIP(run(p, grid, ring));
         return TPAMD_OK;
     }
-    const size_t need = static_cast<size_t>(nsplit) * p.B * p.Hkv * p.rows_pad * (D + 4) * sizeof(float);
-    std::lock_guard<std::mutex> hold(splitk_mutex(dev));
-    void *ws = nullptr;
-    int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
-    if (rc != TPAMD_OK) return rc;
-    if (ws == nullptr) {  // no scratch (first use under stream capture, or more than it holds): one split
-        p.nsplit = 1;
-        p.keys_per_split = (p.Skv + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
-        TPAMD_HIP(run(p, dim3(row_tiles, p.B * p.Hkv, 1), p.Skv >= RING_MIN_TILES * AT_KEYS));
+    if (nsplit > 0) {
+        const size_t need = static_cast<size_t>(nsplit) * p.B * p.Hkv * p.rows_pad * (D + 4) * sizeof(float);
+        std::lock_guard<std::mutex> hold(splitk_mutex(dev));
+        void *ws = nullptr;
+        int rc = splitk_scratch(dev, s, need, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
+        if (rc != TPAMD_OK) return rc;
+        if (ws == nullptr) {  // no scratch (first use under stream capture, or more than it holds)
+            if (newkey) {
+                set_error("%s", "tpamd_attention_decode_rope: no scratch buffer for the partial results of this stream (its first use "
+                                "under stream capture, or a batch that needs more than the buffer holds): call tpamd_rope_append and "
+                                "tpamd_attention instead");
+                return TPAMD_ERR_UNSUPPORTED;
+            }
+            p.nsplit = 1;  // one split, no partials
+            p.keys_per_split = (p.Skv + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
+            TPAMD_HIP(run(p, dim3(row_tiles, p.B * p.Hkv, 1), p.Skv >= RING_MIN_TILES * AT_KEYS));
+            return TPAMD_OK;
+        }
+        p.part = static_cast<float *>(ws);
+        TPAMD_HIP(run(p, grid, ring));
+        // (the merge below is enqueued under the same lock: the buffer is this call's until then)
+        const unsigned cblocks = static_cast<unsigned>((static_cast<int64_t>(nrows) * (D / 4) + 255) / 256);
+        if (newkey) hipLaunchKernelGGL((attention_combine_newkey_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((attention_combine_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
+        TPAMD_HIP(hipGetLastError());
         return TPAMD_OK;
     }
-    p.part = static_cast<float *>(ws);
-    TPAMD_HIP(run(p, grid, ring));
+    // newkey on an empty cache
     const unsigned cblocks = static_cast<unsigned>((static_cast<int64_t>(nrows) * (D / 4) + 255) / 256);
-    hipLaunchKernelGGL((attention_combine_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
+    hipLaunchKernelGGL((attention_combine_newkey_kernel<DT, D>), dim3(cblocks, p.B * p.Hkv), dim3(256), 0, s, p);
     TPAMD_HIP(hipGetLastError());
     return TPAMD_OK;
 }
@@ -560,8 +682,45 @@ int attention_dispatch(const void *q, const void *k, const void *v, void *o, int
     p.k_sb = strides[3]; p.k_sh = strides[4]; p.k_ss = strides[5];
     p.v_sb = strides[6]; p.v_sh = strides[7]; p.v_ss = strides[8];
     p.o_sb = strides[9]; p.o_ss = strides[10]; p.o_sh = strides[11];
+    p.q_sg = p.G * p.q_sh;
     p.scale_log2 = scale * 1.4426950408889634f;
     p.causal = causal;
+    const bool bf = dtype == TPAMD_BF16;
+    if (D == 64) return bf ? launch<TPAMD_BF16, 64>(p, cus, s) : launch<TPAMD_F16, 64>(p, cus, s);
+    return bf ? launch<TPAMD_BF16, 128>(p, cus, s) : launch<TPAMD_F16, 128>(p, cus, s);
+}
+
+// One new position per sequence on a cache of `pos0` positions. strides (elements): {q batch, q head, q group, k batch,
+// k head, v batch, v head, cos/sin batch, k_cache batch, k_cache head, k_cache position, v_cache batch, v_cache head,
+// v_cache position, out batch, out head}.
+int attention_decode_rope_dispatch(const void *q, const void *k, const void *v, const void *cos, const void *sin, void *k_cache,
+                                   void *v_cache, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0,
+                                   const int64_t *strides, float scale, int dtype, hipStream_t s) {
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+    AttnParams p{};
+    p.q = static_cast<const char *>(q);
+    p.k = static_cast<const char *>(k_cache);
+    p.v = static_cast<const char *>(v_cache);
+    p.k_cache_w = static_cast<char *>(k_cache);
+    p.v_cache_w = static_cast<char *>(v_cache);
+    p.new_k = static_cast<const char *>(k);
+    p.new_v = static_cast<const char *>(v);
+    p.cos = static_cast<const char *>(cos);
+    p.sin = static_cast<const char *>(sin);
+    p.o = static_cast<char *>(o);
+    p.B = static_cast<int>(B); p.Hq = static_cast<int>(Hq); p.Hkv = static_cast<int>(Hkv);
+    p.Sq = 1; p.Skv = static_cast<int>(pos0); p.G = static_cast<int>(Hq / Hkv);
+    p.q_sb = strides[0]; p.q_sh = strides[1]; p.q_sg = strides[2]; p.q_ss = 0;
+    p.nk_sb = strides[3]; p.nk_sh = strides[4];
+    p.nv_sb = strides[5]; p.nv_sh = strides[6];
+    p.cs_b = strides[7];
+    p.k_sb = strides[8]; p.k_sh = strides[9]; p.k_ss = strides[10];
+    p.v_sb = strides[11]; p.v_sh = strides[12]; p.v_ss = strides[13];
+    p.o_sb = strides[14]; p.o_sh = strides[15]; p.o_ss = 0;
+    p.scale_log2 = scale * 1.4426950408889634f;
+    p.causal = 0;  // the one new position sees every cached key
     const bool bf = dtype == TPAMD_BF16;
     if (D == 64) return bf ? launch<TPAMD_BF16, 64>(p, cus, s) : launch<TPAMD_F16, 64>(p, cus, s);
     return bf ? launch<TPAMD_BF16, 128>(p, cus, s) : launch<TPAMD_F16, 128>(p, cus, s);

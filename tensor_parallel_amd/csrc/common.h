@@ -161,6 +161,23 @@ __device__ __forceinline__ uint32_t add_packed2(uint32_t a, uint32_t b) {
     return pack2_half<DT>(lo_half_to_f32<DT>(a) + lo_half_to_f32<DT>(b), hi_half_to_f32<DT>(a) + hi_half_to_f32<DT>(b));
 }
 
+// out = round(round(a * c) + round(b * s)) per 16-bit element: the three torch ops of
+// `(x * cos) + (rotate_half(x) * sin)` on tensors of the 16-bit dtype, each an fp32 operation rounded once.
+template <int DT>
+__device__ __forceinline__ uint32_t rot2(uint32_t a, uint32_t c, uint32_t b, uint32_t s, float sign) {
+    const float a0 = lo_half_to_f32<DT>(a), a1 = hi_half_to_f32<DT>(a);
+    const float b0 = sign * lo_half_to_f32<DT>(b), b1 = sign * hi_half_to_f32<DT>(b);
+    const uint32_t ac = pack2_half<DT>(a0 * lo_half_to_f32<DT>(c), a1 * hi_half_to_f32<DT>(c));
+    const uint32_t bs = pack2_half<DT>(b0 * lo_half_to_f32<DT>(s), b1 * hi_half_to_f32<DT>(s));
+    return add_packed2<DT>(ac, bs);
+}
+
+template <int DT>
+__device__ __forceinline__ uint4 rot8(uint4 a, uint4 c, uint4 b, uint4 s, float sign) {
+    return make_uint4(rot2<DT>(a.x, c.x, b.x, s.x, sign), rot2<DT>(a.y, c.y, b.y, s.y, sign), rot2<DT>(a.z, c.z, b.z, s.z, sign),
+                      rot2<DT>(a.w, c.w, b.w, s.w, sign));
+}
+
 // Four int8 (one dword) -> four values of the activation dtype, packed as lo = elements 0,1 and
 // hi = elements 2,3. Exact: |q| <= 128 fits both f16 and bf16 significands.
 template <int DT>
