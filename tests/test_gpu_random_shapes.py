@@ -193,3 +193,34 @@ def test_attention_random_shape(seed):
     want = torch.from_numpy(oat.attention_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale, causal))
     torch.testing.assert_close(got.double().cpu(), want, rtol=RTOL, atol=RTOL * want.std().item(),
                                msg=lambda m: f"B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Skv={Skv} D={D} causal={causal} {dtype}: {m}")
+
+
+@pytest.mark.parametrize("seed", range(700, 730))
+def test_decode_with_folded_rotary_random_shape(seed):
+    """One new position on caches of random length (0 to 3000 positions), random batch and head grouping: cache rows bit for
+    bit against the oracle's rotary step, the output against its attention in float64."""
+    from oracle import attention as oat
+    from oracle import rope as orp
+
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    B, Hkv, per = pick(1, 6), pick(1, 4), [1, 2, 4, 8, 16][pick(0, 4)]
+    D = [64, 128][pick(0, 1)]
+    dtype = [torch.bfloat16, torch.float16][pick(0, 1)]
+    pos0 = [0, 1, pick(2, 200), pick(200, 3000)][pick(0, 3)]
+    L = pos0 + 1 + pick(0, 9)
+    fused = torch.randn(B, 1, Hkv, per + 2, D, generator=g).to(dtype)
+    kc = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
+    vc = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
+    cos, sin = orp.angles(torch.tensor([pos0]), D, dtype=dtype)
+    q = fused[:, :, :, :per].reshape(B, 1, Hkv * per, D)
+    q_rot, want_kc, want_vc = orp.rope_append(q, fused[:, :, :, per], fused[:, :, :, per + 1], cos[None], sin[None], kc.clone(), vc.clone(), pos0)
+    scale = D ** -0.5
+    want = torch.from_numpy(oat.attention_f64(q_rot.float().numpy(), want_kc[:, :, :pos0 + 1].float().numpy(),
+                                              want_vc[:, :, :pos0 + 1].float().numpy(), scale, True))
+    fd, kcd, vcd = fused.to(DEV), kc.to(DEV), vc.to(DEV)
+    got = _native.attention_decode_rope(fd[:, :, :, :per], fd[:, :, :, per], fd[:, :, :, per + 1], cos.to(DEV), sin.to(DEV), kcd, vcd, pos0)
+    as_bits = lambda t: t.detach().cpu().contiguous().view(torch.int16)  # noqa: E731
+    tag = f"B={B} Hkv={Hkv} per={per} D={D} pos0={pos0} {dtype}"
+    assert torch.equal(as_bits(kcd), as_bits(want_kc)) and torch.equal(as_bits(vcd), as_bits(want_vc)), tag
+    torch.testing.assert_close(got.double().cpu(), want, rtol=RTOL, atol=RTOL * want.std().item(), msg=lambda m: f"{tag}: {m}")
