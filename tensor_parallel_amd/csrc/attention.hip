@@ -14,7 +14,9 @@
 // O^T leaves a lane with 4 consecutive head-dim elements of one query row: one 8-byte store into [B, Sq, Hq, D].
 //
 // Long key ranges with few rows (decode) are split over blockIdx.z; every split leaves (m, l, unnormalised O) in
-// the per-device scratch buffer and attention_combine_kernel merges them.
+// the stream's scratch buffer and attention_combine_kernel merges them. For one new position per sequence
+// (tpamd_attention_decode_rope) the kernel also applies the rotary embedding to its Q fragments, and the merge
+// (attention_combine_newkey_kernel) adds the new position's key and value and writes them into the cache.
 #include "common.h"
 
 #include <stdlib.h>
