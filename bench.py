@@ -580,7 +580,53 @@ def api_level_extras(torch, dev) -> dict:
         us = _time_us(torch, lambda i: opt_tp(input_ids=ids, use_cache=False).logits, 5, 20)
         out["c1_opt125m"] = {"us_per_forward": us, "tokens_per_s": 128 / us * 1e6, "dtype": "f32",
                              "what": "tp.tensor_parallel(OPT-125m, W=2) forward of 2 x 64 tokens, both rank shards on this GPU, host orchestration included"}
+        del opt_tp, model
+        out["llama_layer_decode_tp"] = llama_layer_decode(torch, dev)
     return out
+
+
+def llama_layer_decode(torch, dev) -> dict:
+    """One decode step of a Llama-2-7B-shaped decoder (2 layers: d 4096, 32 heads of 128, ffn 11008, bf16) through
+    tp.tensor_parallel at W = 2 with both rank shards on this GPU, batch 8 on 2048 cached positions, host orchestration
+    included: the wrapped attention modules with their own forward (torch rotary embedding and cache update, the library's
+    attention core) and with tp.attention.fuse_rotary_ (rotary embedding, cache append and attention core in the library's
+    decode call). Every step appends a position, so the cache is cropped back between steps."""
+    from copy import deepcopy
+
+    from transformers import DynamicCache, LlamaConfig, LlamaModel
+
+    import tensor_parallel_amd as tp
+
+    name = tp.attention.register()
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=1024, hidden_size=D_MODEL, intermediate_size=2 * FFN_SHARD, num_hidden_layers=2, num_attention_heads=32,
+                      num_key_value_heads=32, max_position_embeddings=4096, attn_implementation="eager")
+    with torch.device(dev):
+        model = LlamaModel(cfg).to(torch.bfloat16).eval()
+    for p in model.parameters():
+        p.normal_(0.0, 0.02)
+    model.config._attn_implementation = name
+    B, L = 8, 2048
+    prompt = torch.randint(0, 1024, (B, L), generator=torch.Generator().manual_seed(1)).to(dev)
+    tok = torch.randint(0, 1024, (B, 1), generator=torch.Generator().manual_seed(2)).to(dev)
+    res = {}
+    for label in ("own_forward", "fuse_rotary"):
+        m = tp.tensor_parallel(deepcopy(model), [dev, dev])
+        if label == "fuse_rotary":
+            tp.attention.fuse_rotary_(m)
+        cache = DynamicCache()
+        m(input_ids=prompt, past_key_values=cache, use_cache=True)
+
+        def step(i, m=m, cache=cache):
+            m(input_ids=tok, past_key_values=cache, use_cache=True)
+            cache.crop(-1)
+
+        us = _time_us(torch, step, 5, 30)
+        res[label] = {"us_per_step": us, "tokens_per_s": B / us * 1e6}
+        del m, cache
+    res["what"] = ("tp.tensor_parallel(2-layer Llama-2-7B-shaped decoder, W=2) decode step, batch 8 on 2048 cached positions, both rank "
+                   "shards on this GPU, host orchestration and the cache crop included")
+    return res
 
 
 def reduce_extra(torch, _native, dev, other) -> dict:

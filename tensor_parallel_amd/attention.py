@@ -9,9 +9,17 @@ named "tpamd" to transformers' attention registry, and a model picks it with
 The kernel covers causal self-attention of decoder models without padding (prefill, and decode on a cache:
 the queries are the last positions of the keys) and unmasked attention. A call with an explicit mask, dropout or a
 head_dim other than 64 / 128 raises: there is no second implementation to fall back to.
+
+`fuse_rotary_(model)` goes one step further for attention modules of the Llama pattern (q_proj / k_proj / v_proj / o_proj,
+rotary position embeddings handed in as `position_embeddings`, a transformers cache object): their forward then runs the
+rotary embedding, the hand-over to the cache and the attention core on the library's kernels too (`tpamd_rope_append` +
+`tpamd_attention` at prefill, `tpamd_attention_decode_rope` for one new position), writing into buffers with room to grow
+that the cache layer's `keys` / `values` are views of. A call those kernels do not cover takes the module's own forward.
 """
 from __future__ import annotations
 
+import inspect
+import types
 from typing import Optional, Tuple
 
 import torch
@@ -50,3 +58,114 @@ def register() -> str:
     # mask construction as for sdpa: a purely causal mask is skipped (None reaches attention_forward)
     AttentionMaskInterface.register(IMPLEMENTATION_NAME, sdpa_mask)
     return IMPLEMENTATION_NAME
+
+
+# ---- rotary embedding + cache append + attention core for attention modules of the Llama pattern ------------------------
+_MIN_CAPACITY = 256
+
+
+def _cache_layer(cache, layer_idx: int):
+    """The plain growing layer `layer_idx` of a transformers cache (made on demand as `Cache.update` would), or None when the
+    cache is of another kind (static, sliding window, quantised, offloaded): those keep the module's own forward."""
+    from transformers.cache_utils import DynamicLayer
+
+    layers = getattr(cache, "layers", None)
+    if layers is None or getattr(cache, "offloading", False):
+        return None
+    if len(layers) <= layer_idx:
+        if getattr(cache, "layer_class_to_replicate", None) is not DynamicLayer:
+            return None
+        while len(layers) <= layer_idx:
+            layers.append(DynamicLayer())
+    layer = layers[layer_idx]
+    return layer if type(layer) is DynamicLayer else None
+
+
+def _buffers_with_room(layer, B: int, Hkv: int, D: int, need: int, like: torch.Tensor):
+    """(k, v) buffers [B, Hkv, capacity >= need, D] that hold the layer's cached positions: the ones its keys / values are
+    views of when they still are and have room, else new ones (twice the need) with the cached positions copied over."""
+    have = layer.get_seq_length()
+    bufs = layer.__dict__.get("_tp_buffers")
+    if bufs is not None and have > 0:
+        kb, vb = bufs
+        same = (layer.keys.data_ptr() == kb.data_ptr() and layer.values.data_ptr() == vb.data_ptr()
+                and layer.keys.shape == (B, Hkv, have, D) and layer.keys.stride() == kb.stride() and layer.values.stride() == vb.stride())
+        if not same:
+            bufs = None
+    if bufs is None or bufs[0].shape[:2] != (B, Hkv) or bufs[0].shape[2] < need or bufs[0].dtype != like.dtype or bufs[0].device != like.device:
+        cap = max(2 * need, _MIN_CAPACITY)
+        kb = torch.empty((B, Hkv, cap, D), dtype=like.dtype, device=like.device)
+        vb = torch.empty_like(kb)
+        if have > 0:
+            kb[:, :, :have].copy_(layer.keys)
+            vb[:, :, :have].copy_(layer.values)
+        bufs = layer.__dict__["_tp_buffers"] = (kb, vb)
+    return bufs
+
+
+def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings=None, attention_mask=None, past_key_values=None,
+                          **kwargs):
+    own = type(self).forward
+    D = getattr(self, "head_dim", None)
+    layer = None
+    usable = (position_embeddings is not None and attention_mask is None and past_key_values is not None and not self.training
+              and hidden_states.dim() == 3 and hidden_states.device.type == "cuda"
+              and hidden_states.dtype in (torch.bfloat16, torch.float16) and D in (64, 128)
+              and not kwargs.get("output_attentions") and getattr(self, "is_causal", True))
+    if usable:
+        layer = _cache_layer(past_key_values, self.layer_idx)
+    if layer is None:
+        return own(self, hidden_states, position_embeddings=position_embeddings, attention_mask=attention_mask,
+                   past_key_values=past_key_values, **kwargs)
+    B, S, _ = hidden_states.shape
+    q = self.q_proj(hidden_states).view(B, S, -1, D)
+    k = self.k_proj(hidden_states).view(B, S, -1, D)
+    v = self.v_proj(hidden_states).view(B, S, -1, D)
+    Hq, Hkv = q.shape[2], k.shape[2]
+    cos, sin = position_embeddings
+    cos, sin = cos.to(q.dtype), sin.to(q.dtype)
+    pos0 = layer.get_seq_length()
+    kb, vb = _buffers_with_room(layer, B, Hkv, D, pos0 + S, q)
+    scale = getattr(self, "scaling", None)
+    if S == 1:
+        out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, pos0, scale=scale)
+    else:
+        q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
+        out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=scale, causal=True)
+    if not layer.is_initialized:
+        layer.dtype, layer.device = q.dtype, q.device
+        layer.is_initialized = True
+    layer.keys, layer.values = kb[:, :, :pos0 + S], vb[:, :, :pos0 + S]
+    return self.o_proj(out.reshape(B, S, Hq * D)), None
+
+
+FUSABLE_ATTENTION_CLASSES = ("LlamaAttention",)
+
+
+def _is_llama_pattern(module: torch.nn.Module, class_names) -> bool:
+    """An attention module whose own forward is exactly: q / k / v projections, rotary embedding of q and k from
+    `position_embeddings`, cache update, attention, output projection (no norms on q / k, no sliding window, no softcap)."""
+    if type(module).__name__ not in class_names:
+        return False
+    children = set(module._modules)
+    if children != {"q_proj", "k_proj", "v_proj", "o_proj"}:
+        return False
+    if not hasattr(module, "layer_idx") or not hasattr(module, "head_dim") or getattr(module, "sliding_window", None) is not None:
+        return False
+    try:
+        params = inspect.signature(type(module).forward).parameters
+    except (TypeError, ValueError):
+        return False
+    return "position_embeddings" in params and "past_key_values" in params and "attention_mask" in params
+
+
+def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES) -> int:
+    """Give every attention module under `model` (before or after `tp.tensor_parallel`) whose class is named in
+    `class_names` and whose structure is the Llama pattern the forward described in the module docstring. Returns how many
+    modules took it. Name further classes only when their forward is the same sequence of operations."""
+    count = 0
+    for module in model.modules():
+        if _is_llama_pattern(module, class_names) and "forward" not in module.__dict__:
+            module.forward = types.MethodType(_fused_rotary_forward, module)
+            count += 1
+    return count

@@ -1,0 +1,96 @@
+"""`tp.attention.fuse_rotary_`: the attention modules of a Llama run rotary embedding, cache append and attention core on the
+library's kernels, inside `tp.tensor_parallel` on two ranks, against the same model with the module's own forward (torch
+rotary embedding and cache update, the library's attention core): logits of the prefill and of decode steps, the cache
+contents bit for bit, `generate`."""
+from copy import deepcopy
+
+import pytest
+import torch
+
+import tensor_parallel_amd as tp
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+RTOL = 2e-2
+
+
+def tiny_llama(dtype):
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    name = tp.attention.register()
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=300, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, max_position_embeddings=2048, attn_implementation="eager", bos_token_id=1, eos_token_id=None,
+                      pad_token_id=0)
+    model = LlamaForCausalLM(cfg).to(dtype).eval()
+    model.config._attn_implementation = name
+    return model
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_rotary_attention_inside_tensor_parallel(dtype):
+    from transformers import DynamicCache
+
+    model = tiny_llama(dtype)
+    plain = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    fused = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    assert tp.attention.fuse_rotary_(fused) == 2 * 2  # ranks x layers
+    assert tp.attention.fuse_rotary_(fused) == 0      # once
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(2, 300, (2, 300), generator=g).to(DEV)  # more positions than the buffers' first capacity holds
+    steps = [torch.randint(2, 300, (2, 1), generator=g).to(DEV) for _ in range(6)]
+    caches = [DynamicCache(), DynamicCache()]
+    with torch.no_grad():
+        outs = [m(input_ids=ids, past_key_values=c, use_cache=True).logits.float() for m, c in zip((plain, fused), caches)]
+        scale = outs[0].std().item()
+        torch.testing.assert_close(outs[1], outs[0], rtol=RTOL, atol=RTOL * scale)
+        for i, tok in enumerate(steps):
+            a, b = (m(input_ids=tok, past_key_values=c, use_cache=True).logits.float() for m, c in zip((plain, fused), caches))
+            torch.testing.assert_close(b, a, rtol=RTOL, atol=RTOL * scale, msg=lambda m: f"decode step {i}: {m}")
+    for cache in caches:
+        assert cache.get_seq_length() == 306
+    # rank 0 writes into the caller's cache object: first layer's keys (rotated by the kernel / by torch) and values.
+    # The first layer sees the same inputs in both models, so its cache rows must be the same bits.
+    k_plain, v_plain = caches[0].layers[0].keys, caches[0].layers[0].values
+    k_fused, v_fused = caches[1].layers[0].keys, caches[1].layers[0].values
+    assert k_fused.shape == k_plain.shape == (2, 1, 306, 64)  # this rank's one key/value head
+    assert torch.equal(k_fused.view(torch.int16), k_plain.view(torch.int16))
+    assert torch.equal(v_fused.view(torch.int16), v_plain.view(torch.int16))
+
+
+def test_generate_with_fused_rotary_attention():
+    model = tiny_llama(torch.float16)
+    with torch.no_grad():
+        for p in model.parameters():
+            p.normal_(0.0, 0.05)
+    plain = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    fused = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    tp.attention.fuse_rotary_(fused)
+    ids = torch.randint(2, 300, (3, 7), generator=torch.Generator().manual_seed(3)).to(DEV)
+    kwargs = dict(max_new_tokens=12, do_sample=False, attention_mask=torch.ones_like(ids), output_scores=True, return_dict_in_generate=True)
+    with torch.no_grad():
+        a = plain.generate(ids, **kwargs)
+        b = fused.generate(ids, **kwargs)
+    assert a.sequences.shape == b.sequences.shape == (3, 19)
+    # greedy tokens can part ways where two logits are a rounding apart: compare the scores until they do
+    for step, (sa, sb) in enumerate(zip(a.scores, b.scores)):
+        same_so_far = torch.equal(a.sequences[:, :7 + step], b.sequences[:, :7 + step])
+        if not same_so_far:
+            break
+        torch.testing.assert_close(sb.float(), sa.float(), rtol=RTOL, atol=3 * RTOL * sa.float().std().item())
+    assert step >= 3
+
+
+def test_modules_outside_the_pattern_keep_their_forward():
+    from transformers import GPT2Config, GPT2LMHeadModel
+
+    model = GPT2LMHeadModel(GPT2Config(n_embd=64, n_head=4, n_layer=1, n_positions=32, vocab_size=50))
+    assert tp.attention.fuse_rotary_(model) == 0
+    llama = tiny_llama(torch.float32)  # float32: the fused forward hands such calls to the module's own forward
+    assert tp.attention.fuse_rotary_(llama) == 2
+    llama = llama.to(DEV)
+    llama.config._attn_implementation = "eager"
+    ids = torch.randint(2, 300, (1, 9), generator=torch.Generator().manual_seed(4)).to(DEV)
+    with torch.no_grad():
+        out = llama(input_ids=ids, use_cache=True)
+    assert out.logits.shape == (1, 9, 300) and out.past_key_values.get_seq_length() == 9
