@@ -45,6 +45,9 @@ def test_fused_rotary_attention_inside_tensor_parallel(dtype):
         scale = outs[0].std().item()
         torch.testing.assert_close(outs[1], outs[0], rtol=RTOL, atol=RTOL * scale)
         for i, tok in enumerate(steps):
+            if i == 3:  # beam search reorders the batch: the layer's tensors are new ones then, and are taken over again
+                for c in caches:
+                    c.reorder_cache(torch.tensor([1, 0], device=DEV))
             a, b = (m(input_ids=tok, past_key_values=c, use_cache=True).logits.float() for m, c in zip((plain, fused), caches))
             torch.testing.assert_close(b, a, rtol=RTOL, atol=RTOL * scale, msg=lambda m: f"decode step {i}: {m}")
     for cache in caches:
