@@ -139,6 +139,44 @@ def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings
     return self.o_proj(out.reshape(B, S, Hq * D)), None
 
 
+def _fused_falcon_forward(self, hidden_states: torch.Tensor, alibi=None, attention_mask=None, position_ids=None, layer_past=None,
+                          use_cache: bool = False, output_attentions: bool = False, position_embeddings=None, **kwargs):
+    """FalconAttention with rotary embeddings and grouped heads (the new decoder architecture). transformers always
+    hands this module a materialised mask; it is ignored here, which is what `fuse_rotary_(..., assume_no_padding=True)`
+    was told is right (the mask is then the causal pattern the kernels apply themselves)."""
+    D = self.head_dim
+    layer = None
+    usable = (alibi is None and position_embeddings is not None and layer_past is not None and not self.training and not output_attentions
+              and self.new_decoder_architecture and hidden_states.dim() == 3 and hidden_states.device.type == "cuda"
+              and hidden_states.dtype in (torch.bfloat16, torch.float16) and D in (64, 128))
+    if usable:
+        layer = _cache_layer(layer_past, self.layer_idx)
+    if layer is None:
+        return type(self).forward(self, hidden_states, alibi, attention_mask, position_ids=position_ids, layer_past=layer_past,
+                                  use_cache=use_cache, output_attentions=output_attentions, position_embeddings=position_embeddings, **kwargs)
+    B, S, _ = hidden_states.shape
+    fused_qkv = self.query_key_value(hidden_states)
+    # [.., kv head, its query heads + key + value, D]
+    per = self.num_heads // self.num_kv_heads
+    qkv = fused_qkv.view(B, S, self.num_kv_heads, per + 2, D)
+    q, k, v = qkv[:, :, :, :per], qkv[:, :, :, per], qkv[:, :, :, per + 1]
+    Hkv = self.num_kv_heads
+    cos, sin = position_embeddings
+    cos, sin = cos.to(fused_qkv.dtype), sin.to(fused_qkv.dtype)
+    pos0 = layer.get_seq_length()
+    kb, vb = _buffers_with_room(layer, B, Hkv, D, pos0 + S, fused_qkv)
+    if S == 1:
+        out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, pos0, scale=self.inv_norm_factor)
+    else:
+        q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
+        out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=self.inv_norm_factor, causal=True)
+    if not layer.is_initialized:
+        layer.dtype, layer.device = fused_qkv.dtype, fused_qkv.device
+        layer.is_initialized = True
+    layer.keys, layer.values = kb[:, :, :pos0 + S], vb[:, :, :pos0 + S]
+    return self.dense(out.reshape(B, S, self.num_heads * D)), None
+
+
 FUSABLE_ATTENTION_CLASSES = ("LlamaAttention",)
 
 
@@ -159,13 +197,32 @@ def _is_llama_pattern(module: torch.nn.Module, class_names) -> bool:
     return "position_embeddings" in params and "past_key_values" in params and "attention_mask" in params
 
 
-def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES) -> int:
+def _is_rotary_falcon(module: torch.nn.Module) -> bool:
+    """transformers' FalconAttention with rotary embeddings and grouped heads (the 40B layout)."""
+    if type(module).__name__ != "FalconAttention" or set(module._modules) != {"query_key_value", "dense", "attention_dropout"}:
+        return False
+    config = getattr(module, "config", None)
+    return getattr(config, "alibi", True) is False and module.new_decoder_architecture and getattr(module, "layer_idx", None) is not None
+
+
+def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, assume_no_padding: bool = False) -> int:
     """Give every attention module under `model` (before or after `tp.tensor_parallel`) whose class is named in
     `class_names` and whose structure is the Llama pattern the forward described in the module docstring. Returns how many
-    modules took it. Name further classes only when their forward is the same sequence of operations."""
+    modules took it. Name further classes only when their forward is the same sequence of operations.
+
+    `assume_no_padding=True` also takes transformers' FalconAttention (rotary, grouped heads: the 40B layout): that model
+    hands its attention modules a materialised mask on every call, which cannot be told from a padding mask without
+    reading it back, so the caller vouches that the batches carry no padding and the mask is ignored. Such a module then
+    caches its key/value heads once, not once per query head as its own forward does: every call of a fused model must
+    be one the fused forward takes (16-bit tensors on the device, a growing cache, inference)."""
     count = 0
     for module in model.modules():
-        if _is_llama_pattern(module, class_names) and "forward" not in module.__dict__:
+        if "forward" in module.__dict__:
+            continue
+        if _is_llama_pattern(module, class_names):
             module.forward = types.MethodType(_fused_rotary_forward, module)
+            count += 1
+        elif assume_no_padding and _is_rotary_falcon(module):
+            module.forward = types.MethodType(_fused_falcon_forward, module)
             count += 1
     return count

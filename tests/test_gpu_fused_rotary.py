@@ -97,3 +97,34 @@ def test_modules_outside_the_pattern_keep_their_forward():
     with torch.no_grad():
         out = llama(input_ids=ids, use_cache=True)
     assert out.logits.shape == (1, 9, 300) and out.past_key_values.get_seq_length() == 9
+
+
+def test_fused_rotary_falcon_inside_tensor_parallel():
+    """transformers' Falcon with rotary embeddings in the 40B layout (grouped heads in a fused query_key_value) on two
+    ranks: its own forward (torch rotary embedding, cache update and attention on every query head's copy of the keys)
+    against the fused one, which keeps each rank's key/value heads once."""
+    from transformers import DynamicCache, FalconConfig, FalconForCausalLM
+
+    torch.manual_seed(0)
+    cfg = FalconConfig(vocab_size=300, hidden_size=512, num_hidden_layers=2, num_attention_heads=8, num_kv_heads=4,
+                       new_decoder_architecture=True, multi_query=True, parallel_attn=True, alibi=False, bias=False,
+                       max_position_embeddings=1024, bos_token_id=1, eos_token_id=None, pad_token_id=0)
+    model = FalconForCausalLM(cfg).to(torch.bfloat16).eval()
+    plain = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    fused = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    assert tp.attention.fuse_rotary_(fused) == 0  # Falcon only on the caller's word that there is no padding
+    assert tp.attention.fuse_rotary_(fused, assume_no_padding=True) == 2 * 2
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(2, 300, (2, 70), generator=g).to(DEV)
+    steps = [torch.randint(2, 300, (2, 1), generator=g).to(DEV) for _ in range(4)]
+    caches = [DynamicCache(), DynamicCache()]
+    with torch.no_grad():
+        outs = [m(input_ids=ids, past_key_values=c, use_cache=True).logits.float() for m, c in zip((plain, fused), caches)]
+        scale = outs[0].std().item()
+        torch.testing.assert_close(outs[1], outs[0], rtol=RTOL, atol=RTOL * scale)
+        for i, tok in enumerate(steps):
+            a, b = (m(input_ids=tok, past_key_values=c, use_cache=True).logits.float() for m, c in zip((plain, fused), caches))
+            torch.testing.assert_close(b, a, rtol=RTOL, atol=RTOL * scale, msg=lambda m: f"decode step {i}: {m}")
+    assert caches[1].get_seq_length() == 74
+    # the fused forward keeps this rank's key/value heads once (2 of the 4 groups), the module's own one copy per query head
+    assert caches[1].layers[0].keys.shape == (2, 2, 74, 64) and caches[0].layers[0].keys.shape == (2, 4, 74, 64)
