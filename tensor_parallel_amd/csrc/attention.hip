@@ -371,8 +371,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         if (k_begin < k_end) {
             fetch(k_begin);
             stage(0);
-            if (k_begin + AT_KEYS < k_end) fetch(k_begin + AT_KEYS);
         }
+        // Wait here, on every path into the loop, for all that was requested so far (the Q fragments among it): the
+        // compiler then knows that the only loads in flight at the top of the loop are the tile requested ahead, which
+        // nothing reads before the end of the tile's arithmetic. Without it the first MFMAs of every tile waited for
+        // all loads (s_waitcnt vmcnt(0)), the tile requested one barrier earlier included.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters left alone
+        if (k_begin + AT_KEYS < k_end) fetch(k_begin + AT_KEYS);
         __syncthreads();
         int buf = 0;
         int k0 = k_begin;
