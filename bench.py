@@ -580,7 +580,11 @@ def api_level_extras(torch, dev) -> dict:
         us = _time_us(torch, lambda i: opt_tp(input_ids=ids, use_cache=False).logits, 5, 20)
         out["c1_opt125m"] = {"us_per_forward": us, "tokens_per_s": 128 / us * 1e6, "dtype": "f32",
                              "what": "tp.tensor_parallel(OPT-125m, W=2) forward of 2 x 64 tokens, both rank shards on this GPU, host orchestration included"}
-        del opt_tp, model
+        graphed = tp.graphs.capture(opt_tp, input_ids=ids, use_cache=False)
+        us_g = _time_us(torch, lambda i: graphed.replay().logits, 5, 20)
+        out["c1_opt125m"]["graph"] = {"us_per_forward": us_g, "tokens_per_s": 128 / us_g * 1e6,
+                                      "what": "the same forward recorded once with tp.graphs.capture and replayed as a HIP graph"}
+        del graphed, opt_tp, model
         out["llama_layer_decode_tp"] = llama_layer_decode(torch, dev)
     return out
 

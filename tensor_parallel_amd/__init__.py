@@ -6,7 +6,7 @@ single-device partial-sum reduction, behind the Python surface of BlackSamorez/t
     model = tp.tensor_parallel(model, ["cuda:0", "cuda:0"])      # two rank shards on one GPU
     shards = tp.convert_state_dict(state_dict, config, world_size=2)
 """
-from . import _native, attention, int8, kv_cache, state_actions
+from . import _native, attention, graphs, int8, kv_cache, state_actions
 from .config import Config
 from .dispatch import convert_state_dict, infer_sharded_device_map, save_tensor_parallel
 from .factory import tensor_parallel

@@ -789,3 +789,10 @@ def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert res.returncode == 2 and res.stdout == ""
     assert "--gpus above 1 is not supported" in res.stderr
+
+
+def test_graph_capture_needs_a_hip_device():
+    """`tp.graphs.capture` records kernels of one HIP device: a host module is refused before anything runs."""
+    module = torch.nn.Linear(8, 8)
+    with pytest.raises(ValueError, match="one HIP device"):
+        tp.graphs.capture(module, torch.zeros(2, 8))
