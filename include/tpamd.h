@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define TPAMD_ABI_VERSION 4
+#define TPAMD_ABI_VERSION 5
 
 typedef enum tpamd_status {
     TPAMD_OK = 0,
@@ -279,6 +279,18 @@ int tpamd_attention_decode_rope(const void *q_dev, const void *k_dev, const void
                                 const void *sin_dev, void *k_cache_dev, void *v_cache_dev, void *out_dev, int64_t B,
                                 int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0, int64_t cache_len, const int64_t *strides,
                                 float scale, int dtype, void *stream);
+
+/* tpamd_attention_decode_rope with the number of cached positions read on the device: *pos_dev (int64, device memory, 8-byte
+ * aligned) is read by the kernels when they run, not by this call, so a HIP graph that holds the call serves every decode
+ * step (the caller adds 1 to *pos_dev after each step, on the same stream). No counterpart in the reference, whose
+ * forwards are Python (src/tensor_parallel/tensor_parallel.py:139-161); transformers' StaticLayer keeps this count on the
+ * device as `cumulative_length`. The launches are laid out for `cache_len` positions (the capacity of the caches) and the
+ * blocks share out the positions there are; a count outside [0, cache_len) leaves the caches unwritten. Same arguments,
+ * requirements and errors otherwise. */
+int tpamd_attention_decode_rope_devpos(const void *q_dev, const void *k_dev, const void *v_dev, const void *cos_dev,
+                                       const void *sin_dev, void *k_cache_dev, void *v_cache_dev, void *out_dev, int64_t B,
+                                       int64_t Hq, int64_t Hkv, int64_t D, const int64_t *pos_dev, int64_t cache_len,
+                                       const int64_t *strides, float scale, int dtype, void *stream);
 
 /* Weight-only int8 shard Linear with fp16/bf16 outlier columns:
  *   y[m,n] = act( scale[n] * sum_k x[m,k]*wq[n,k]  +  sum_j x[m,outlier_idx[j]] * w_out[n,j]  + bias[n] )

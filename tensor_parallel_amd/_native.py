@@ -38,9 +38,10 @@ EXPORTS = (
     "tpamd_attention",
     "tpamd_rope_append",
     "tpamd_attention_decode_rope",
+    "tpamd_attention_decode_rope_devpos",
 )
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 BF16, F16, F32 = 0, 1, 2
 ACCUM_STEPWISE, ACCUM_F32 = 0, 1
@@ -122,6 +123,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.tpamd_attention.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, c.POINTER(i64), c.c_float, ci, ci, vp]
     lib.tpamd_attention_decode_rope.restype = ci
     lib.tpamd_attention_decode_rope.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, c.POINTER(i64), c.c_float, ci, vp]
+    lib.tpamd_attention_decode_rope_devpos.restype = ci
+    lib.tpamd_attention_decode_rope_devpos.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp, i64, c.POINTER(i64), c.c_float, ci, vp]
     lib.tpamd_rope_append.restype = ci
     lib.tpamd_rope_append.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, c.POINTER(i64), ci, vp]
     lib.tpamd_linear_w8.restype = ci
@@ -542,12 +545,16 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
 
 
 def attention_decode_rope(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
-                          k_cache: torch.Tensor, v_cache: torch.Tensor, pos0: int, scale: Optional[float] = None,
+                          k_cache: torch.Tensor, v_cache: torch.Tensor, pos0, scale: Optional[float] = None,
                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`rope_append` and `attention` for one new position per sequence, in two launches instead of three.
     q [B, 1, Hq, D] or [B, 1, Hkv, Hq / Hkv, D], k / v [B, 1, Hkv, D] (views of the projection output), cos / sin [B or 1, 1, D]
     (or [1, D] / [D]); the caches [B, Hkv, L, D] hold pos0 positions and receive the new one at pos0. Returns [B, 1, Hq, D].
-    Where the library has no scratch buffer for the stream (first use under graph capture) the two calls are made instead."""
+    Where the library has no scratch buffer for the stream (first use under graph capture) the two calls are made instead.
+
+    `pos0` may also be an int64 tensor of one element on the device: the kernels then read the count when they run
+    (`tpamd_attention_decode_rope_devpos`), the launches are laid out for the L positions the caches can hold, and the call
+    can sit in a HIP graph that is replayed for every decode step. The caller advances the count."""
     require_device(q, "attention_decode_rope")
     if not (q.dtype == k.dtype == v.dtype == cos.dtype == sin.dtype == k_cache.dtype == v_cache.dtype) or q.dtype not in (
             torch.bfloat16, torch.float16):
@@ -579,6 +586,18 @@ def attention_decode_rope(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos
     strides = (ctypes.c_int64 * 16)(q.stride(0), q_head, q_group, k.stride(0), k.stride(2), v.stride(0), v.stride(2),
                                     cos.stride(0) if cos.shape[0] > 1 else 0, k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
                                     v_cache.stride(0), v_cache.stride(1), v_cache.stride(2), out.stride(0), out.stride(2))
+    if isinstance(pos0, torch.Tensor):
+        if pos0.dtype != torch.int64 or pos0.numel() != 1 or pos0.device != q.device:
+            raise ValueError(f"attention_decode_rope: a position on the device must be one int64 element on {q.device}, "
+                             f"got {tuple(pos0.shape)} {pos0.dtype} on {pos0.device}")
+        with _on_device(q.device):
+            rc = lib().tpamd_attention_decode_rope_devpos(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                                          k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), B, Hq, Hkv, D,
+                                                          ctypes.c_void_p(pos0.data_ptr()), k_cache.shape[2], strides,
+                                                          float(scale if scale is not None else D ** -0.5), dtype_code(q.dtype),
+                                                          ctypes.c_void_p(current_stream_ptr(q.device)))
+        _check(rc, "tpamd_attention_decode_rope_devpos")
+        return out
     with _on_device(q.device):
         rc = lib().tpamd_attention_decode_rope(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(), sin.data_ptr(),
                                                k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), B, Hq, Hkv, D, int(pos0),

@@ -29,7 +29,7 @@ int gemm_w8_dispatch(const void *x, const void *wq, const void *scale, const voi
 int attention_dispatch(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq,
                        int64_t Skv, int64_t D, const int64_t *strides, float scale, int causal, int dtype, hipStream_t s);
 int attention_decode_rope_dispatch(const void *q, const void *k, const void *v, const void *cos, const void *sin, void *k_cache,
-                                   void *v_cache, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0,
+                                   void *v_cache, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0, const int64_t *pos_dev,
                                    const int64_t *strides, float scale, int dtype, hipStream_t s);
 
 namespace {
@@ -188,7 +188,33 @@ extern "C" int tpamd_attention_decode_rope(const void *q_dev, const void *k_dev,
         return TPAMD_ERR_UNSUPPORTED;
     }
     return attention_decode_rope_dispatch(q_dev, k_dev, v_dev, cos_dev, sin_dev, k_cache_dev, v_cache_dev, out_dev, B, Hq, Hkv, D,
-                                          pos0, strides, scale, dtype, static_cast<hipStream_t>(stream));
+                                          pos0, nullptr, strides, scale, dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tpamd_attention_decode_rope_devpos(const void *q_dev, const void *k_dev, const void *v_dev, const void *cos_dev,
+                                                  const void *sin_dev, void *k_cache_dev, void *v_cache_dev, void *out_dev,
+                                                  int64_t B, int64_t Hq, int64_t Hkv, int64_t D, const int64_t *pos_dev,
+                                                  int64_t cache_len, const int64_t *strides, float scale, int dtype,
+                                                  void *stream) {
+    const char *who = "tpamd_attention_decode_rope_devpos";
+    TPAMD_REQUIRE(dtype == TPAMD_BF16 || dtype == TPAMD_F16, "%s: dtype must be BF16 or F16", who);
+    TPAMD_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0, "%s: bad dimension", who);
+    TPAMD_REQUIRE(Hq % Hkv == 0, "%s: %lld query heads are not a multiple of %lld key/value heads", who, (long long)Hq, (long long)Hkv);
+    TPAMD_REQUIRE(cache_len > 0 && cache_len < (1ll << 30), "%s: the caches must hold between 1 and 2^30 positions", who);
+    TPAMD_REQUIRE(strides != nullptr, "%s: strides is NULL", who);
+    if (B == 0) return TPAMD_OK;
+    TPAMD_REQUIRE(q_dev && k_dev && v_dev && cos_dev && sin_dev && k_cache_dev && v_cache_dev && out_dev && pos_dev, "%s: null pointer", who);
+    TPAMD_REQUIRE(Hq / Hkv < (1ll << 20), "%s: too many query heads per key/value head", who);
+    bool ok = (D == 64 || D == 128) && aligned(q_dev, 16) && aligned(k_dev, 16) && aligned(v_dev, 16) && aligned(cos_dev, 16) &&
+              aligned(sin_dev, 16) && aligned(k_cache_dev, 16) && aligned(v_cache_dev, 16) && aligned(out_dev, 8) && aligned(pos_dev, 8);
+    for (int i = 0; i < 14; ++i) ok = ok && strides[i] % 8 == 0;   // 16-byte loads of every row
+    for (int i = 14; i < 16; ++i) ok = ok && strides[i] % 4 == 0;  // 8-byte stores
+    if (!ok) {
+        set_error("%s: head_dim must be 64 or 128 and rows 16-byte aligned", who);
+        return TPAMD_ERR_UNSUPPORTED;
+    }
+    return attention_decode_rope_dispatch(q_dev, k_dev, v_dev, cos_dev, sin_dev, k_cache_dev, v_cache_dev, out_dev, B, Hq, Hkv, D,
+                                          cache_len, pos_dev, strides, scale, dtype, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tpamd_linear_w8(const void *x_dev, const void *wq_dev, const void *scale_dev, const void *outlier_idx_dev,

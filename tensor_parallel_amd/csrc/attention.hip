@@ -77,6 +77,9 @@ struct AttnParams {
     char *k_cache_w, *v_cache_w;  // k and v above, writable
     int64_t cs_b, nk_sb, nk_sh, nv_sb, nv_sh;
     int force_partials;
+    // The number of cached positions read on the device (tpamd_attention_decode_rope_devpos): Skv above is then the
+    // capacity of the caches, which the launch geometry is made for, and the kernels take the key count from here.
+    const int64_t *skv_dev;
 };
 
 constexpr int AT_KEYS = 64;   // keys per tile
@@ -99,6 +102,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, lq = lane >> 4;
     const int nrows = p.G * p.Sq;
+    // keys in the cache and keys per block of a split: launch arguments, or derived from a count that lives on the device
+    int Skv = p.Skv, keys_per_split = p.keys_per_split;
+    if (p.skv_dev != nullptr) {
+        const int64_t have = *p.skv_dev;
+        Skv = have < 0 ? 0 : have < p.Skv ? static_cast<int>(have) : p.Skv;
+        keys_per_split = ((Skv + p.nsplit - 1) / p.nsplit + AT_KEYS - 1) / AT_KEYS * AT_KEYS;
+    }
     // Causal: a block's key range grows with the positions of its rows, and blocks are handed to the 8 XCDs in turn, so
     // the order must not let block lengths repeat with a period that divides 8 (position tiles within a head do:
     // one XCD would get every longest block and the kernel would take as long as without the mask). The (batch, kv head)
@@ -116,7 +126,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     }
     const int b = bh / p.Hkv, hkv = bh % p.Hkv;
     const int row0 = row_tile * ROWS;
-    const int shift = p.Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
+    const int shift = Skv - p.Sq;  // causal: key j visible to position sq iff j <= sq + shift
 
     // Causal: the wavefronts that own a block's first rows stop early (below), and a wavefront's number fixes its SIMD, so
     // every other row tile hands the rows out in the opposite order.
@@ -132,7 +142,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
         const int g = row_ok[r] ? row[r] / p.Sq : 0;
         sq[r] = row_ok[r] ? row[r] % p.Sq : 0;
         head[r] = hkv * p.G + g;
-        my_lim[r] = p.causal ? sq[r] + shift : p.Skv - 1;  // last key this row may see
+        my_lim[r] = p.causal ? sq[r] + shift : Skv - 1;  // last key this row may see
         const char *qrow = p.q + (static_cast<int64_t>(b) * p.q_sb + static_cast<int64_t>(hkv) * p.q_sg + static_cast<int64_t>(g) * p.q_sh + static_cast<int64_t>(sq[r]) * p.q_ss) * 2;
 #pragma unroll
         for (int kk = 0; kk < DK; ++kk)
@@ -154,8 +164,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     }
 
     // ---- key range of this block
-    int k_begin = blockIdx.z * p.keys_per_split;
-    int k_end = k_begin + p.keys_per_split < p.Skv ? k_begin + p.keys_per_split : p.Skv;
+    int k_begin = blockIdx.z * keys_per_split;
+    int k_end = k_begin + keys_per_split < Skv ? k_begin + keys_per_split : Skv;
+    if (k_begin > k_end) k_begin = k_end;  // a split behind the last key (count read on the device): an empty range
     if (p.causal) {
         // the largest position among this block's rows (a block that straddles two heads contains position Sq - 1)
         const int last_row = row0 + ROWS - 1 < nrows - 1 ? row0 + ROWS - 1 : nrows - 1;
@@ -222,7 +233,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) voi
     // loads are unconditional and sit on no branch, so the compiler can count, per slot, how many younger loads may still
     // be in flight when a slot is written to LDS, instead of waiting for all of them. A key past the end of the range reads
     // the first key of the range instead: finite numbers, whose scores are masked and whose probabilities are 0.
-    const int64_t k_safe = k_begin < p.Skv ? k_begin : 0;
+    const int64_t k_safe = k_begin < Skv ? k_begin : 0;
     auto fetch_slot = [&](auto slot, int tile) {
         static_for<LPT>([&](auto jc) {
             constexpr int S = decltype(slot)::value, j = decltype(jc)::value;
@@ -532,9 +543,17 @@ __global__ __launch_bounds__(256) void attention_combine_newkey_kernel(AttnParam
 #pragma unroll
     for (int d = 1; d < per_row; d *= 2) dot += __shfl_xor(dot, d);
     const float x_new = dot * p.scale_log2;
-    if (live && row == 0) {  // the new position's cache rows
-        *reinterpret_cast<uint2 *>(p.k_cache_w + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh + static_cast<int64_t>(p.Skv) * p.k_ss + d4) * 2) = kr;
-        *reinterpret_cast<uint2 *>(p.v_cache_w + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh + static_cast<int64_t>(p.Skv) * p.v_ss + d4) * 2) = vn;
+    // where the new position goes: a launch argument, or the count on the device (then p.Skv is the caches' capacity, and a
+    // count that has reached it leaves the caches alone)
+    int64_t pos = p.Skv;
+    bool room = true;
+    if (p.skv_dev != nullptr) {
+        pos = *p.skv_dev;
+        room = pos >= 0 && pos < p.Skv;
+    }
+    if (live && row == 0 && room) {  // the new position's cache rows
+        *reinterpret_cast<uint2 *>(p.k_cache_w + (static_cast<int64_t>(b) * p.k_sb + static_cast<int64_t>(hkv) * p.k_sh + pos * p.k_ss + d4) * 2) = kr;
+        *reinterpret_cast<uint2 *>(p.v_cache_w + (static_cast<int64_t>(b) * p.v_sb + static_cast<int64_t>(hkv) * p.v_sh + pos * p.v_ss + d4) * 2) = vn;
     }
     if (!live) return;
 
@@ -700,9 +719,11 @@ int attention_dispatch(const void *q, const void *k, const void *v, void *o, int
 // One new position per sequence on a cache of `pos0` positions. strides (elements): {q batch, q head, q group, k batch,
 // k head, v batch, v head, cos/sin batch, k_cache batch, k_cache head, k_cache position, v_cache batch, v_cache head,
 // v_cache position, out batch, out head}.
+// pos_dev == NULL: `pos0` positions are cached. Otherwise the count is read from *pos_dev by the kernels and `pos0` is the
+// capacity of the caches: the grid and the key splits are made for the capacity, the blocks share out the keys there are.
 int attention_decode_rope_dispatch(const void *q, const void *k, const void *v, const void *cos, const void *sin, void *k_cache,
                                    void *v_cache, void *o, int64_t B, int64_t Hq, int64_t Hkv, int64_t D, int64_t pos0,
-                                   const int64_t *strides, float scale, int dtype, hipStream_t s) {
+                                   const int64_t *pos_dev, const int64_t *strides, float scale, int dtype, hipStream_t s) {
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
     if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
@@ -719,6 +740,7 @@ int attention_decode_rope_dispatch(const void *q, const void *k, const void *v, 
     p.o = static_cast<char *>(o);
     p.B = static_cast<int>(B); p.Hq = static_cast<int>(Hq); p.Hkv = static_cast<int>(Hkv);
     p.Sq = 1; p.Skv = static_cast<int>(pos0); p.G = static_cast<int>(Hq / Hkv);
+    p.skv_dev = pos_dev;
     p.q_sb = strides[0]; p.q_sh = strides[1]; p.q_sg = strides[2]; p.q_ss = 0;
     p.nk_sb = strides[3]; p.nk_sh = strides[4];
     p.nv_sb = strides[5]; p.nv_sh = strides[6];
