@@ -628,8 +628,27 @@ def llama_layer_decode(torch, dev) -> dict:
         us = _time_us(torch, step, 5, 30)
         res[label] = {"us_per_step": us, "tokens_per_s": B / us * 1e6}
         del m, cache
+    # the same step on a static cache (the count of cached positions stays on the device), recorded once as a HIP graph
+    from transformers import StaticCache
+
+    m = tp.tensor_parallel(deepcopy(model), [dev, dev])
+    tp.attention.fuse_rotary_(m, assume_no_padding=True)
+    cache = StaticCache(config=cfg, max_cache_len=L + 64)
+    m(input_ids=prompt, past_key_values=cache, use_cache=True)
+    graphed = tp.graphs.capture(m, input_ids=tok, past_key_values=cache, use_cache=True)
+    counts = [layer.cumulative_length for c in [cache] + cache.__dict__["_tp_rank_siblings"] for layer in c.layers]
+
+    def replay(i):
+        graphed.replay()
+        for count in counts:  # back to 2048 cached positions (the counterpart of the crop above)
+            count.sub_(1)
+
+    us = _time_us(torch, replay, 5, 30)
+    res["fuse_rotary_static_cache_graph"] = {"us_per_step": us, "tokens_per_s": B / us * 1e6}
+    del m, cache, graphed
     res["what"] = ("tp.tensor_parallel(2-layer Llama-2-7B-shaped decoder, W=2) decode step, batch 8 on 2048 cached positions, both rank "
-                   "shards on this GPU, host orchestration and the cache crop included")
+                   "shards on this GPU, host orchestration and the cache crop included; the last entry: transformers' StaticCache, "
+                   "fuse_rotary_(assume_no_padding=True), the whole step replayed as one HIP graph (tp.graphs.capture)")
     return res
 
 

@@ -81,6 +81,18 @@ def _cache_layer(cache, layer_idx: int):
     return layer if type(layer) is DynamicLayer else None
 
 
+def _static_layer(cache, layer_idx: int):
+    """Layer `layer_idx` of a transformers static cache (preallocated keys / values, the number of cached positions kept on
+    the device as `cumulative_length`), or None."""
+    from transformers.cache_utils import StaticLayer
+
+    layers = getattr(cache, "layers", None)
+    if layers is None or getattr(cache, "offloading", False) or len(layers) <= layer_idx:
+        return None
+    layer = layers[layer_idx]
+    return layer if type(layer) is StaticLayer else None
+
+
 def _buffers_with_room(layer, B: int, Hkv: int, D: int, need: int, like: torch.Tensor):
     """(k, v) buffers [B, Hkv, capacity >= need, D] that hold the layer's cached positions: the ones its keys / values are
     views of when they still are and have room, else new ones (twice the need) with the cached positions copied over."""
@@ -107,14 +119,17 @@ def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings
                           **kwargs):
     own = type(self).forward
     D = getattr(self, "head_dim", None)
-    layer = None
-    usable = (position_embeddings is not None and attention_mask is None and past_key_values is not None and not self.training
+    layer = static = None
+    no_padding = self.__dict__.get("_tp_no_padding", False)  # the caller's word: masks are the causal pattern and nothing else
+    usable = (position_embeddings is not None and past_key_values is not None and not self.training
               and hidden_states.dim() == 3 and hidden_states.device.type == "cuda"
               and hidden_states.dtype in (torch.bfloat16, torch.float16) and D in (64, 128)
               and not kwargs.get("output_attentions") and getattr(self, "is_causal", True))
-    if usable:
+    if usable and (attention_mask is None or no_padding):
         layer = _cache_layer(past_key_values, self.layer_idx)
-    if layer is None:
+        if layer is None and no_padding:  # a static cache always comes with a materialised mask
+            static = _static_layer(past_key_values, self.layer_idx)
+    if layer is None and static is None:
         return own(self, hidden_states, position_embeddings=position_embeddings, attention_mask=attention_mask,
                    past_key_values=past_key_values, **kwargs)
     B, S, _ = hidden_states.shape
@@ -124,9 +139,29 @@ def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings
     Hq, Hkv = q.shape[2], k.shape[2]
     cos, sin = position_embeddings
     cos, sin = cos.to(q.dtype), sin.to(q.dtype)
+    scale = getattr(self, "scaling", None)
+    if static is not None:
+        # Preallocated keys / values and a count that lives on the device: a decode step reads the count inside the kernels
+        # (no host value depends on the step, so the forward can be replayed as a HIP graph); a prefill reads it back.
+        if not static.is_initialized:
+            static.lazy_initialization(k.transpose(1, 2), v.transpose(1, 2))
+        kb, vb = static.keys, static.values
+        if kb.shape[0] != B or kb.shape[1] != Hkv or kb.shape[3] != D or kb.dtype != q.dtype:
+            raise ValueError(f"the static cache of layer {self.layer_idx} holds {tuple(kb.shape)} {kb.dtype}, this call needs "
+                             f"[{B}, {Hkv}, positions, {D}] {q.dtype}")
+        count = static.cumulative_length
+        if S == 1:
+            out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, count.reshape(1), scale=scale)
+        else:
+            pos0 = int(count)
+            if pos0 + S > kb.shape[2]:
+                raise ValueError(f"{pos0} cached + {S} new positions do not fit the static cache of {kb.shape[2]}")
+            q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
+            out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=scale, causal=True)
+        count.add_(S)
+        return self.o_proj(out.reshape(B, S, Hq * D)), None
     pos0 = layer.get_seq_length()
     kb, vb = _buffers_with_room(layer, B, Hkv, D, pos0 + S, q)
-    scale = getattr(self, "scaling", None)
     if S == 1:
         out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, pos0, scale=scale)
     else:
@@ -210,7 +245,11 @@ def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, 
     `class_names` and whose structure is the Llama pattern the forward described in the module docstring. Returns how many
     modules took it. Name further classes only when their forward is the same sequence of operations.
 
-    `assume_no_padding=True` also takes transformers' FalconAttention (rotary, grouped heads: the 40B layout): that model
+    `assume_no_padding=True` is the caller's word that the batches carry no padding, so that a mask handed to an attention
+    module is the causal pattern and can be ignored. With it the Llama-pattern modules also take transformers' static
+    caches (which always come with a materialised mask): preallocated keys and values whose number of cached positions
+    lives on the device, read there by the decode kernels, so that a decode step makes no host decision that depends
+    on the step and `tp.graphs.capture` can record it once and replay it for every new token. It also takes transformers' FalconAttention (rotary, grouped heads: the 40B layout): that model
     hands its attention modules a materialised mask on every call, which cannot be told from a padding mask without
     reading it back, so the caller vouches that the batches carry no padding and the mask is ignored. Such a module then
     caches its key/value heads once, not once per query head as its own forward does: every call of a fused model must
@@ -221,6 +260,8 @@ def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, 
             continue
         if _is_llama_pattern(module, class_names):
             module.forward = types.MethodType(_fused_rotary_forward, module)
+            if assume_no_padding:
+                module.__dict__["_tp_no_padding"] = True
             count += 1
         elif assume_no_padding and _is_rotary_falcon(module):
             module.forward = types.MethodType(_fused_falcon_forward, module)

@@ -8,14 +8,25 @@ on one HIP device run on one stream of one thread (the ranks are greenlets of th
     graphed = tp.graphs.capture(model, input_ids=ids, use_cache=False)
     out = graphed(input_ids=other_ids)        # same shapes; new values are copied into the captured inputs
 
-What a capture fixes: every shape, every argument that is not a tensor, and every host-side decision the forward took
-(a key/value cache that grows from call to call therefore stays outside). The tensors inside the returned value are
-the graph's own output buffers: the next replay overwrites them.
+What a capture fixes: every shape, every argument that is not a tensor, and every host-side decision the forward took.
+A key/value cache that grows from call to call therefore stays outside; a decode step on one of transformers' static
+caches (preallocated, its number of cached positions kept on the device) can be captured once the attention modules
+read that count on the device, which `tp.attention.fuse_rotary_(model, assume_no_padding=True)` makes them do:
+
+    cache = StaticCache(config=model.config, max_cache_len=4096)
+    model(input_ids=prompt, past_key_values=cache, use_cache=True)                  # the prefill, eager
+    step = tp.graphs.capture(model, input_ids=token, past_key_values=cache, use_cache=True)
+    logits = step(input_ids=next_token, past_key_values=cache, use_cache=True).logits   # every further token: one replay
+
+The forwards that a capture runs beforehand (to let first uses happen outside it) advance such a cache like any other
+forward: the counts of static caches among the arguments, and the tensors named in `restore`, are put back to what
+they were before `capture` returns; what those forwards wrote behind the count is overwritten by the steps that follow.
+The tensors inside the returned value are the graph's own output buffers: the next replay overwrites them.
 """
 from __future__ import annotations
 
 import importlib
-from typing import Any, List, Tuple
+from typing import Any, List, Sequence, Tuple
 
 import torch
 from torch import nn
@@ -44,10 +55,28 @@ def _rebuild(value: Any, replace) -> Any:
     return replace(value)
 
 
+def _caches_with_counts(leaves) -> list:
+    """Cache objects among the arguments whose layers keep a count of cached positions on the device, with the per-rank
+    siblings that `tp.TensorParallel` gave them."""
+    found = []
+    for _, value in leaves:
+        layers = getattr(value, "layers", None)
+        if isinstance(layers, list) and any(hasattr(layer, "cumulative_length") for layer in layers):
+            found.append(value)
+    return found
+
+
+def _count_tensors(cache) -> list:
+    out = []
+    for one in [cache] + list(cache.__dict__.get("_tp_rank_siblings") or []):
+        out.append([getattr(layer, "cumulative_length", None) for layer in one.layers])
+    return out
+
+
 class GraphedForward:
     """`module(*args, **kwargs)` captured once; calls replay it on new values of the same tensors."""
 
-    def __init__(self, module: nn.Module, *args, warmup: int = 2, **kwargs):
+    def __init__(self, module: nn.Module, *args, warmup: int = 2, restore: Sequence[torch.Tensor] = (), **kwargs):
         # (the package attribute `tensor_parallel` is the factory function, not the module)
         tp_module = importlib.import_module(__package__ + ".tensor_parallel")
 
@@ -67,6 +96,10 @@ class GraphedForward:
         # the captured inputs: clones that the replays read
         self._static_args, self._static_kwargs = _rebuild((args, kwargs), lambda v: v.clone() if isinstance(v, torch.Tensor) else v)
         self._static_leaves = self._leaves(self._static_args, self._static_kwargs)
+        # state that the forwards below advance and that is put back afterwards
+        caches = _caches_with_counts(self._static_leaves)
+        counts_before = [[None if c is None else c.clone() for c in _count_tensors(cache)[0]] for cache in caches]
+        kept = [(t, t.clone()) for t in restore]
         with torch.cuda.device(self.device):
             stream = torch.cuda.Stream()
             stream.wait_stream(torch.cuda.current_stream())
@@ -79,6 +112,14 @@ class GraphedForward:
             self.graph = torch.cuda.CUDAGraph()
             with torch.no_grad(), torch.cuda.graph(self.graph, stream=stream):
                 self.output = module(*self._static_args, **self._static_kwargs)
+            with torch.no_grad():
+                for cache, before in zip(caches, counts_before):
+                    for per_rank in _count_tensors(cache):  # the rank siblings exist by now; every rank's layer i holds the same count
+                        for count, was in zip(per_rank, before):
+                            if isinstance(count, torch.Tensor):
+                                count.fill_(0) if was is None else count.copy_(was)
+                for tensor, was in kept:
+                    tensor.copy_(was)
         self._stream = stream  # its scratch buffer in the library belongs to the graph from now on
 
     @staticmethod
@@ -113,7 +154,8 @@ class GraphedForward:
         return self._static_args, self._static_kwargs
 
 
-def capture(module: nn.Module, *args, warmup: int = 2, **kwargs) -> GraphedForward:
+def capture(module: nn.Module, *args, warmup: int = 2, restore: Sequence[torch.Tensor] = (), **kwargs) -> GraphedForward:
     """Record `module(*args, **kwargs)` (inference, no gradients) as a HIP graph; the result is called with new values of
-    the same tensors and returns the forward's value."""
-    return GraphedForward(module, *args, warmup=warmup, **kwargs)
+    the same tensors and returns the forward's value. `restore`: tensors that a forward changes in place and that are to
+    hold their present values again when this returns."""
+    return GraphedForward(module, *args, warmup=warmup, restore=restore, **kwargs)

@@ -128,3 +128,42 @@ def test_fused_rotary_falcon_inside_tensor_parallel():
     assert caches[1].get_seq_length() == 74
     # the fused forward keeps this rank's key/value heads once (2 of the 4 groups), the module's own one copy per query head
     assert caches[1].layers[0].keys.shape == (2, 2, 74, 64) and caches[0].layers[0].keys.shape == (2, 4, 74, 64)
+
+
+def test_static_cache_decode_eager_and_as_one_graph():
+    """A transformers static cache behind the fused attention forward: the count of cached positions stays on the device
+    (the decode kernels read it there), so one captured decode step is replayed for every new token. Against the same model
+    with the module's own forward on a growing cache, step by step."""
+    from transformers import DynamicCache, StaticCache
+
+    model = tiny_llama(torch.bfloat16)
+    plain = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    fused = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    assert tp.attention.fuse_rotary_(fused, assume_no_padding=True) == 2 * 2
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(2, 300, (2, 37), generator=g).to(DEV)
+    steps = [torch.randint(2, 300, (2, 1), generator=g).to(DEV) for _ in range(40)]  # past a tile of 64 keys
+    growing, static = DynamicCache(), StaticCache(config=model.config, max_cache_len=128)
+    with torch.no_grad():
+        want = plain(input_ids=ids, past_key_values=growing, use_cache=True).logits.float()
+        got = fused(input_ids=ids, past_key_values=static, use_cache=True).logits.float()
+        scale = want.std().item()
+        torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * scale)
+        for tok in steps[:2]:  # eager decode steps
+            want = plain(input_ids=tok, past_key_values=growing, use_cache=True).logits.float()
+            got = fused(input_ids=tok, past_key_values=static, use_cache=True).logits.float()
+            torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * scale)
+        assert int(static.get_seq_length()) == 39
+        step = tp.graphs.capture(fused, input_ids=steps[2], past_key_values=static, use_cache=True)
+        # the forwards that a capture runs first advanced every rank's counts; they are back where they were
+        for cache in [static] + static.__dict__["_tp_rank_siblings"]:
+            assert [int(layer.cumulative_length) for layer in cache.layers] == [39, 39]
+        for i, tok in enumerate(steps[2:]):
+            got = step(input_ids=tok, past_key_values=static, use_cache=True).logits.float().clone()
+            torch.cuda.synchronize()
+            want = plain(input_ids=tok, past_key_values=growing, use_cache=True).logits.float()  # eager work between the replays
+            torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * scale, msg=lambda m: f"replayed step {i}: {m}")
+        assert int(static.get_seq_length()) == growing.get_seq_length() == 37 + 40
+    # the first layer sees the same inputs in both models: its cached keys (rotated by the kernel / by torch) are the same bits
+    k_static = static.layers[0].keys[:, :, :77]
+    assert torch.equal(k_static.view(torch.int16), growing.layers[0].keys.view(torch.int16))
