@@ -104,6 +104,12 @@ class TensorParallelPreTrainedModel(PreTrainedModel, GenerationMixin):
     def _supports_default_dynamic_cache(self) -> bool:
         return self.wrapped_model.module_shards[0]._supports_default_dynamic_cache()
 
+    def _valid_auto_compile_criteria(self, model_kwargs, generation_config) -> bool:
+        # `generate` wraps the forward in torch.compile when it is given a static cache. The rank shards call a C ABI
+        # through ctypes and take turns as greenlets, which a tracing compiler cannot follow: the forward stays as it is
+        # (`tp.graphs.capture` is this package's way to take the host out of a decode step).
+        return False
+
     def get_encoder(self, *args, **kwargs):
         shards = self.wrapped_model.module_shards
         assert len(shards), "Can't get encoder since no module shards present"

@@ -167,3 +167,16 @@ def test_static_cache_decode_eager_and_as_one_graph():
     # the first layer sees the same inputs in both models: its cached keys (rotated by the kernel / by torch) are the same bits
     k_static = static.layers[0].keys[:, :, :77]
     assert torch.equal(k_static.view(torch.int16), growing.layers[0].keys.view(torch.int16))
+
+
+def test_generate_on_a_static_cache():
+    """`generate(cache_implementation="static")`: transformers would hand the forward to torch.compile for such a cache; the
+    wrapper declines that, and the tokens are those of the growing cache."""
+    model = tiny_llama(torch.bfloat16)
+    plain = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    fused = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    tp.attention.fuse_rotary_(fused, assume_no_padding=True)
+    ids = torch.randint(2, 300, (2, 12), generator=torch.Generator().manual_seed(0)).to(DEV)
+    want = plain.generate(ids, max_new_tokens=8, do_sample=False)
+    got = fused.generate(ids, max_new_tokens=8, do_sample=False, cache_implementation="static")
+    assert torch.equal(got, want)
