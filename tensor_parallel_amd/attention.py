@@ -115,6 +115,64 @@ def _buffers_with_room(layer, B: int, Hkv: int, D: int, need: int, like: torch.T
     return bufs
 
 
+def _share_qkv_storage(module: torch.nn.Module) -> bool:
+    """Lay the weights of q_proj / k_proj / v_proj out as one [Nq + Nk + Nv, K] matrix (each Linear's weight becomes a view
+    of its rows), so that the fused forward makes one projection call instead of three. Only for plain shard Linears with
+    16-bit weights on one HIP device and all or none with a bias."""
+    from .shard_modules import ShardLinear, _has_hooks
+
+    parts = [module._modules.get(n) for n in ("q_proj", "k_proj", "v_proj")]
+    if not all(type(p) is ShardLinear and not _has_hooks(p) for p in parts):
+        return False
+    ws = [p.weight for p in parts]
+    first = ws[0]
+    if first.device.type != "cuda" or first.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if any(w.dtype != first.dtype or w.device != first.device or w.dim() != 2 or w.shape[1] != first.shape[1] for w in ws):
+        return False
+    biases = [p.bias for p in parts]
+    if any(b is None for b in biases) != all(b is None for b in biases):
+        return False
+    with torch.no_grad():
+        fused_w = torch.cat([w.detach() for w in ws], 0)
+        fused_b = None if biases[0] is None else torch.cat([b.detach() for b in biases], 0)
+        row = 0
+        for p, w, b in zip(parts, ws, biases):
+            n = w.shape[0]
+            p.weight = torch.nn.Parameter(fused_w[row:row + n], requires_grad=w.requires_grad)
+            if b is not None:
+                p.bias = torch.nn.Parameter(fused_b[row:row + n], requires_grad=b.requires_grad)
+            row += n
+    module.__dict__["_tp_qkv"] = (fused_w, fused_b)
+    return True
+
+
+def _project_qkv(self, hidden_states: torch.Tensor, D: int):
+    """q, k, v as [B, S, heads, D]: one call on the shared weight matrix when the three Linears still are views of it."""
+    from .shard_modules import ShardLinear, _guard
+
+    B, S, _ = hidden_states.shape
+    shared = self.__dict__.get("_tp_qkv")
+    if shared is not None:
+        w, b = shared
+        q_proj, k_proj, v_proj = self.q_proj, self.k_proj, self.v_proj
+        intact = type(q_proj) is ShardLinear and type(k_proj) is ShardLinear and type(v_proj) is ShardLinear
+        if intact:
+            nk = k_proj.weight.shape[0]
+            nq = w.shape[0] - 2 * nk
+            row_bytes = w.stride(0) * w.element_size()
+            intact = (q_proj.weight.data_ptr() == w.data_ptr() and q_proj.weight.shape[0] == nq and v_proj.weight.shape[0] == nk
+                      and k_proj.weight.data_ptr() == w.data_ptr() + nq * row_bytes
+                      and v_proj.weight.data_ptr() == w.data_ptr() + (nq + nk) * row_bytes)
+        if intact and hidden_states.dtype == w.dtype:
+            qkv = _guard(_native.linear(hidden_states.detach(), w, b), hidden_states, q_proj.weight)
+            return (qkv[..., :nq].view(B, S, -1, D), qkv[..., nq:nq + nk].view(B, S, -1, D), qkv[..., nq + nk:].view(B, S, -1, D))
+        if not intact:  # a projection was replaced (quantised, re-assigned): three calls from now on
+            del self.__dict__["_tp_qkv"]
+    return (self.q_proj(hidden_states).view(B, S, -1, D), self.k_proj(hidden_states).view(B, S, -1, D),
+            self.v_proj(hidden_states).view(B, S, -1, D))
+
+
 def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings=None, attention_mask=None, past_key_values=None,
                           **kwargs):
     own = type(self).forward
@@ -133,9 +191,7 @@ def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings
         return own(self, hidden_states, position_embeddings=position_embeddings, attention_mask=attention_mask,
                    past_key_values=past_key_values, **kwargs)
     B, S, _ = hidden_states.shape
-    q = self.q_proj(hidden_states).view(B, S, -1, D)
-    k = self.k_proj(hidden_states).view(B, S, -1, D)
-    v = self.v_proj(hidden_states).view(B, S, -1, D)
+    q, k, v = _project_qkv(self, hidden_states, D)
     Hq, Hkv = q.shape[2], k.shape[2]
     cos, sin = position_embeddings
     cos, sin = cos.to(q.dtype), sin.to(q.dtype)
@@ -240,7 +296,8 @@ def _is_rotary_falcon(module: torch.nn.Module) -> bool:
     return getattr(config, "alibi", True) is False and module.new_decoder_architecture and getattr(module, "layer_idx", None) is not None
 
 
-def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, assume_no_padding: bool = False) -> int:
+def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, assume_no_padding: bool = False,
+                 share_qkv: bool = True) -> int:
     """Give every attention module under `model` (before or after `tp.tensor_parallel`) whose class is named in
     `class_names` and whose structure is the Llama pattern the forward described in the module docstring. Returns how many
     modules took it. Name further classes only when their forward is the same sequence of operations.
@@ -253,7 +310,12 @@ def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, 
     hands its attention modules a materialised mask on every call, which cannot be told from a padding mask without
     reading it back, so the caller vouches that the batches carry no padding and the mask is ignored. Such a module then
     caches its key/value heads once, not once per query head as its own forward does: every call of a fused model must
-    be one the fused forward takes (16-bit tensors on the device, a growing cache, inference)."""
+    be one the fused forward takes (16-bit tensors on the device, a growing cache, inference).
+
+    `share_qkv=True` (Llama pattern, rank shards already on the device): the weights of q_proj / k_proj / v_proj move into
+    one matrix that each of them keeps a view of (names, shapes and values in `state_dict` stay what they were), and the
+    fused forward multiplies by it once instead of three times: two launches and two host calls fewer per module and
+    decode step. A projection that is replaced later (quantised, say) ends the sharing for its module."""
     count = 0
     for module in model.modules():
         if "forward" in module.__dict__:
@@ -262,6 +324,8 @@ def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, 
             module.forward = types.MethodType(_fused_rotary_forward, module)
             if assume_no_padding:
                 module.__dict__["_tp_no_padding"] = True
+            if share_qkv:
+                _share_qkv_storage(module)
             count += 1
         elif assume_no_padding and _is_rotary_falcon(module):
             module.forward = types.MethodType(_fused_falcon_forward, module)

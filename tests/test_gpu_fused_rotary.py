@@ -180,3 +180,34 @@ def test_generate_on_a_static_cache():
     want = plain.generate(ids, max_new_tokens=8, do_sample=False)
     got = fused.generate(ids, max_new_tokens=8, do_sample=False, cache_implementation="static")
     assert torch.equal(got, want)
+
+
+def test_shared_qkv_storage_keeps_the_state_and_survives_a_replaced_projection():
+    from transformers import DynamicCache
+
+    model = tiny_llama(torch.bfloat16)
+    separate = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    shared = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    before = {k: v.clone() for k, v in shared.state_dict().items()}
+    assert tp.attention.fuse_rotary_(separate, share_qkv=False) == 4
+    assert tp.attention.fuse_rotary_(shared) == 4
+    attn = shared.wrapped_model.module_shards[1].model.layers[0].self_attn.tp_wrapped_module
+    w, b = attn.__dict__["_tp_qkv"]
+    assert b is None and w.shape == (2 * 64 + 64 + 64, 256)  # this rank's 2 query heads and 1 key/value head
+    assert attn.k_proj.weight.data_ptr() == w.data_ptr() + 128 * 256 * 2
+    after = shared.state_dict()
+    assert after.keys() == before.keys() and all(torch.equal(after[k], before[k]) for k in before)  # un-sharded: the model's own weights
+    g = torch.Generator().manual_seed(4)
+    ids = torch.randint(2, 300, (2, 20), generator=g).to(DEV)
+    tok = torch.randint(2, 300, (2, 1), generator=g).to(DEV)
+    caches = [DynamicCache(), DynamicCache()]
+    with torch.no_grad():
+        for inp in (ids, tok, tok):
+            a, b2 = (m(input_ids=inp, past_key_values=c, use_cache=True).logits.float() for m, c in zip((separate, shared), caches))
+            torch.testing.assert_close(b2, a, rtol=RTOL, atol=RTOL * a.std().item())
+        # a projection replaced afterwards: the module goes back to three calls
+        assert tp.int8.quantize_linears_(shared, skip=lambda name, m: not name.endswith("layers.0.self_attn.tp_wrapped_module.k_proj")) == 2
+        want = separate(input_ids=tok, past_key_values=caches[0], use_cache=True).logits.float()
+        got = shared(input_ids=tok, past_key_values=caches[1], use_cache=True).logits.float()
+        assert "_tp_qkv" not in attn.__dict__
+        torch.testing.assert_close(got, want, rtol=5e-2, atol=5e-2 * want.std().item())  # one int8 projection in
