@@ -173,6 +173,48 @@ def _project_qkv(self, hidden_states: torch.Tensor, D: int):
             self.v_proj(hidden_states).view(B, S, -1, D))
 
 
+def _attend_on_cache(q, k, v, cos, sin, layer, static, scale, layer_idx: int) -> torch.Tensor:
+    """Rotary embedding of the new q / k rows, their hand-over to the cache and the attention core, for the new positions
+    q / k / v [B, S, heads, D] (views of the projection output): on the growing layer `layer`, or on the static layer
+    `static`. Returns [B, S, Hq, D] (5-dimensional grouped queries come back flat)."""
+    B, S, D = q.shape[0], q.shape[1], q.shape[-1]
+    Hkv = k.shape[2]
+    Hq = q.shape[2] if q.dim() == 4 else q.shape[2] * q.shape[3]
+    cos, sin = cos.to(k.dtype), sin.to(k.dtype)
+    if static is not None:
+        # Preallocated keys / values and a count that lives on the device: a decode step reads the count inside the kernels
+        # (no host value depends on the step, so the forward can be replayed as a HIP graph); a prefill reads it back.
+        if not static.is_initialized:
+            static.lazy_initialization(k.transpose(1, 2), v.transpose(1, 2))
+        kb, vb = static.keys, static.values
+        if kb.shape[0] != B or kb.shape[1] != Hkv or kb.shape[3] != D or kb.dtype != k.dtype:
+            raise ValueError(f"the static cache of layer {layer_idx} holds {tuple(kb.shape)} {kb.dtype}, this call needs "
+                             f"[{B}, {Hkv}, positions, {D}] {k.dtype}")
+        count = static.cumulative_length
+        if S == 1:
+            out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, count.reshape(1), scale=scale)
+        else:
+            pos0 = int(count)
+            if pos0 + S > kb.shape[2]:
+                raise ValueError(f"{pos0} cached + {S} new positions do not fit the static cache of {kb.shape[2]}")
+            q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
+            out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=scale, causal=True)
+        count.add_(S)
+        return out.reshape(B, S, Hq, D)
+    pos0 = layer.get_seq_length()
+    kb, vb = _buffers_with_room(layer, B, Hkv, D, pos0 + S, k)
+    if S == 1:
+        out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, pos0, scale=scale)
+    else:
+        q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
+        out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=scale, causal=True)
+    if not layer.is_initialized:
+        layer.dtype, layer.device = k.dtype, k.device
+        layer.is_initialized = True
+    layer.keys, layer.values = kb[:, :, :pos0 + S], vb[:, :, :pos0 + S]
+    return out.reshape(B, S, Hq, D)
+
+
 def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings=None, attention_mask=None, past_key_values=None,
                           **kwargs):
     own = type(self).forward
@@ -192,42 +234,9 @@ def _fused_rotary_forward(self, hidden_states: torch.Tensor, position_embeddings
                    past_key_values=past_key_values, **kwargs)
     B, S, _ = hidden_states.shape
     q, k, v = _project_qkv(self, hidden_states, D)
-    Hq, Hkv = q.shape[2], k.shape[2]
     cos, sin = position_embeddings
-    cos, sin = cos.to(q.dtype), sin.to(q.dtype)
-    scale = getattr(self, "scaling", None)
-    if static is not None:
-        # Preallocated keys / values and a count that lives on the device: a decode step reads the count inside the kernels
-        # (no host value depends on the step, so the forward can be replayed as a HIP graph); a prefill reads it back.
-        if not static.is_initialized:
-            static.lazy_initialization(k.transpose(1, 2), v.transpose(1, 2))
-        kb, vb = static.keys, static.values
-        if kb.shape[0] != B or kb.shape[1] != Hkv or kb.shape[3] != D or kb.dtype != q.dtype:
-            raise ValueError(f"the static cache of layer {self.layer_idx} holds {tuple(kb.shape)} {kb.dtype}, this call needs "
-                             f"[{B}, {Hkv}, positions, {D}] {q.dtype}")
-        count = static.cumulative_length
-        if S == 1:
-            out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, count.reshape(1), scale=scale)
-        else:
-            pos0 = int(count)
-            if pos0 + S > kb.shape[2]:
-                raise ValueError(f"{pos0} cached + {S} new positions do not fit the static cache of {kb.shape[2]}")
-            q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
-            out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=scale, causal=True)
-        count.add_(S)
-        return self.o_proj(out.reshape(B, S, Hq * D)), None
-    pos0 = layer.get_seq_length()
-    kb, vb = _buffers_with_room(layer, B, Hkv, D, pos0 + S, q)
-    if S == 1:
-        out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, pos0, scale=scale)
-    else:
-        q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
-        out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=scale, causal=True)
-    if not layer.is_initialized:
-        layer.dtype, layer.device = q.dtype, q.device
-        layer.is_initialized = True
-    layer.keys, layer.values = kb[:, :, :pos0 + S], vb[:, :, :pos0 + S]
-    return self.o_proj(out.reshape(B, S, Hq * D)), None
+    out = _attend_on_cache(q, k, v, cos, sin, layer, static, getattr(self, "scaling", None), self.layer_idx)
+    return self.o_proj(out.reshape(B, S, -1)), None
 
 
 def _fused_falcon_forward(self, hidden_states: torch.Tensor, alibi=None, attention_mask=None, position_ids=None, layer_past=None,
@@ -236,13 +245,15 @@ def _fused_falcon_forward(self, hidden_states: torch.Tensor, alibi=None, attenti
     hands this module a materialised mask; it is ignored here, which is what `fuse_rotary_(..., assume_no_padding=True)`
     was told is right (the mask is then the causal pattern the kernels apply themselves)."""
     D = self.head_dim
-    layer = None
+    layer = static = None
     usable = (alibi is None and position_embeddings is not None and layer_past is not None and not self.training and not output_attentions
               and self.new_decoder_architecture and hidden_states.dim() == 3 and hidden_states.device.type == "cuda"
               and hidden_states.dtype in (torch.bfloat16, torch.float16) and D in (64, 128))
     if usable:
         layer = _cache_layer(layer_past, self.layer_idx)
-    if layer is None:
+        if layer is None:
+            static = _static_layer(layer_past, self.layer_idx)
+    if layer is None and static is None:
         return type(self).forward(self, hidden_states, alibi, attention_mask, position_ids=position_ids, layer_past=layer_past,
                                   use_cache=use_cache, output_attentions=output_attentions, position_embeddings=position_embeddings, **kwargs)
     B, S, _ = hidden_states.shape
@@ -251,20 +262,8 @@ def _fused_falcon_forward(self, hidden_states: torch.Tensor, alibi=None, attenti
     per = self.num_heads // self.num_kv_heads
     qkv = fused_qkv.view(B, S, self.num_kv_heads, per + 2, D)
     q, k, v = qkv[:, :, :, :per], qkv[:, :, :, per], qkv[:, :, :, per + 1]
-    Hkv = self.num_kv_heads
     cos, sin = position_embeddings
-    cos, sin = cos.to(fused_qkv.dtype), sin.to(fused_qkv.dtype)
-    pos0 = layer.get_seq_length()
-    kb, vb = _buffers_with_room(layer, B, Hkv, D, pos0 + S, fused_qkv)
-    if S == 1:
-        out = _native.attention_decode_rope(q, k, v, cos, sin, kb, vb, pos0, scale=self.inv_norm_factor)
-    else:
-        q_rot = _native.rope_append(q, k, v, cos, sin, kb, vb, pos0)
-        out = _native.attention(q_rot, kb[:, :, :pos0 + S], vb[:, :, :pos0 + S], scale=self.inv_norm_factor, causal=True)
-    if not layer.is_initialized:
-        layer.dtype, layer.device = fused_qkv.dtype, fused_qkv.device
-        layer.is_initialized = True
-    layer.keys, layer.values = kb[:, :, :pos0 + S], vb[:, :, :pos0 + S]
+    out = _attend_on_cache(q, k, v, cos, sin, layer, static, self.inv_norm_factor, self.layer_idx)
     return self.dense(out.reshape(B, S, self.num_heads * D)), None
 
 

@@ -128,6 +128,21 @@ def test_fused_rotary_falcon_inside_tensor_parallel():
     assert caches[1].get_seq_length() == 74
     # the fused forward keeps this rank's key/value heads once (2 of the 4 groups), the module's own one copy per query head
     assert caches[1].layers[0].keys.shape == (2, 2, 74, 64) and caches[0].layers[0].keys.shape == (2, 4, 74, 64)
+    # the same model on a static cache, the decode step replayed as one HIP graph
+    from transformers import StaticCache
+
+    static = StaticCache(config=cfg, max_cache_len=96)
+    growing = DynamicCache()
+    with torch.no_grad():
+        want = plain(input_ids=ids, past_key_values=growing, use_cache=True).logits.float()
+        got = fused(input_ids=ids, past_key_values=static, use_cache=True).logits.float()
+        torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * scale)
+        step = tp.graphs.capture(fused, input_ids=steps[0], past_key_values=static, use_cache=True)
+        for i, tok in enumerate(steps):
+            got = step(input_ids=tok, past_key_values=static, use_cache=True).logits.float().clone()
+            want = plain(input_ids=tok, past_key_values=growing, use_cache=True).logits.float()
+            torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * scale, msg=lambda m: f"replayed step {i}: {m}")
+    assert int(static.get_seq_length()) == 74 and static.layers[0].keys.shape == (2, 2, 96, 64)
 
 
 def test_static_cache_decode_eager_and_as_one_graph():
