@@ -127,6 +127,8 @@ def main() -> int:
     ap.add_argument("--settle", type=int, default=240, help="untimed steps before the counted warm-up (clock settling)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--no-model-graphs", action="store_true",
+                    help="leave out the two figures that replay a whole model forward as a HIP graph (counter-collecting profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the tensor-parallel layer; --gpus above 1 is not supported "
@@ -221,7 +223,7 @@ def main() -> int:
         "roofline": roofline,
     }
     if not args.no_extra:
-        out["extra"] = extra_measurements(torch, _native, dev, sets, other)
+        out["extra"] = extra_measurements(torch, _native, dev, sets, other, model_graphs=not args.no_model_graphs)
         out["extra"]["copy_bandwidth"] = copy_bandwidth(torch, _native, dev)
         add_copy_fractions(out["extra"], out["extra"]["copy_bandwidth"]["GBps"])
     if not args.no_cpu_baseline:
@@ -290,7 +292,7 @@ def _time_us(torch, fn, warm, iters):
     return a.elapsed_time(b) / iters * 1e3
 
 
-def extra_measurements(torch, _native, dev, sets, other) -> dict:
+def extra_measurements(torch, _native, dev, sets, other, model_graphs: bool = True) -> dict:
     """The other two targets of the same path, reported beside the headline: decode (M = 1, HBM-bound) and
     state-dict slicing (every split tensor of a Llama-2-7B-shaped dict, all ranks' shards, W = 2, HBM-bound)."""
     extra = {}
@@ -346,7 +348,7 @@ def extra_measurements(torch, _native, dev, sets, other) -> dict:
     extra["attention_falcon40b_shard"] = attention_extra(torch, _native, dev)
     extra["c4_decode_step"] = falcon_attention_decode_step(torch, _native, dev)
     extra["c4_prefill_step"] = falcon_attention_prefill_step(torch, _native, dev)
-    extra.update(api_level_extras(torch, dev))
+    extra.update(api_level_extras(torch, dev, model_graphs))
 
     from types import SimpleNamespace
 
@@ -519,7 +521,7 @@ def falcon_attention_prefill_step(torch, _native, dev) -> dict:
             "algorithmic_flops": flops, "step": "qkv projection + rotary/cache fill + causal attention core + dense projection, eager"}
 
 
-def api_level_extras(torch, dev) -> dict:
+def api_level_extras(torch, dev, model_graphs: bool = True) -> dict:
     """Two figures through the package's Python surface (tp.TensorParallel / tp.tensor_parallel), host orchestration
     included, with BOTH rank shards on this one GPU:
     c2_tp_module_m4096: the Llama-7B MLP (d 4096, ffn 11008, bf16) split by the Llama rules at W = 2, 4096 tokens per
@@ -580,16 +582,18 @@ def api_level_extras(torch, dev) -> dict:
         us = _time_us(torch, lambda i: opt_tp(input_ids=ids, use_cache=False).logits, 5, 20)
         out["c1_opt125m"] = {"us_per_forward": us, "tokens_per_s": 128 / us * 1e6, "dtype": "f32",
                              "what": "tp.tensor_parallel(OPT-125m, W=2) forward of 2 x 64 tokens, both rank shards on this GPU, host orchestration included"}
-        graphed = tp.graphs.capture(opt_tp, input_ids=ids, use_cache=False)
-        us_g = _time_us(torch, lambda i: graphed.replay().logits, 5, 20)
-        out["c1_opt125m"]["graph"] = {"us_per_forward": us_g, "tokens_per_s": 128 / us_g * 1e6,
-                                      "what": "the same forward recorded once with tp.graphs.capture and replayed as a HIP graph"}
-        del graphed, opt_tp, model
-        out["llama_layer_decode_tp"] = llama_layer_decode(torch, dev)
+        if model_graphs:
+            graphed = tp.graphs.capture(opt_tp, input_ids=ids, use_cache=False)
+            us_g = _time_us(torch, lambda i: graphed.replay().logits, 5, 20)
+            out["c1_opt125m"]["graph"] = {"us_per_forward": us_g, "tokens_per_s": 128 / us_g * 1e6,
+                                          "what": "the same forward recorded once with tp.graphs.capture and replayed as a HIP graph"}
+            del graphed
+        del opt_tp, model
+        out["llama_layer_decode_tp"] = llama_layer_decode(torch, dev, model_graphs)
     return out
 
 
-def llama_layer_decode(torch, dev) -> dict:
+def llama_layer_decode(torch, dev, model_graphs: bool = True) -> dict:
     """One decode step of a Llama-2-7B-shaped decoder (2 layers: d 4096, 32 heads of 128, ffn 11008, bf16) through
     tp.tensor_parallel at W = 2 with both rank shards on this GPU, batch 8 on 2048 cached positions, host orchestration
     included: the wrapped attention modules with their own forward (torch rotary embedding and cache update, the library's
@@ -628,6 +632,10 @@ def llama_layer_decode(torch, dev) -> dict:
         us = _time_us(torch, step, 5, 30)
         res[label] = {"us_per_step": us, "tokens_per_s": B / us * 1e6}
         del m, cache
+    res["what"] = ("tp.tensor_parallel(2-layer Llama-2-7B-shaped decoder, W=2) decode step, batch 8 on 2048 cached positions, both rank "
+                   "shards on this GPU, host orchestration and the cache crop included")
+    if not model_graphs:
+        return res
     # the same step on a static cache (the count of cached positions stays on the device), recorded once as a HIP graph
     from transformers import StaticCache
 
