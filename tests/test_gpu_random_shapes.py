@@ -209,6 +209,9 @@ def test_decode_with_folded_rotary_random_shape(seed):
     dtype = [torch.bfloat16, torch.float16][pick(0, 1)]
     pos0 = [0, 1, pick(2, 200), pick(200, 3000)][pick(0, 3)]
     L = pos0 + 1 + pick(0, 9)
+    on_device = seed % 2 == 1  # every other case: the count read by the kernels, in caches with room for up to 1500 more positions
+    if on_device:
+        L = pos0 + 1 + pick(0, 1500)
     fused = torch.randn(B, 1, Hkv, per + 2, D, generator=g).to(dtype)
     kc = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
     vc = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
@@ -219,8 +222,9 @@ def test_decode_with_folded_rotary_random_shape(seed):
     want = torch.from_numpy(oat.attention_f64(q_rot.float().numpy(), want_kc[:, :, :pos0 + 1].float().numpy(),
                                               want_vc[:, :, :pos0 + 1].float().numpy(), scale, True))
     fd, kcd, vcd = fused.to(DEV), kc.to(DEV), vc.to(DEV)
-    got = _native.attention_decode_rope(fd[:, :, :, :per], fd[:, :, :, per], fd[:, :, :, per + 1], cos.to(DEV), sin.to(DEV), kcd, vcd, pos0)
+    pos = torch.tensor([pos0], dtype=torch.int64, device=DEV) if on_device else pos0
+    got = _native.attention_decode_rope(fd[:, :, :, :per], fd[:, :, :, per], fd[:, :, :, per + 1], cos.to(DEV), sin.to(DEV), kcd, vcd, pos)
     as_bits = lambda t: t.detach().cpu().contiguous().view(torch.int16)  # noqa: E731
-    tag = f"B={B} Hkv={Hkv} per={per} D={D} pos0={pos0} {dtype}"
+    tag = f"B={B} Hkv={Hkv} per={per} D={D} pos0={pos0} L={L} count on the device={on_device} {dtype}"
     assert torch.equal(as_bits(kcd), as_bits(want_kc)) and torch.equal(as_bits(vcd), as_bits(want_vc)), tag
     torch.testing.assert_close(got.double().cpu(), want, rtol=RTOL, atol=RTOL * want.std().item(), msg=lambda m: f"{tag}: {m}")
