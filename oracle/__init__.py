@@ -25,7 +25,7 @@ Modules and the reference code each one follows:
 How each function is pinned (tests/test_oracle_*.py):
   slicing      the reference's three docstring vectors (state_actions.py:40,67,94); torch.tensor_split on
                every (n, W) with n < 40, W <= 9; brute-force index enumeration on small tensors;
-               undo(split) == identity; the shapes SURVEY lists for Llama-2-7B and Falcon-40B
+               undo(split) == identity; the shard shapes of Llama-2-7B and of Falcon-40B at W = 2, 4, 8
   naming       hand-derived Llama names; golden vectors written by tests/golden/make_golden.py
   reduce       torch CPU bf16/fp16 addition (a third-party routine), W = 2 and chained W = 3..8
   forward      sum of row-parallel partials == unsplit Linear, concat of column-parallel == unsplit Linear,
