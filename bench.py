@@ -379,8 +379,34 @@ def extra_measurements(torch, _native, dev, sets, other, model_graphs: bool = Tr
         extra[f"slicing_w{world}"] = {"tensors": len(state), "shards": len(keep), "bytes_read_plus_written": moved, "us_per_launch": us,
                                       "GBps": moved / us / 1e3, "hbm_frac": moved / us / 1e3 / PEAK_HBM_GBS}
         torch.cuda.synchronize()
+        if world == 2:
+            # the way back (what TensorParallel.state_dict does per tensor): action.undo on the two rank shards of every
+            # split tensor, one launch of the region mover each, host time of the 226 calls included
+            plan.run()
+            torch.cuda.synchronize()
+            names = list(state)
+            actions = [next(a for p, a in cfg.state_rules.items() if p.search(name)) for name in names]
+
+            def unshard(i):
+                for j, action in enumerate(actions):
+                    action.undo([keep[j], keep[len(names) + j]])
+
+            us_u = _time_us(torch, unshard, 1, 3)
+            extra["unshard_w2"] = {"tensors": len(names), "bytes_read_plus_written": moved, "us_per_dict": us_u, "GBps": moved / us_u / 1e3,
+                                   "hbm_frac": moved / us_u / 1e3 / PEAK_HBM_GBS,
+                                   "what": "StateAction.undo over the W=2 shards of every split tensor of the same dict (one launch per tensor)"}
         batch.close()
         del keep, plan, batch
+    # the "gather -1" rule of the output head at BASELINE config 1: two ranks' halves of [2, 64, 50272] fp32 logits, every
+    # rank handed its own copy of the whole, one launch
+    from tensor_parallel_amd.slicing import concat_dim
+
+    halves = [torch.randn(2, 64, 25136, device=dev) for _ in range(2)]
+    us = _time_us(torch, lambda i: concat_dim(halves, -1, copies=2), 5, 30)
+    moved = float(2 * 2 * halves[0].numel() * 4 + 2 * 2 * halves[0].numel() * 4)  # both halves read for each copy, two whole copies written
+    extra["gather_c1_logits_w2"] = {"us_per_call": us, "bytes_read_plus_written": moved, "GBps": moved / us / 1e3,
+                                    "hbm_frac": moved / us / 1e3 / PEAK_HBM_GBS,
+                                    "what": "DeviceAllGather's concatenation for two ranks (2 x [2, 64, 25136] fp32 -> two copies of [2, 64, 50272]), host call included"}
     return extra
 
 
