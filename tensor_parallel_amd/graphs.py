@@ -21,7 +21,10 @@ read that count on the device, which `tp.attention.fuse_rotary_(model, assume_no
 The forwards that a capture runs beforehand (to let first uses happen outside it) advance such a cache like any other
 forward: the counts of static caches among the arguments, and the tensors named in `restore`, are put back to what
 they were before `capture` returns; what those forwards wrote behind the count is overwritten by the steps that follow.
-The tensors inside the returned value are the graph's own output buffers: the next replay overwrites them.
+The tensors inside the returned value are the graph's own output buffers: the next replay overwrites them. The recorded
+kernels also keep using the scratch buffer that the library gave the capture stream: replays of graphs, and eager work on
+a stream that torch hands out again later, are the caller's to order, as the kernels of any two launches that share
+memory are.
 """
 from __future__ import annotations
 
