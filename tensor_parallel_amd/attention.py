@@ -318,9 +318,13 @@ def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, 
     count = 0
     for module in model.modules():
         if "forward" in module.__dict__:
-            # already fused (a second call may still bring the caller's word about padding), or somebody else's forward
-            if assume_no_padding and getattr(module.__dict__["forward"], "__func__", None) is _fused_rotary_forward:
-                module.__dict__["_tp_no_padding"] = True
+            # already fused (a second call may still bring the caller's word about padding, or find the projections on the
+            # device now), or somebody else's forward
+            if getattr(module.__dict__["forward"], "__func__", None) is _fused_rotary_forward:
+                if assume_no_padding:
+                    module.__dict__["_tp_no_padding"] = True
+                if share_qkv and "_tp_qkv" not in module.__dict__:
+                    _share_qkv_storage(module)
             continue
         if _is_llama_pattern(module, class_names):
             module.forward = types.MethodType(_fused_rotary_forward, module)

@@ -227,3 +227,23 @@ def test_shared_qkv_storage_keeps_the_state_and_survives_a_replaced_projection()
         got = shared(input_ids=tok, past_key_values=caches[1], use_cache=True).logits.float()
         assert "_tp_qkv" not in attn.__dict__
         torch.testing.assert_close(got, want, rtol=5e-2, atol=5e-2 * want.std().item())  # one int8 projection in
+
+
+def test_fusing_before_wrapping_then_sharing_the_projections_afterwards():
+    """`fuse_rotary_` on the plain model (its Linears are still torch's, on the host), `tp.tensor_parallel`, then a second call:
+    the rank shards' projections now live on the device and move into one matrix."""
+    from transformers import DynamicCache
+
+    model = tiny_llama(torch.bfloat16)
+    reference = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    early = deepcopy(model)
+    assert tp.attention.fuse_rotary_(early) == 2
+    early = tp.tensor_parallel(early, [DEV, DEV])
+    attn = early.wrapped_model.module_shards[0].model.layers[1].self_attn.tp_wrapped_module
+    assert "_tp_qkv" not in attn.__dict__
+    assert tp.attention.fuse_rotary_(early) == 0 and "_tp_qkv" in attn.__dict__
+    ids = torch.randint(2, 300, (2, 16), generator=torch.Generator().manual_seed(6)).to(DEV)
+    with torch.no_grad():
+        want = reference(input_ids=ids, past_key_values=DynamicCache(), use_cache=True).logits.float()
+        got = early(input_ids=ids, past_key_values=DynamicCache(), use_cache=True).logits.float()
+    torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * want.std().item())
