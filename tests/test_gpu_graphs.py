@@ -101,3 +101,39 @@ def test_ranks_that_run_as_threads_are_refused(monkeypatch):
     monkeypatch.setattr(tp_module, "RANK_GREENLETS", False)
     with pytest.raises(RuntimeError, match="greenlets"):
         tp.graphs.capture(model, input_ids=ids, use_cache=False)
+
+
+def test_int8_shard_linears_inside_a_captured_decode_step():
+    """Rank shards with int8 weight-only Linears (their K-split kernels keep partial sums in the stream's scratch buffer) on
+    a static cache: the captured decode step against the same model run eagerly, token by token."""
+    from copy import deepcopy as dc
+
+    from transformers import LlamaConfig, LlamaForCausalLM, StaticCache
+
+    name = tp.attention.register()
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=300, hidden_size=1024, intermediate_size=2048, num_hidden_layers=2, num_attention_heads=8,
+                      num_key_value_heads=4, max_position_embeddings=256, attn_implementation="eager")
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16).eval()
+    model.config._attn_implementation = name
+    models = []
+    for _ in range(2):
+        m = tp.tensor_parallel(dc(model), [DEV, DEV])
+        tp.attention.fuse_rotary_(m, assume_no_padding=True)
+        assert tp.int8.quantize_linears_(m, skip=lambda n, mod: "lm_head" in n) == 2 * 2 * 7
+        models.append(m)
+    eager, graphed_model = models
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(2, 300, (4, 9), generator=g).to(DEV)
+    toks = [torch.randint(2, 300, (4, 1), generator=g).to(DEV) for _ in range(6)]
+    caches = [StaticCache(config=cfg, max_cache_len=64), StaticCache(config=cfg, max_cache_len=64)]
+    with torch.no_grad():
+        for m, c in zip(models, caches):
+            m(input_ids=prompt, past_key_values=c, use_cache=True)
+        step = tp.graphs.capture(graphed_model, input_ids=toks[0], past_key_values=caches[1], use_cache=True)
+        for i, tok in enumerate(toks):
+            want = eager(input_ids=tok, past_key_values=caches[0], use_cache=True).logits.float()
+            got = step(input_ids=tok, past_key_values=caches[1], use_cache=True).logits.float()
+            # the same kernels on the same inputs; only torch's attention-mask handling differs under capture, and the
+            # fused attention ignores the mask
+            torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2 * want.std().item(), msg=lambda m: f"step {i}: {m}")
