@@ -1388,8 +1388,16 @@ inline bool pick_resident(const SkinnyParams &p, int cus) {
         if (p.K <= 6144) return tiles * 2 >= cus;
         return p.M >= 8 && tiles < cus;
     }
-    if (p.K <= 6144) return p.M >= 12 && tiles * 2 >= 3ll * cus;
-    return (tiles >= cus && tiles * 2 < 3ll * cus) || (p.M >= 10 && tiles >= cus && tiles * 2 <= 5ll * cus);
+    // A sweep of 240 shapes (N from 2048 to 16384, K from 2048 to 8192, 4 to 16 rows, in a HIP graph) put the rules below
+    // within 2 % of the better kernel on all but a handful. Between one and two tiles per CU the plain kernel's blocks fill
+    // the CUs unevenly and the persistent x-resident blocks win at every row count (4608 / 5120 / 6144 x 4096 ... 6144:
+    // 8-37 %); at exactly one tile per CU the plain kernel does (4096 x 8192: 10-15 %); two to three tiles per CU at
+    // K = 8192 go to the resident kernel from 10 rows on (11008 / 12288 x 8192 at 12-16 rows: 47 -> 34 us).
+    // Fewer tiles than CUs and long rows (K >= 5504) from 12 rows on: resident by 5-20 % (2048 / 3072 x 5504 ... 8192).
+    const bool between_one_and_two = tiles > cus && tiles < 2ll * cus;
+    const bool few_long = tiles < cus && p.K >= 5504 && p.M >= 12;
+    if (p.K <= 6144) return few_long || (between_one_and_two && (p.K >= 4096 || p.M >= 12)) || (p.M >= 12 && tiles * 2 >= 3ll * cus);
+    return few_long || (tiles > cus && tiles * 2 <= 3ll * cus) || (p.M >= 10 && tiles > cus && tiles <= 3ll * cus);
 }
 
 template <int DT, int MODE>
