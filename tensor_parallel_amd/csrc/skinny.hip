@@ -1385,8 +1385,15 @@ inline bool pick_resident(const SkinnyParams &p, int cus) {
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
     if (p.M < 3 || p.K < 3072) return false;
     if (MODE == SK_SWIGLU) {
-        if (p.K <= 6144) return tiles * 2 >= cus;
-        return p.M >= 8 && tiles < cus;
+        // Refitted on a sweep of 220 pair shapes (N from 1376 to 14336, K from 2048 to 8192, 4 to 16 rows, in a HIP graph,
+        // plain 8-column kernel | this one | x staged in LDS). Whole rounds of one tile per CU suit the plain kernel, whose
+        // blocks then fill the CUs evenly (2048 x 3072 ... 8192: 4-36 %; 4096 and 8192 x 8192: 16-41 %); otherwise this
+        // kernel is the fastest from K = 3072 on, except on few tiles at K = 3072 and, at K = 8192, few tiles below 8 rows
+        // and more than four tiles per CU up to 8 rows.
+        if (tiles == cus) return false;
+        if (p.K <= 6144) return tiles * 2 >= cus && !(p.K < 4096 && tiles < cus);
+        if ((tiles % cus == 0 && tiles <= 4ll * cus) || (tiles > 4ll * cus && tiles < 7ll * cus && p.M <= 8)) return false;
+        return tiles > cus || p.M >= 8;
     }
     // A sweep of 240 shapes (N from 2048 to 16384, K from 2048 to 8192, 4 to 16 rows, in a HIP graph) put the rules below
     // within 2 % of the better kernel on all but a handful. Between one and two tiles per CU the plain kernel's blocks fill
@@ -1706,6 +1713,10 @@ int launch_pair_xlds(const SkinnyParams &p, int cus, hipStream_t s, bool *done) 
         const int units = (p.K + XL_UNIT_K - 1) / XL_UNIT_K, padded = (units + XL_CH - 1) / XL_CH * XL_CH;
         if (padded * 100 > units * 107) return TPAMD_OK;
         if (tiles < cus && p.M < 12) return TPAMD_OK;
+        // The later sweep of 220 pair shapes: this kernel is the fastest of the three only for short rows (K below 3072)
+        // on more than two tiles per CU (5504 ... 14336 x 2048: 2-8 %); where the x-resident kernel declines a longer K
+        // the plain kernel is the better second choice (K = 8192: by 8-41 %).
+        if (p.K >= 3072 || tiles <= 2ll * cus) return TPAMD_OK;
     }
     static thread_local int configured_dev = -1;  // per instantiation and host thread
     int dev = 0;
