@@ -48,7 +48,7 @@ struct Tuning {
     int w8_cols;             // TPAMD_W8_COLS: int8 K-split kernel whose wavefronts own columns (x of the split in LDS): 0 = off, 1 = whenever the shape allows
     int skinny_max_m;        // TPAMD_SKINNY_MAX_M: most rows of a single 16-bit matrix that go to the weight-streaming kernels (16 to 64; unset: by shape)
     int skinny_xlds;         // TPAMD_SKINNY_XLDS: 0 = gated pair at 4-16 rows through the older kernels
-    int gemv_rows;           // TPAMD_GEMV_ROWS: wavefronts per block of the unrolled M <= 3 kernel (2, 4, 8, 16); 0 = the general kernel
+    int gemv_rows;           // TPAMD_GEMV_ROWS: wavefronts per block of the unrolled M <= 3 kernel (4, 8, 16); 0 = the general kernel, -1 = the MFMA kernels
     int attn_splits;         // TPAMD_ATTN_SPLITS: key-range splits of the attention kernel
     int attn_ring;           // TPAMD_ATTN_RING: 1 / 0 = the few-row attention kernel with / without several K / V tiles in flight
     int copy_tile_units;     // TPAMD_COPY_TILE_UNITS: 16-byte units per copy tile

@@ -1317,21 +1317,56 @@ void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
 #undef TPAMD_ROWS_M
 }
 
+// Which kernel takes M <= 3 rows of 16-bit weights. Fitted on a sweep of 342 shapes (single matrix and gated pair, M = 1..3,
+// N = 1376..32000, K = 2048..8192, each timed inside a HIP graph on weights that rotate through more memory than the
+// caches hold): sum over the sweep 7197 us with the rules before, 6986 us with these, 6948 us with the best kernel per shape.
+//  - a block of W wavefronts owns W output columns (W column pairs of a gated pair) and a CU's share of HBM bandwidth
+//    is what bounds it, so what counts is the most columns any CU gets: ceil(ceil(N / W) / CUs) * W. 16 wavefronts
+//    win when that is no worse than with 8 (N = 5504: 32 against 24 on 256 CUs, 13 % slower) and rows are long enough
+//    to pay for the larger block; 4 wavefronts win on small N where they balance better (N = 2752: 12 against 16);
+//  - 2 rows of long rows (K > 6144 single, K >= 5120 gated pair) on large N go to the MFMA kernels like 3 rows do
+//    (single 8192 x 8192: 24.2 us there, 26.3 us here; pair 5504 x 8192: 29.7 against 33.1 us);
+//  - gated pairs with 2 rows, 8192 columns or more and K around 4096 go to the general kernel (11008 x 4096: 28.1 against 29.0 us).
+enum RowsPath { ROWS_W4, ROWS_W8, ROWS_W16, ROWS_GENERAL, ROWS_MFMA };
+inline RowsPath pick_rows_path(bool pair, int64_t M, int64_t N, int64_t K, int cus) {
+    if (M == 3 && K >= 3072 && K <= 8192) return ROWS_MFMA;
+    auto most_cols = [&](int64_t w) { return ((N + w - 1) / w + cus - 1) / cus * w; };
+    const bool bal16 = most_cols(16) <= most_cols(8) && N >= 2752;
+    const bool bal4 = most_cols(4) < most_cols(8) && N < 4096;
+    if (!pair) {
+        if (M == 2 && K > 6144) return N >= 4096 && bal16 ? ROWS_MFMA : bal4 ? ROWS_W4 : ROWS_W8;
+        if (M == 3) return ROWS_W8;
+        return bal16 && K >= (M == 2 ? 3584 : 3072) ? ROWS_W16 : ROWS_W8;
+    }
+    const bool near_4096 = K >= 3584 && K <= 4608;
+    if (M == 1) {
+        if (near_4096 && bal16) return ROWS_W16;
+        return bal4 || (K > 6144 && N >= 2752 && N <= 11008) ? ROWS_W4 : ROWS_W8;
+    }
+    if (M == 2) {
+        if (K >= 5120 && N >= 4096) return ROWS_MFMA;
+        if (K >= 3584 && N >= 8192) return ROWS_GENERAL;
+        if (near_4096 && bal16) return ROWS_W16;
+        return bal4 ? ROWS_W4 : ROWS_W8;
+    }
+    return ROWS_W8;
+}
+
 // M <= 3 and at most 16 pieces per row: K <= 8192 for 16-bit weights, K <= 16384 (and at most 128 outlier columns) for
-// int8. *done = false: not taken.
+// int8. `path`: what pick_rows_path chose (int8: ROWS_W8). *done = false: not taken.
 template <int DT, bool W8, int MODE>
-int launch_gemv_rows(const SkinnyParams &p, hipStream_t s, bool *done) {
+int launch_gemv_rows(const SkinnyParams &p, hipStream_t s, RowsPath path, bool *done) {
     *done = false;
     const int knob = tuning().gemv_rows;  // wavefronts per block; 0 = the general kernel
     const int piece_k = W8 ? 1024 : 512;
-    if (knob == 0 || p.K > 16 * piece_k || p.K % (W8 ? 16 : 8) != 0 || (W8 && p.n_out > 128)) return TPAMD_OK;
+    if (knob == 0 || (knob == TUNE_UNSET && path == ROWS_GENERAL)) return TPAMD_OK;
+    if (p.K > 16 * piece_k || p.K % (W8 ? 16 : 8) != 0 || (W8 && p.n_out > 128)) return TPAMD_OK;
     // int8 with 2 or 3 rows of x: every further row costs as much again in LDS reads (32 bytes of x per 16 weights), and
     // the general kernel's staggered blocks hide that better (Falcon-40B MLP shard, 2 rows: 66 us against 83 us here)
     if (W8 && p.M > 1) return TPAMD_OK;
-    // measured on the Llama-7B shard at M = 1 (inside a HIP graph): single matrix 4096 x 5504 with 16 / 8 / 4 wavefronts
-    // per block 8.7 / 9.1 / 9.5 us, gated pair 2 x 5504 x 4096 16.8 / 15.1 / 15.6 us; int8 16384 x 8192 + 8192 x 16384:
-    // 51.6 / 48.0 / 50.4 us (the general kernel: 58.8 us)
-    const int waves = knob != TUNE_UNSET ? knob : (!W8 && MODE == SK_LINEAR && p.N >= 4096) ? 16 : 8;
+    // int8, M = 1, 16384 x 8192 + 8192 x 16384 with 16 / 8 / 4 wavefronts per block: 51.6 / 48.0 / 50.4 us (the general
+    // kernel: 58.8 us)
+    const int waves = knob != TUNE_UNSET ? knob : path == ROWS_W16 ? 16 : path == ROWS_W4 ? 4 : 8;
     const int np = (p.K + piece_k - 1) / piece_k;
 #define TPAMD_ROWS_CASE(W) \
     if (np <= 4) launch_gemv_rows_m<DT, W8, MODE, W, 4>(p, s); else if (np <= 8) launch_gemv_rows_m<DT, W8, MODE, W, 8>(p, s); \
@@ -1831,23 +1866,31 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
     p.ldx = ldx; p.ldw = ldw; p.ldy = ldy; p.ld_wout = ld_wout;
     p.act = act;
     const bool bf = dtype == TPAMD_BF16;
-    // 3 rows of a large matrix are faster through the MFMA kernels (Llama-7B MLP shard step: 36.4 us here, 28.3 us there,
-    // as at 4 rows), and so are 2 and 3 rows of int8 weights through the K-split kernel where it applies
+    // 2 and 3 rows of int8 weights are faster through the K-split kernel where it applies
     if (w8 && M >= 2 && M <= GEMV_MAX_M) {
         bool done = false;
         const int rc = bf ? launch_w8_cols<TPAMD_BF16>(p, s, &done) : launch_w8_cols<TPAMD_F16>(p, s, &done);
         if (rc != TPAMD_OK || done) return rc;
     }
-    const bool rows3_to_mfma = !w8 && M == 3 && K >= 3072 && K <= 8192;
-    if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES && !rows3_to_mfma) {
-        bool done = false;
-        const int rc = w8 ? (bf ? launch_gemv_rows<TPAMD_BF16, true, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, true, SK_LINEAR>(p, s, &done))
-                     : swiglu ? (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_SWIGLU>(p, s, &done) : launch_gemv_rows<TPAMD_F16, false, SK_SWIGLU>(p, s, &done))
-                              : (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_LINEAR>(p, s, &done) : launch_gemv_rows<TPAMD_F16, false, SK_LINEAR>(p, s, &done));
-        if (rc != TPAMD_OK || done) return rc;
-        if (w8) return bf ? launch_gemv<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, true, SK_LINEAR>(p, s);
-        if (swiglu) return bf ? launch_gemv<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_gemv<TPAMD_F16, false, SK_SWIGLU>(p, s);
-        return bf ? launch_gemv<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, false, SK_LINEAR>(p, s);
+    if (M <= GEMV_MAX_M && M * K * 2 <= GEMV_MAX_X_BYTES) {
+        RowsPath path = ROWS_W8;
+        if (!w8) {
+            int dev = 0, cus = 256;
+            TPAMD_HIP(hipGetDevice(&dev));
+            if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+            const int knob = tuning().gemv_rows;  // -1: the MFMA kernels; other values: launch_gemv_rows
+            path = knob == -1 ? ROWS_MFMA : knob != TUNE_UNSET && !(M == 3 && K >= 3072 && K <= 8192) ? ROWS_W8 : pick_rows_path(swiglu, M, N, K, cus);
+        }
+        if (path != ROWS_MFMA) {
+            bool done = false;
+            const int rc = w8 ? (bf ? launch_gemv_rows<TPAMD_BF16, true, SK_LINEAR>(p, s, path, &done) : launch_gemv_rows<TPAMD_F16, true, SK_LINEAR>(p, s, path, &done))
+                         : swiglu ? (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_SWIGLU>(p, s, path, &done) : launch_gemv_rows<TPAMD_F16, false, SK_SWIGLU>(p, s, path, &done))
+                                  : (bf ? launch_gemv_rows<TPAMD_BF16, false, SK_LINEAR>(p, s, path, &done) : launch_gemv_rows<TPAMD_F16, false, SK_LINEAR>(p, s, path, &done));
+            if (rc != TPAMD_OK || done) return rc;
+            if (w8) return bf ? launch_gemv<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, true, SK_LINEAR>(p, s);
+            if (swiglu) return bf ? launch_gemv<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_gemv<TPAMD_F16, false, SK_SWIGLU>(p, s);
+            return bf ? launch_gemv<TPAMD_BF16, false, SK_LINEAR>(p, s) : launch_gemv<TPAMD_F16, false, SK_LINEAR>(p, s);
+        }
     }
     if (w8) return bf ? launch_skinny<TPAMD_BF16, true, SK_LINEAR>(p, s) : launch_skinny<TPAMD_F16, true, SK_LINEAR>(p, s);
     if (swiglu) return bf ? launch_skinny<TPAMD_BF16, false, SK_SWIGLU>(p, s) : launch_skinny<TPAMD_F16, false, SK_SWIGLU>(p, s);

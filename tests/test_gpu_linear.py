@@ -474,10 +474,11 @@ def test_other_dispatch_paths_inside_a_hip_graph(case, tune):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [1, 2, 3])
-@pytest.mark.parametrize("N,K", [(2048, 512), (2053, 520), (4100, 5504), (6000, 1032), (3000, 8192)])
+@pytest.mark.parametrize("N,K", [(2048, 512), (2053, 520), (4100, 5504), (6000, 1032), (3000, 8192), (4096, 4096), (8192, 6656), (8200, 4096)])
 def test_row_streaming_kernel_on_wide_matrices(dtype, M, N, K):
     """M <= 3 and thousands of output columns (ragged column count, ragged last K step): against the fp32 host
-    product, the gated pair against the oracle, the fused sum bit for bit."""
+    product, the gated pair against the oracle, the fused sum bit for bit. The shapes reach every choice of the rule
+    for these row counts: blocks of 4, 8 and 16 wavefronts, the general row kernel, the MFMA kernels at 2 rows."""
     x, w, w2, b = rnd((M, K), 1, 1.0, dtype).to(DEV), rnd((N, K), 0, 0.02, dtype).to(DEV), rnd((N, K), 5, 0.02, dtype).to(DEV), rnd((N,), 2, 0.1, dtype).to(DEV)
     lin = _native.linear(x, w, b)
     check_half(lin, F.linear(x.float().cpu(), w.float().cpu(), b.float().cpu()), K)
