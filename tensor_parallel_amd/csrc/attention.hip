@@ -607,26 +607,34 @@ int launch(AttnParams p, int cus, hipStream_t s) {
     const int block_rows = wide ? 128 : 64;
     const int row_tiles = (nrows + block_rows - 1) / block_rows;
     const int64_t blocks = static_cast<int64_t>(row_tiles) * p.B * p.Hkv;
-    // Split the keys when the rows alone leave CUs idle and there are enough keys to share out. Where every CU can get a
-    // block with a long key range (RING_MIN_TILES tiles or more), one block per CU and the ring kernel streams them
-    // (batch 8 on 8192 keys: 20.0 us); otherwise two blocks per CU with at least 128 keys each, for the kernel with one
-    // tile in flight per block (that shape: 23.4 us; batch 8 on 2048 keys: 9.4 us against 11.4 us for 4 ring blocks
-    // of 8 tiles per head).
+    // Split the keys when the rows alone leave CUs idle. Fitted on a sweep of 144 decode shapes (D = 64 / 128, 1-1024
+    // blocks, 512-32768 keys) and 32 shapes with several positions per sequence (short causal prefills, 8-256 new
+    // positions on 2048-8192 cached keys), each with 1-64 splits, with and without the ring kernel, inside a HIP graph
+    // on caches that rotate through more memory than the chip caches: within 1 % of the best choice per decode shape
+    // in the geometric mean (the rules before: 5 %, up to 31 % on 8192 keys with few heads).
+    //  - as many splits as give every CU a block, or two where blocks are light (D = 64 from 32 blocks on) or full
+    //    (64 rows: the MFMA work of one block no longer hides another's loads);
+    //  - but every split costs a partial to write and merge, every key a fixed time: the sum is least near
+    //    sqrt(keys / 8) splits (512 keys: 8, 8192: 32, 32768: 64), which caps the count where heads are few; blocks of
+    //    64 rows write 4-64 times the partials of a decode block: half as many splits, and 256 keys or more in each
+    //    (a causal prefill of 512 positions on 16 heads: 8.9 us unsplit, 13.3 us in four);
+    //  - with a block for every other CU, 512 keys are not worth a second launch (D = 64, 128 blocks: 8.5 us against
+    //    9.1 us), and with one for every CU splitting pays only on long caches (D = 64, 256 blocks, 32768 keys: 431 us
+    //    unsplit, 366 us in two).
+    // The ring kernel (several tiles in flight per block) never beat the best split count of the plain kernel by more
+    // than 1 % in these sweeps and stays behind TPAMD_ATTN_RING.
     int nsplit = 1;
     bool ring = false;
-    if (blocks < 2 * cus) {
-        const int by_cu = blocks < cus ? static_cast<int>(cus / blocks) : 1;
-        const int by_keys = p.Skv / (RING_MIN_TILES * AT_KEYS);
-        if (by_keys >= by_cu) {
-            ring = true;
-            nsplit = by_cu;
-        } else {
-            nsplit = static_cast<int>((2 * cus + blocks - 1) / blocks);
-            const int max_by_keys = (p.Skv + 127) / 128;
-            if (nsplit > max_by_keys) nsplit = max_by_keys;
-            if (nsplit < 1) nsplit = 1;
-        }
+    const bool full_rows = nrows >= 64;
+    const int per_cu = (D <= 64 && blocks >= 32) || full_rows ? 2 : 1;
+    const int64_t keys_seen = p.causal && p.Sq > 1 ? p.Skv - (p.Sq < p.Skv ? p.Sq : p.Skv) / 2 : p.Skv;  // what a row sees on average
+    if (blocks < static_cast<int64_t>(per_cu) * cus && !(blocks >= cus && keys_seen < 8192) && !(blocks * 2 >= cus && keys_seen <= 512)) {
+        nsplit = static_cast<int>((static_cast<int64_t>(per_cu) * cus + blocks - 1) / blocks);
+        int by_keys = static_cast<int>(lroundf(sqrtf(static_cast<float>(keys_seen) / 8.f)));
+        if (full_rows) by_keys = by_keys / 2 < keys_seen / 256 ? by_keys / 2 : static_cast<int>(keys_seen / 256);
+        if (nsplit > by_keys) nsplit = by_keys;
         if (nsplit > 64) nsplit = 64;
+        if (nsplit < 1) nsplit = 1;
     }
     if (tuning().attn_splits != TUNE_UNSET) {
         nsplit = tuning().attn_splits > 0 ? tuning().attn_splits : 1;
