@@ -683,7 +683,54 @@ def llama_layer_decode(torch, dev, model_graphs: bool = True) -> dict:
     res["what"] = ("tp.tensor_parallel(2-layer Llama-2-7B-shaped decoder, W=2) decode step, batch 8 on 2048 cached positions, both rank "
                    "shards on this GPU, host orchestration and the cache crop included; the last entry: transformers' StaticCache, "
                    "fuse_rotary_(assume_no_padding=True), the whole step replayed as one HIP graph (tp.graphs.capture)")
+    res["generate"] = llama_generate(torch, dev, cfg, model, prompt)
     return res
+
+
+def llama_generate(torch, dev, cfg, decoder, prompt) -> dict:
+    """`generate` of the same decoder under a language-model head (greedy, batch 8, 2048 prompt positions): time per new token
+    = (a call for 33 new tokens - a call for 1) / 32, so the prefill and the set-up of a call drop out. Three ways: the
+    wrapped modules' own forward on a growing cache; fuse_rotary_ on a growing cache; fuse_rotary_(assume_no_padding=True) with
+    cache_implementation="static", where the wrapper records the decode step as a HIP graph at its first use in a call
+    (the recording is inside the timed call) and replays it for every further token."""
+    import time
+    from copy import deepcopy
+
+    from transformers import LlamaForCausalLM
+
+    import tensor_parallel_amd as tp
+
+    with torch.device(dev):
+        lm = LlamaForCausalLM(cfg).to(torch.bfloat16).eval()
+    lm.model.load_state_dict(decoder.state_dict())
+    lm.lm_head.weight.data.normal_(0.0, 0.02)
+    lm.config._attn_implementation = decoder.config._attn_implementation
+    lm.generation_config.pad_token_id = 0
+    out = {}
+    for label in ("own_forward", "fuse_rotary", "fuse_rotary_static_cache_graph"):
+        m = tp.tensor_parallel(deepcopy(lm), [dev, dev])
+        kwargs = {}
+        if label == "fuse_rotary":
+            tp.attention.fuse_rotary_(m)
+        elif label != "own_forward":
+            tp.attention.fuse_rotary_(m, assume_no_padding=True)
+            kwargs["cache_implementation"] = "static"
+
+        def run(n):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            m.generate(prompt, max_new_tokens=n, min_new_tokens=n, do_sample=False, **kwargs)
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0
+
+        run(3)  # first uses
+        one = min(run(1) for _ in range(2))
+        many = min(run(33) for _ in range(2))
+        ms = (many - one) / 32 * 1e3
+        out[label] = {"ms_per_new_token_step": ms, "tokens_per_s": prompt.shape[0] / ms * 1e3}
+        del m
+    out["what"] = "tp.tensor_parallel(LlamaForCausalLM over the same 2 layers, W=2).generate, greedy, batch 8 on a 2048-token prompt, (33 new tokens - 1 new token) / 32"
+    return out
 
 
 def reduce_extra(torch, _native, dev, other) -> dict:

@@ -295,6 +295,23 @@ def _is_rotary_falcon(module: torch.nn.Module) -> bool:
     return getattr(config, "alibi", True) is False and module.new_decoder_architecture and getattr(module, "layer_idx", None) is not None
 
 
+def decode_step_is_static(model: torch.nn.Module) -> bool:
+    """True when every attention module under `model` has the fused forward in the form that reads a static cache's
+    count of cached positions on the device (`fuse_rotary_(model, assume_no_padding=True)`): a decode step then takes no
+    host decision that depends on the step, which is what recording it as a HIP graph needs."""
+    fused = 0
+    for module in model.modules():
+        func = getattr(module.__dict__.get("forward"), "__func__", None)
+        if func is _fused_falcon_forward:
+            fused += 1
+        elif func is _fused_rotary_forward:
+            if not module.__dict__.get("_tp_no_padding", False):
+                return False
+            fused += 1
+    layers = getattr(getattr(model, "config", None), "num_hidden_layers", None)
+    return fused > 0 and (layers is None or fused >= layers)
+
+
 def fuse_rotary_(model: torch.nn.Module, class_names=FUSABLE_ATTENTION_CLASSES, assume_no_padding: bool = False,
                  share_qkv: bool = True) -> int:
     """Give every attention module under `model` (before or after `tp.tensor_parallel`) whose class is named in

@@ -3,12 +3,14 @@ rank shards (reference: src/tensor_parallel/pretrained_model.py:21-165). The att
 (see kv_cache): there is no cache reordering hook here, the cache objects reorder themselves."""
 from __future__ import annotations
 
+import importlib
 import logging
 from typing import Optional, Sequence
 
 import torch
 from transformers import GenerationMixin, PretrainedConfig, PreTrainedModel
 
+from . import attention, graphs
 from .config import Config
 from .slicing_configs import PREDEFINED_CONFIGS
 from .tensor_parallel import TensorParallel, check_device_ids, parallel_apply_simple
@@ -106,9 +108,47 @@ class TensorParallelPreTrainedModel(PreTrainedModel, GenerationMixin):
 
     def _valid_auto_compile_criteria(self, model_kwargs, generation_config) -> bool:
         # `generate` wraps the forward in torch.compile when it is given a static cache. The rank shards call a C ABI
-        # through ctypes and take turns as greenlets, which a tracing compiler cannot follow: the forward stays as it is
-        # (`tp.graphs.capture` is this package's way to take the host out of a decode step).
-        return False
+        # through ctypes and take turns as greenlets, which a tracing compiler cannot follow. What takes its place: the
+        # decode step recorded as one HIP graph (get_compiled_call below), where a step can be recorded at all, i.e. where
+        # every attention module reads the count of cached positions on the device
+        # (`tp.attention.fuse_rotary_(model, assume_no_padding=True)`); the forward as it is otherwise.
+        if generation_config.disable_compile:
+            return False
+        cache = model_kwargs.get("past_key_values")
+        layers = getattr(cache, "layers", None)
+        if not isinstance(layers, list) or not layers or not all(hasattr(layer, "cumulative_length") for layer in layers):
+            return False
+        return self._decode_step_can_be_recorded()
+
+    def _decode_step_can_be_recorded(self) -> bool:
+        tp_module = importlib.import_module(__package__ + ".tensor_parallel")
+        shards = self.wrapped_model.module_shards
+        if len(shards) > 1 and not tp_module.RANK_GREENLETS:
+            return False
+        if any(device.type != "cuda" for device in self.wrapped_model.devices) or len(set(self.wrapped_model.devices)) != 1:
+            return False
+        return all(attention.decode_step_is_static(shard) for shard in shards)
+
+    def get_compiled_call(self, compile_config=None):
+        """What `generate` calls for every decode step once `_valid_auto_compile_criteria` has said yes: the step recorded
+        as one HIP graph by `tp.graphs.capture` at its first call and replayed afterwards. The padding mask is left out
+        of the recorded arguments (it grows by a column per step, and the fused attention was promised that there is no
+        padding). One graph is kept: a step on another cache object, or with other shapes, records a new one; the graph
+        holds its cache alive until then. `generate(..., disable_compile=True)` keeps the forward as it is."""
+        return self._recorded_decode_step
+
+    def _recorded_decode_step(self, **model_inputs):
+        model_inputs.pop("attention_mask", None)
+        model_inputs = {k: v for k, v in model_inputs.items() if v is not None}
+        graphed = self.__dict__.get("_tp_decode_graph")
+        if graphed is not None:
+            try:
+                return graphed(**model_inputs)
+            except ValueError:  # another cache object, batch size or set of arguments: record again
+                self.__dict__["_tp_decode_graph"] = graphed = None
+        graphed = graphs.capture(self, **model_inputs)
+        self.__dict__["_tp_decode_graph"] = graphed
+        return graphed(**model_inputs)
 
     def get_encoder(self, *args, **kwargs):
         shards = self.wrapped_model.module_shards

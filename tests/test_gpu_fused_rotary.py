@@ -186,16 +186,41 @@ def test_static_cache_decode_eager_and_as_one_graph():
 
 
 def test_generate_on_a_static_cache():
-    """`generate(cache_implementation="static")`: transformers would hand the forward to torch.compile for such a cache; the
-    wrapper declines that, and the tokens are those of the growing cache."""
+    """`generate(cache_implementation="static")`: transformers would hand the forward to torch.compile for such a cache. The
+    wrapper records the decode step as one HIP graph instead, when every attention module reads the cache's count on the
+    device, and declines otherwise; either way the tokens are those of the growing cache."""
     model = tiny_llama(torch.bfloat16)
     plain = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
     fused = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
     tp.attention.fuse_rotary_(fused, assume_no_padding=True)
-    ids = torch.randint(2, 300, (2, 12), generator=torch.Generator().manual_seed(0)).to(DEV)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(2, 300, (2, 12), generator=g).to(DEV)
     want = plain.generate(ids, max_new_tokens=8, do_sample=False)
+    eager = fused.generate(ids, max_new_tokens=8, do_sample=False, cache_implementation="static", disable_compile=True)
+    assert torch.equal(eager, want) and "_tp_decode_graph" not in fused.__dict__
     got = fused.generate(ids, max_new_tokens=8, do_sample=False, cache_implementation="static")
     assert torch.equal(got, want)
+    # transformers builds a new cache for every such call, and a step on another cache is recorded anew; a cache of the
+    # caller's that is reset between calls keeps its recording
+    from transformers import StaticCache
+
+    cache = StaticCache(config=model.config, max_cache_len=32)
+    assert torch.equal(fused.generate(ids, max_new_tokens=8, do_sample=False, past_key_values=cache), want)
+    first = fused.__dict__["_tp_decode_graph"]
+    cache.reset()
+    other = torch.randint(2, 300, (2, 12), generator=g).to(DEV)
+    assert torch.equal(fused.generate(other, max_new_tokens=8, do_sample=False, past_key_values=cache), plain.generate(other, max_new_tokens=8, do_sample=False))
+    assert fused.__dict__["_tp_decode_graph"] is first
+    # another batch size: a new cache, a new recording
+    ids3 = torch.randint(2, 300, (3, 9), generator=g).to(DEV)
+    want3 = plain.generate(ids3, max_new_tokens=6, do_sample=False)
+    assert torch.equal(fused.generate(ids3, max_new_tokens=6, do_sample=False, cache_implementation="static"), want3)
+    assert fused.__dict__["_tp_decode_graph"] is not first
+    # modules that were fused without the caller's word about padding take no static cache step as a graph
+    halfway = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
+    tp.attention.fuse_rotary_(halfway)
+    assert not halfway._decode_step_can_be_recorded() and not plain._decode_step_can_be_recorded()
+    assert fused._decode_step_can_be_recorded()
 
 
 def test_shared_qkv_storage_keeps_the_state_and_survives_a_replaced_projection():
