@@ -143,6 +143,13 @@ def test_fused_rotary_falcon_inside_tensor_parallel():
             want = plain(input_ids=tok, past_key_values=growing, use_cache=True).logits.float()
             torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * scale, msg=lambda m: f"replayed step {i}: {m}")
     assert int(static.get_seq_length()) == 74 and static.layers[0].keys.shape == (2, 2, 96, 64)
+    # ... and through generate, which records the step by itself on a static cache (greedy tokens of a random model can
+    # flip between two orders of summation, so the first tokens are compared, and the recorded run with the eager one)
+    short = ids[:, :20]
+    eager = fused.generate(short, max_new_tokens=6, do_sample=False, cache_implementation="static", disable_compile=True)
+    got = fused.generate(short, max_new_tokens=6, do_sample=False, cache_implementation="static")
+    assert "_tp_decode_graph" in fused.__dict__ and torch.equal(got, eager)
+    assert torch.equal(got[:, :21], plain.generate(short, max_new_tokens=1, do_sample=False))
 
 
 def test_static_cache_decode_eager_and_as_one_graph():
