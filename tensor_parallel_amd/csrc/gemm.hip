@@ -936,8 +936,15 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
 //   S2 (k 32..63)  reads the fragments of k 0..31 of tile kt+1; loads: first half of tile kt + NS into the freed stage
 // SPLIT: the block covers K tiles [blockIdx.y * kt_per_split, ...) and leaves its fp32 partial tile in p.ws for
 // splitk_finish_kernel.
-template <int DT, int MODE, int NS, bool SPLIT>
+// XQ < 4 (SPLIT, single matrix, M <= 32 * XQ): only the first XQ quarters of the x tile exist. The loads of the others
+// are left out, and the two wavefronts that own x rows 64-127 only load: they read no fragments and multiply nothing,
+// so LDS serves the other two and the incoming tiles alone. Measured at 17-64 rows inside a HIP graph: 4096 x 5504
+// 17.3-19.2 -> 15.5-17.8 us, 4096 x 4096 14.2-15.6 -> 12.8-14.5 us, 8192 x 8192 29.0-33.0 -> 27.8-32.0 us, no difference from
+// 11008 columns on (whole tiles there); leaving out the loads alone gives 1-2 %. The gated pair is 1-5 % slower this way (its wavefronts
+// have half as many columns each) and keeps whole tiles.
+template <int DT, int MODE, int NS, bool SPLIT, int XQ = 4>
 __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
+    static_assert(XQ == 4 || (SPLIT && NS == 2 && MODE == MODE_LINEAR && (XQ == 1 || XQ == 2)), "part tiles of x: split kernel, single matrix");
     constexpr int BM = 128, BN = 128, WAVES_N = 2, NW = 4;
     constexpr int BLK = 1152;
     constexpr int XREG = (BM / 8) * BLK, WREG = (BN / 8) * BLK, STAGE = XREG + WREG;
@@ -993,6 +1000,7 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
     // loads of local tile j (clamped to the last one: such loads refill a stage nobody reads any more and keep
     // the loop free of branches)
     auto gx = [&](int i, int j) {
+        if (i >= XQ) return;  // i is a constant at every call
         const int jj = j < last ? j : last;
         buffer_load16_to_lds(x_rsrc, x_off[i], static_cast<uint32_t>(kt0 + jj) * (BK * 2), smem + (j & (NS - 1)) * STAGE + (wave_s + i * NW) * BLK);
     };
@@ -1071,6 +1079,18 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
         for (int i = 0; i < 4; ++i) gw(i, j);
     }
     TPAMD_TILE_BARRIER();
+    if (XQ < 4 && wave_s >= WAVES_N) {
+        // x rows 64-127 do not exist: this wavefront keeps its share of the loads going, in the places the others have
+        // them, and meets them at every barrier
+        gx(0, NS - 1); gx(1, NS - 1);
+        for (int j = 0; j < last; ++j) {
+            gw(0, j + NS - 1); gw(1, j + NS - 1); gw(2, j + NS - 1); gw(3, j + NS - 1);
+            TPAMD_TILE_BARRIER();
+            gx(0, j + NS); gx(1, j + NS);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing on its way into LDS when the block ends
+        return;
+    }
     {
         const uint32_t xa = smem_base + x_rd0 + kk_off[0];
         const uint32_t wa = smem_base + w_rd0 + kk_off[0];
@@ -1807,11 +1827,11 @@ int launch_direct(GemmParams p, int cus, int splits, hipStream_t s) {
 
 }  // namespace
 
-template <int DT, int MODE, int NS, bool SPLIT>
+template <int DT, int MODE, int NS, bool SPLIT, int XQ = 4>
 int configure128(int dev) {
     static thread_local int configured_dev = -1;
     if (configured_dev != dev) {
-        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct128_kernel<DT, MODE, NS, SPLIT>),
+        TPAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_direct128_kernel<DT, MODE, NS, SPLIT, XQ>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, NS * 32 * 1152));
         configured_dev = dev;
     }
@@ -1860,7 +1880,12 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     splits = (KT + p.kt_per_split - 1) / p.kt_per_split;   // no empty split
     constexpr int LDS2 = 2 * 32 * 1152;
     if (splits > 1) {
+        const int xq = MODE != MODE_LINEAR || tuning().gemm_part_x == 0 || tiles > 64 ? 4 : p.M <= 32 ? 1 : p.M <= 64 ? 2 : 4;  // tiles > 64: measured, no gain
         int rc = configure128<DT, MODE, 2, true>(dev);
+        if constexpr (MODE == MODE_LINEAR) {
+            if (xq == 1) rc = configure128<DT, MODE, 2, true, 1>(dev);
+            else if (xq == 2) rc = configure128<DT, MODE, 2, true, 2>(dev);
+        }
         if (rc != TPAMD_OK) return rc;
         const size_t ws_bytes = static_cast<size_t>(splits) * tiles * 128 * 128 * sizeof(float);
         // the scratch buffer is ours until both launches are enqueued
@@ -1870,7 +1895,14 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
         if (rc != TPAMD_OK) return rc;
         if (ws != nullptr) {
             p.ws = static_cast<float *>(ws);
-            hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true>), dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(splits)), dim3(256), LDS2, s, p);
+            const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits));
+            bool launched = false;
+            if constexpr (MODE == MODE_LINEAR) {
+                if (xq == 1) hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true, 1>), grid, dim3(256), LDS2, s, p);
+                else if (xq == 2) hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true, 2>), grid, dim3(256), LDS2, s, p);
+                launched = xq != 4;
+            }
+            if (!launched) hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true>), grid, dim3(256), LDS2, s, p);
             TPAMD_HIP(hipGetLastError());
             hipLaunchKernelGGL((splitk_finish_kernel<DT, MODE>), dim3(MODE == MODE_SWIGLU ? 8 : 16, static_cast<unsigned>(tiles)), dim3(256), 0, s, p, splits);
             TPAMD_HIP(hipGetLastError());

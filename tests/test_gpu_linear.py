@@ -385,6 +385,24 @@ def test_single_matrix_with_few_tiles_at_17_to_64_rows(dtype, M, N, K):
     check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [17, 20, 32, 33, 50, 64])
+@pytest.mark.parametrize("N,K", [(4608, 4096), (5504, 4096), (4100, 2048)])
+def test_k_split_tiles_with_part_of_the_x_tile(tune, dtype, M, N, K):
+    """17 to 64 rows of a single matrix with more than one 16-column tile per CU go to the K-split 128 x 128 kernel, which
+    then loads only the quarter or half of the x tile that exists and lets the two wavefronts of the missing rows only
+    load: against the fp32 host product, and bit for bit what the kernel with whole tiles gives (bias, GELU and the
+    fused addend included; a ragged last column tile)."""
+    x, w, b = rnd((M, K), 1, 1.0, dtype).to(DEV), rnd((N, K), 0, 0.02, dtype).to(DEV), rnd((N,), 2, 0.1, dtype).to(DEV)
+    other = rnd((M, N), 7, 1.0, dtype).to(DEV)
+    part = _native.linear(x, w, b, act=_native.ACT_GELU)
+    part_sum = _native.linear(x, w, None, addend=other)
+    check_half(part, F.gelu(F.linear(x.float().cpu(), w.float().cpu(), b.float().cpu())), K)
+    tune("TPAMD_GEMM_PART_X", "0")
+    assert torch.equal(_native.linear(x, w, b, act=_native.ACT_GELU), part)
+    assert torch.equal(_native.linear(x, w, None, addend=other), part_sum)
+
+
 def test_rows_limit_of_the_weight_streaming_kernels_can_be_forced(tune):
     """TPAMD_SKINNY_MAX_M = 64 sends 17 to 64 rows of any single 16-bit matrix to the weight-streaming kernel, 16 sends
     them to the tiled kernels: same result within rounding."""
