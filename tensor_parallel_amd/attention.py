@@ -187,6 +187,11 @@ def _attend_on_cache(q, k, v, cos, sin, layer, static, scale, layer_idx: int) ->
         if not static.is_initialized:
             static.lazy_initialization(k.transpose(1, 2), v.transpose(1, 2))
         kb, vb = static.keys, static.values
+        if S > 1 and kb.shape[1] != Hkv and kb.shape[0] == B and kb.shape[3] == D and int(static.cumulative_length) == 0:
+            # laid out ahead of its first use (transformers does that for a prefill in chunks), with the whole model's
+            # key/value heads: an empty layer is laid out again for the heads of this rank
+            static.lazy_initialization(k.transpose(1, 2), v.transpose(1, 2))
+            kb, vb = static.keys, static.values
         if kb.shape[0] != B or kb.shape[1] != Hkv or kb.shape[3] != D or kb.dtype != k.dtype:
             raise ValueError(f"the static cache of layer {layer_idx} holds {tuple(kb.shape)} {kb.dtype}, this call needs "
                              f"[{B}, {Hkv}, positions, {D}] {k.dtype}")

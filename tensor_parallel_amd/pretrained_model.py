@@ -138,6 +138,9 @@ class TensorParallelPreTrainedModel(PreTrainedModel, GenerationMixin):
         return self._recorded_decode_step
 
     def _recorded_decode_step(self, **model_inputs):
+        tokens = model_inputs.get("input_ids")
+        if tokens is None or tokens.dim() != 2 or tokens.shape[1] != 1:
+            return self(**model_inputs)  # a chunk of a prefill: its attention asks the cache's count on the host
         model_inputs.pop("attention_mask", None)
         model_inputs = {k: v for k, v in model_inputs.items() if v is not None}
         graphed = self.__dict__.get("_tp_decode_graph")

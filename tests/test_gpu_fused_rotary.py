@@ -223,6 +223,10 @@ def test_generate_on_a_static_cache():
     want3 = plain.generate(ids3, max_new_tokens=6, do_sample=False)
     assert torch.equal(fused.generate(ids3, max_new_tokens=6, do_sample=False, cache_implementation="static"), want3)
     assert fused.__dict__["_tp_decode_graph"] is not first
+    # a prefill in chunks goes through the same hook: its chunks run as they are, the decode steps are replayed
+    long_ids = torch.randint(2, 300, (2, 24), generator=g).to(DEV)
+    chunked = fused.generate(long_ids, max_new_tokens=6, do_sample=False, cache_implementation="static", prefill_chunk_size=8)
+    assert torch.equal(chunked, plain.generate(long_ids, max_new_tokens=6, do_sample=False))
     # modules that were fused without the caller's word about padding take no static cache step as a graph
     halfway = tp.tensor_parallel(deepcopy(model), [DEV, DEV])
     tp.attention.fuse_rotary_(halfway)
