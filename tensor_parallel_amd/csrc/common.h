@@ -41,6 +41,7 @@ struct Tuning {
     int gemm_splitk;         // TPAMD_GEMM_SPLITK: K splits of the 128 x 128 tiling
     int gemm_splitk256;      // TPAMD_GEMM_SPLITK256: K splits of the 256 x 256 tiling
     int gemm_tile;           // TPAMD_GEMM_TILE: 256 or 128
+    int gemm_stages;         // TPAMD_GEMM_STAGES: 4 / 2 = the K-split 128 x 128 kernel with four / two LDS stages (unset: four when there is at most one block per CU)
     int gemm_part_x;         // TPAMD_GEMM_PART_X: 0 = the K-split 128 x 128 kernel loads whole x tiles also for M <= 64
     int skinny_cg;           // TPAMD_SKINNY_CG: column groups per block (1, 2, 4)
     int skinny_pair;         // TPAMD_SKINNY_PAIR: 8-column form of the gated pair

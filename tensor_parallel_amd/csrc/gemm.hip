@@ -944,7 +944,7 @@ __global__ __launch_bounds__(256) void gemm_direct4_kernel(GemmParams p) {
 // have half as many columns each) and keeps whole tiles.
 template <int DT, int MODE, int NS, bool SPLIT, int XQ = 4>
 __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
-    static_assert(XQ == 4 || (SPLIT && NS == 2 && MODE == MODE_LINEAR && (XQ == 1 || XQ == 2)), "part tiles of x: split kernel, single matrix");
+    static_assert(XQ == 4 || (SPLIT && MODE == MODE_LINEAR && (XQ == 1 || XQ == 2)), "part tiles of x: split kernel, single matrix");
     constexpr int BM = 128, BN = 128, WAVES_N = 2, NW = 4;
     constexpr int BLK = 1152;
     constexpr int XREG = (BM / 8) * BLK, WREG = (BN / 8) * BLK, STAGE = XREG + WREG;
@@ -1068,7 +1068,9 @@ __global__ __launch_bounds__(256) void gemm_direct128_kernel(GemmParams p) {
     // the tile's barrier: all fragment reads of this wavefront done, all but the loads of the NS-2 youngest tiles landed
 #define TPAMD_TILE_BARRIER()                                                                                        \
     if constexpr (NS == 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");                 \
-    else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+    else if constexpr (XQ == 4) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");          \
+    else if constexpr (XQ == 2) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");          \
+    else asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
     // prologue: tiles 0 .. NS-2 in flight, tile 0 landed, its first fragments read, first half of tile NS-1 issued
 #pragma unroll
@@ -1858,6 +1860,14 @@ inline double estimate128(int64_t tiles, int KT, int cus, double valid_rows, int
     return best;
 }
 
+template <int DT, int MODE, int NS, int XQ>
+int launch_split128(const GemmParams &p, dim3 grid, int dev, hipStream_t s) {
+    if (int rc = configure128<DT, MODE, NS, true, XQ>(dev); rc != TPAMD_OK) return rc;
+    hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, NS, true, XQ>), grid, dim3(256), NS * 32 * 1152, s, p);
+    TPAMD_HIP(hipGetLastError());
+    return TPAMD_OK;
+}
+
 // 128 x 128 tiles; split over K (fp32 partial tiles in stream-ordered scratch memory, then one finishing pass)
 // when the tiles alone would not give every CU two blocks.
 template <int DT, int MODE>
@@ -1881,29 +1891,26 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     constexpr int LDS2 = 2 * 32 * 1152;
     if (splits > 1) {
         const int xq = MODE != MODE_LINEAR || tuning().gemm_part_x == 0 || tiles > 64 ? 4 : p.M <= 32 ? 1 : p.M <= 64 ? 2 : 4;  // tiles > 64: measured, no gain
-        int rc = configure128<DT, MODE, 2, true>(dev);
-        if constexpr (MODE == MODE_LINEAR) {
-            if (xq == 1) rc = configure128<DT, MODE, 2, true, 1>(dev);
-            else if (xq == 2) rc = configure128<DT, MODE, 2, true, 2>(dev);
-        }
-        if (rc != TPAMD_OK) return rc;
+        // four LDS stages (three K tiles of look-ahead, one block per CU) where every block has its CU to itself anyway:
+        // measured at 24-512 rows, 4096 x 5504 15.5-21.5 -> 14.3-20.3 us, 2048 x 4096 12.8-22.5 -> 11.0-18.5 us, 4096 x 11008
+        // 23.1-29.9 -> 20.9-27.8 us, the gated pair 2 x 4096 x 4096 at 128 rows 28.2 -> 24.5 us; with more units than CUs the
+        // second block of a CU would have to wait for the first, and the launch is 5-15 % slower
+        const bool deep = tuning().gemm_stages != TUNE_UNSET ? tuning().gemm_stages == 4 : tiles * splits <= cus;
         const size_t ws_bytes = static_cast<size_t>(splits) * tiles * 128 * 128 * sizeof(float);
         // the scratch buffer is ours until both launches are enqueued
         std::lock_guard<std::mutex> hold(splitk_mutex(dev));
         void *ws = nullptr;
-        rc = splitk_scratch(dev, s, ws_bytes, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws);
-        if (rc != TPAMD_OK) return rc;
+        if (int rc = splitk_scratch(dev, s, ws_bytes, static_cast<size_t>(4) * cus * 128 * 128 * sizeof(float), &ws); rc != TPAMD_OK) return rc;
         if (ws != nullptr) {
             p.ws = static_cast<float *>(ws);
             const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits));
-            bool launched = false;
+            int launched = -1;
             if constexpr (MODE == MODE_LINEAR) {
-                if (xq == 1) hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true, 1>), grid, dim3(256), LDS2, s, p);
-                else if (xq == 2) hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true, 2>), grid, dim3(256), LDS2, s, p);
-                launched = xq != 4;
+                if (xq == 1) launched = deep ? launch_split128<DT, MODE, 4, 1>(p, grid, dev, s) : launch_split128<DT, MODE, 2, 1>(p, grid, dev, s);
+                else if (xq == 2) launched = deep ? launch_split128<DT, MODE, 4, 2>(p, grid, dev, s) : launch_split128<DT, MODE, 2, 2>(p, grid, dev, s);
             }
-            if (!launched) hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 2, true>), grid, dim3(256), LDS2, s, p);
-            TPAMD_HIP(hipGetLastError());
+            if (launched < 0) launched = deep ? launch_split128<DT, MODE, 4, 4>(p, grid, dev, s) : launch_split128<DT, MODE, 2, 4>(p, grid, dev, s);
+            if (launched != TPAMD_OK) return launched;
             hipLaunchKernelGGL((splitk_finish_kernel<DT, MODE>), dim3(MODE == MODE_SWIGLU ? 8 : 16, static_cast<unsigned>(tiles)), dim3(256), 0, s, p, splits);
             TPAMD_HIP(hipGetLastError());
             return TPAMD_OK;

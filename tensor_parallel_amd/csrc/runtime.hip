@@ -25,6 +25,7 @@ Tuning read_tuning() {
     t.gemm_splitk256 = env_int("TPAMD_GEMM_SPLITK256");
     t.gemm_tile = env_int("TPAMD_GEMM_TILE");
     t.gemm_part_x = env_int("TPAMD_GEMM_PART_X");
+    t.gemm_stages = env_int("TPAMD_GEMM_STAGES");
     t.skinny_cg = env_int("TPAMD_SKINNY_CG");
     t.skinny_pair = env_int("TPAMD_SKINNY_PAIR");
     t.skinny_resident = env_int("TPAMD_SKINNY_RESIDENT");

@@ -403,6 +403,27 @@ def test_k_split_tiles_with_part_of_the_x_tile(tune, dtype, M, N, K):
     assert torch.equal(_native.linear(x, w, None, addend=other), part_sum)
 
 
+@pytest.mark.parametrize("M", [24, 128, 300])
+@pytest.mark.parametrize("N,K", [(2048, 4096), (4096, 5504), (1028, 1088)])
+def test_k_split_tiles_with_two_and_four_lds_stages(tune, M, N, K):
+    """The K-split 128 x 128 kernel keeps four K tiles in LDS where every block has a CU to itself, two otherwise: the same
+    bits either way, for the single matrix (with its part tiles of x at few rows) and for the gated pair, also with the
+    four stages forced on a launch that has more blocks than CUs."""
+    x, w, w2 = rnd((M, K), 1).to(DEV), rnd((N, K), 0, 0.02).to(DEV), rnd((N, K), 5, 0.02).to(DEV)
+    tune("TPAMD_SKINNY_MAX_M", "16")
+    lin, pair = _native.linear(x, w), _native.swiglu_up(x, w, w2)
+    check_half(lin, F.linear(x.float().cpu(), w.float().cpu()), K)
+    for stages in ("2", "4"):
+        tune("TPAMD_GEMM_STAGES", stages)
+        assert torch.equal(_native.linear(x, w), lin) and torch.equal(_native.swiglu_up(x, w, w2), pair)
+    tune("TPAMD_GEMM_SPLITK", "8")  # 8 splits: more blocks than CUs on the larger shapes, still four stages
+    tune("TPAMD_GEMM_TILE", "128")
+    forced = _native.linear(x, w)
+    tune("TPAMD_GEMM_STAGES", "2")
+    assert torch.equal(_native.linear(x, w), forced)
+    check_half(forced, F.linear(x.float().cpu(), w.float().cpu()), K)
+
+
 def test_rows_limit_of_the_weight_streaming_kernels_can_be_forced(tune):
     """TPAMD_SKINNY_MAX_M = 64 sends 17 to 64 rows of any single 16-bit matrix to the weight-streaming kernel, 16 sends
     them to the tiled kernels: same result within rounding."""
