@@ -1840,28 +1840,43 @@ int configure128(int dev) {
     return TPAMD_OK;
 }
 
-// Predicted time (microseconds) of the 128 x 128 tiling and the K split that gives it, from a small cost model
-// fitted (least squares over 290 timings of 48 mid-sized shapes) on this part: a block that has its CU to itself takes
-// 0.82 per K tile, two blocks sharing a CU 0.98 each (the pace of the CU's global->LDS path), 0.92 when blocks queue
-// for several rounds of two per CU; the partial tiles cost 4.6 + 0.39 per MB (written, read back and finished by a
-// second launch; valid_rows = the fraction of the tiles' rows that lie inside M: the others are not stored).
-// Two later terms, fitted on 800 timings of 100 shapes at 64-1024 rows: a split launch whose blocks have a CU each keeps
-// four K tiles in LDS and takes 0.55 per K tile, and no launch streams its weights (tiles_n column tiles of 16 KiB per
-// K tile) faster than 5 TB/s. With them the choices are within 1.5 % of the best split per shape over that sweep
-// (4.7 % before; the Llama-7B down projection at 512 rows: 43.4 -> 36.1 us in two splits instead of four).
-inline double estimate128(int64_t tiles, int64_t tiles_n, int KT, int cus, double valid_rows, int *splits) {
+// Predicted time (microseconds) of the 128 x 128 tiling, with the K split and the number of LDS stages that give it,
+// from a small cost model fitted on this part (least squares over 290 timings of 48 mid-sized shapes, then two sweeps of
+// 100 shapes at 64-2048 rows with every split count and both stage counts, 1500 timings).
+//  - two stages (two blocks fit a CU): a block that has its CU to itself takes 0.82 per K tile, two blocks sharing a CU
+//    0.98 each (the pace of the CU's global->LDS path), 0.92 when blocks queue for several rounds of two per CU;
+//  - four stages (one block per CU, three K tiles of look-ahead), in rounds of one block per CU: split launches 0.55 per
+//    K tile; unsplit ones 0.66 when there is one row tile (every block streams weights nobody shares, about 25 GB/s
+//    per CU), 0.42 with at most half the CUs busy and 0.55 otherwise for a single matrix, 0.62 (two row tiles) / 0.44 and
+//    0.64 for the gated pair;
+//  - no launch streams its weights (tiles_n column tiles of 16 KiB per K tile) faster than 5 TB/s;
+//  - the partial tiles cost 4.6 + 0.39 per MB (written, read back and finished by a second launch; valid_rows = the
+//    fraction of the tiles' rows that lie inside M: the others are not stored).
+// Over the second sweep the choices are within 1.8 % of the best (split, stages) per shape; with two stages only they
+// were 4.7 % off the best split (a single matrix 4096 x 4096 at 1024 rows: 51.5 us unsplit on two stages, 33.7 us on four).
+inline double estimate128(int64_t tiles, int64_t tiles_m, int64_t tiles_n, int KT, int cus, double valid_rows, bool swiglu, int *splits,
+                          bool *deep) {
     double best = 1e30;
     *splits = 1;
+    *deep = false;
+    const double stream = static_cast<double>(tiles_n) * KT * 16384.0 / 5.0e6;
     for (int sp = 1; sp <= 8; ++sp) {
         const int kt = (KT + sp - 1) / sp;
         if (sp > 1 && (kt < 4 || tiles * sp > 4ll * cus)) break;  // too little K per split / more than the scratch buffer holds
-        const double units = static_cast<double>(tiles) * sp;
-        const double rounds = units <= cus ? 1.0 : static_cast<double>((static_cast<int64_t>(units) + 2 * cus - 1) / (2 * cus));
-        const double per_kt = units <= cus ? (sp > 1 ? 0.55 : 0.82) : units <= 2.0 * cus ? 0.98 : 0.92;
-        const double stream = static_cast<double>(tiles_n) * KT * 16384.0 / 5.0e6;
+        const int64_t units = tiles * sp;
+        const double finish = sp > 1 ? 4.6 + units * 0.065536 * valid_rows * 0.39 : 0.0;
+        const double per_deep = sp > 1 ? 0.55
+                                : tiles_m == 1 ? 0.66
+                                : units * 2 <= cus ? (swiglu ? (tiles_m == 2 ? 0.62 : 0.44) : 0.42)
+                                : (swiglu ? 0.64 : 0.55);
+        const double loop_deep = static_cast<double>((units + cus - 1) / cus) * kt * per_deep;
+        const double t_deep = (loop_deep > stream ? loop_deep : stream) + finish;
+        if (t_deep < best) { best = t_deep; *splits = sp; *deep = true; }
+        const double rounds = units <= cus ? 1.0 : static_cast<double>((units + 2 * cus - 1) / (2 * cus));
+        const double per_kt = units <= cus ? 0.82 : units <= 2ll * cus ? 0.98 : 0.92;
         const double loop = rounds * kt * per_kt;
-        const double t = (loop > stream ? loop : stream) + (sp > 1 ? 4.6 + units * 0.065536 * valid_rows * 0.39 : 0.0);
-        if (t < best) { best = t; *splits = sp; }
+        const double t = (loop > stream ? loop : stream) + finish;
+        if (t < best) { best = t; *splits = sp; *deep = false; }
     }
     return best;
 }
@@ -1887,8 +1902,13 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     TPAMD_REQUIRE(tiles < (1ll << 31), "gemm: too many tiles");
     const int KT = p.K / 64;
     int splits = 1;
-    if (tuning().gemm_splitk != TUNE_UNSET) splits = tuning().gemm_splitk;
-    else estimate128(tiles, p.tiles_n, KT, cus, static_cast<double>(p.M) / (p.tiles_m * 128.0), &splits);
+    bool deep = false;
+    estimate128(tiles, p.tiles_m, p.tiles_n, KT, cus, static_cast<double>(p.M) / (p.tiles_m * 128.0), MODE == MODE_SWIGLU, &splits, &deep);
+    if (tuning().gemm_splitk != TUNE_UNSET) {
+        splits = tuning().gemm_splitk;
+        deep = tiles * splits <= cus;
+    }
+    if (tuning().gemm_stages != TUNE_UNSET) deep = tuning().gemm_stages == 4;
     if (splits > 8) splits = 8;
     if (splits > KT) splits = KT;
     if (splits < 1) splits = 1;
@@ -1897,11 +1917,6 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
     constexpr int LDS2 = 2 * 32 * 1152;
     if (splits > 1) {
         const int xq = MODE != MODE_LINEAR || tuning().gemm_part_x == 0 || tiles > 64 ? 4 : p.M <= 32 ? 1 : p.M <= 64 ? 2 : 4;  // tiles > 64: measured, no gain
-        // four LDS stages (three K tiles of look-ahead, one block per CU) where every block has its CU to itself anyway:
-        // measured at 24-512 rows, 4096 x 5504 15.5-21.5 -> 14.3-20.3 us, 2048 x 4096 12.8-22.5 -> 11.0-18.5 us, 4096 x 11008
-        // 23.1-29.9 -> 20.9-27.8 us, the gated pair 2 x 4096 x 4096 at 128 rows 28.2 -> 24.5 us; with more units than CUs the
-        // second block of a CU would have to wait for the first, and the launch is 5-15 % slower
-        const bool deep = tuning().gemm_stages != TUNE_UNSET ? tuning().gemm_stages == 4 : tiles * splits <= cus;
         const size_t ws_bytes = static_cast<size_t>(splits) * tiles * 128 * 128 * sizeof(float);
         // the scratch buffer is ours until both launches are enqueued
         std::lock_guard<std::mutex> hold(splitk_mutex(dev));
@@ -1921,6 +1936,13 @@ int launch_direct128(GemmParams p, int cus, hipStream_t s) {
             TPAMD_HIP(hipGetLastError());
             return TPAMD_OK;
         }
+    }
+    if (deep) {
+        int rc4 = configure128<DT, MODE, 4, false>(dev);
+        if (rc4 != TPAMD_OK) return rc4;
+        hipLaunchKernelGGL((gemm_direct128_kernel<DT, MODE, 4, false>), dim3(static_cast<unsigned>(tiles)), dim3(256), 2 * LDS2, s, p);
+        TPAMD_HIP(hipGetLastError());
+        return TPAMD_OK;
     }
     int rc = configure128<DT, MODE, 2, false>(dev);
     if (rc != TPAMD_OK) return rc;
@@ -1961,8 +1983,10 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
     }
     if (tuning().gemm_splitk256 != TUNE_UNSET) splits256 = tuning().gemm_splitk256;
     int unused_splits = 1;
-    const double t128 = estimate128(small_tiles, (p.N + (swiglu ? 63 : 127)) / (swiglu ? 64 : 128), KT, cus,
-                                    static_cast<double>(p.M) / (((p.M + 127) / 128) * 128.0), &unused_splits);
+    bool unused_deep = false;
+    const int64_t small_tiles_m = (p.M + 127) / 128;
+    const double t128 = estimate128(small_tiles, small_tiles_m, small_tiles / small_tiles_m, KT, cus,
+                                    static_cast<double>(p.M) / (small_tiles_m * 128.0), swiglu, &unused_splits, &unused_deep);
     const bool big = tuning().gemm_tile != TUNE_UNSET ? tuning().gemm_tile == 256 : t256 < t128;
     if (direct_ok) {
         if (big) return swiglu ? launch_direct<DT, MODE_SWIGLU>(p, cus, splits256, s) : launch_direct<DT, MODE_LINEAR>(p, cus, splits256, s);
