@@ -37,11 +37,18 @@ namespace {
 // Largest M served by the weight-streaming kernels; above it the tiled MFMA kernels take over.
 constexpr int64_t SKINNY_MAX_M = 16;
 
-// A single 16-bit matrix with few output tiles per CU stays with the weight-streaming kernel for more rows: the tiled
-// kernels split K over blocks there and pay a second launch. Measured inside a HIP graph (us, tiled | streaming) at
-// 17 / 32 / 48 / 64 rows: 2048 x 4096 13.4 14.1 14.7 15.0 | 9.3 10.3 12.8 13.4; 4096 x 4096 14.5 14.8 15.4 15.9 | 10.8 12.1 14.8 15.7;
-// 4096 x 5504 16.7 17.4 17.8 18.5 | 13.7 15.1 17.9 19.7; 11008 x 4096 24.6 25.4 25.3 26.5 | 26.5 29.0 36.2 39.0. (The gated
-// pair is faster through the tiled kernels at all of these sizes.)
+// A single 16-bit matrix with at most one 16-column tile per CU stays with the weight-streaming kernel for more rows: the
+// tiled kernels split K over blocks there and pay a second launch. How far depends on the row length. Measured inside a
+// HIP graph (us, streaming / tiled) at 17 / 32 / 48 / 64 rows:
+//   2048 x 2048   6.3  6.8  8.6  8.9 /  9.3  9.9 10.3 10.9     4096 x 2048   6.9  7.7 10.2 10.7 / 10.3 11.2 11.6 12.6
+//   3072 x 3072   8.0  9.1 10.7 11.3 / 11.0 11.8 12.0 12.8     (K <= 3072: streaming up to 64 rows)
+//   2048 x 4096   9.1 10.2 12.9 13.5 / 10.6 11.2 11.6 12.2     4096 x 4096  10.0 11.4 14.8 16.0 / 12.0 12.6 13.4 14.4
+//   4096 x 5504  13.5 15.0 18.5 19.9 / 16.3 16.9 18.0 19.1     4096 x 8192  16.7 18.7 23.3 24.7 / 17.9 18.8 19.5 20.3
+//                                                              (longer rows: streaming up to 32 rows)
+//   2048 x 8192  14.4 16.4 21.0 22.9 / 13.2 13.9 15.1 16.0     1536 x 6144  11.8 13.6 17.1 18.5 / 11.7 12.2 12.6 13.1
+//                                                              (K >= 6144 on at most half a tile per CU: tiled from 17 rows)
+// With more tiles the tiled kernels win from 17 rows on (11008 x 4096: 26.5 29.0 36.2 39.0 / 24.6 25.4 25.3 26.5), and the
+// gated pair is faster through them at all of these sizes.
 int skinny_row_limit(int64_t N, int64_t K, int64_t *rows) {
     *rows = SKINNY_MAX_M;
     if (tuning().skinny_max_m != TUNE_UNSET) {
@@ -52,9 +59,9 @@ int skinny_row_limit(int64_t N, int64_t K, int64_t *rows) {
     TPAMD_HIP(hipGetDevice(&dev));
     if (int rc = device_cus(dev, &cus); rc != TPAMD_OK) return rc;
     const int64_t tiles = (N + 15) / 16;
-    if (K < 2048 || K > 8192) return TPAMD_OK;
-    if (tiles * 2 <= cus) *rows = 64;
-    else if (tiles <= cus) *rows = 32;
+    if (K < 2048 || K > 8192 || tiles > cus) return TPAMD_OK;
+    if (K <= 3072) *rows = 64;
+    else if (!(K >= 6144 && tiles * 2 <= cus)) *rows = 32;
     return TPAMD_OK;
 }
 constexpr int64_t SKINNY_W8_SLAB = 64;

@@ -375,11 +375,11 @@ def test_x_resident_weight_streaming_kernel(dtype, M, N, K, tune):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 64])
-@pytest.mark.parametrize("N,K", [(2048, 4096), (4096, 5504), (1000, 2056), (132, 8192)])
+@pytest.mark.parametrize("N,K", [(2048, 4096), (4096, 5504), (1000, 2056), (132, 8192), (3072, 3072)])
 def test_single_matrix_with_few_tiles_at_17_to_64_rows(dtype, M, N, K):
     """A single 16-bit matrix with at most one 16-column tile per CU stays on the weight-streaming kernel up to 32 rows
-    (up to 64 with at most half a tile per CU): two and four row tiles of x, a partly filled last one, a ragged last K
-    chunk, bias and GELU; and the same shapes with the rows limited to 16 (the tiled kernels) agree."""
+    (up to 64 with rows of at most 3072 elements; not at all with long rows on few tiles, which the tiled kernels split
+    over K): two and four row tiles of x, a partly filled last one, a ragged last K chunk, bias and GELU."""
     x, w, b = rnd((M, K), 1, 1.0, dtype), rnd((N, K), 0, 0.02, dtype), rnd((N,), 2, 0.1, dtype)
     got = _native.linear(x.to(DEV), w.to(DEV), b.to(DEV), act=_native.ACT_GELU)
     check_half(got, F.gelu(F.linear(x.float(), w.float(), b.float())), K)
