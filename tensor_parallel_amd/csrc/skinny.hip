@@ -1405,12 +1405,6 @@ inline bool pick_pair(const SkinnyParams &p) {
 //   pair 1376 x 8192:   11.8 12.7 13.7 14.6 | 11.9 11.9 12.1 12.1 | 15.1 15.6 16.6 17.9
 //   pair 16384 x 8192:  85.1 84.9 88.2 93.2 | 93.1 92.4 94.8 95.4 | 86.7 86.6 86.8 87.8
 //   pair 4096 x 2048:    9.2  9.3  9.7 10.0 | 10.5 10.5 10.4 10.6 |  9.5  9.6  9.9 10.2
-//   4096 x 5504:        10.6 11.0 11.3 11.7 | 11.7 12.0 12.1 12.6       (one tile per CU: the plain kernel)
-//   11008 x 4096:       18.1 18.7 23.1 23.7 | 19.1 19.3 19.4 19.8       (2.7 tiles per CU)
-//   32000 x 4096:       43.9 45.1 48.4 49.0 | 44.6 44.8 43.7 44.0
-//   4608 x 8192:        20.7 21.1 21.8 22.7 | 18.4 18.5 18.9 18.8       (1.125 tiles per CU: the plain kernel's blocks fill
-//   8192 x 8192:        25.7 26.0 32.7 32.8 | 30.7 30.5 30.0 30.7        the CUs unevenly)
-//   16384 x 8192:       47.1 47.4 47.8 47.6 | 48.7 49.5 48.9 49.1
 // 16-bit weights, 4 to 16 rows, K from 3072 to 8192 (the x fragments have to fit the registers: 4 chunks per wavefront
 // and 4 register slots for the weights up to K = 4096, 6 and 3 up to 6144, 8 and 2 up to 8192).
 template <int MODE>
@@ -1430,16 +1424,26 @@ inline bool pick_resident(const SkinnyParams &p, int cus) {
         if ((tiles % cus == 0 && tiles <= 4ll * cus) || (tiles > 4ll * cus && tiles < 7ll * cus && p.M <= 8)) return false;
         return tiles > cus || p.M >= 8;
     }
-    // A sweep of 240 shapes (N from 2048 to 16384, K from 2048 to 8192, 4 to 16 rows, in a HIP graph) put the rules below
-    // within 2 % of the better kernel on all but a handful. Between one and two tiles per CU the plain kernel's blocks fill
-    // the CUs unevenly and the persistent x-resident blocks win at every row count (4608 / 5120 / 6144 x 4096 ... 6144:
-    // 8-37 %); at exactly one tile per CU the plain kernel does (4096 x 8192: 10-15 %); two to three tiles per CU at
-    // K = 8192 go to the resident kernel from 10 rows on (11008 / 12288 x 8192 at 12-16 rows: 47 -> 34 us).
-    // Fewer tiles than CUs and long rows (K >= 5504) from 12 rows on: resident by 5-20 % (2048 / 3072 x 5504 ... 8192).
-    const bool between_one_and_two = tiles > cus && tiles < 2ll * cus;
-    const bool few_long = tiles < cus && p.K >= 5504 && p.M >= 12;
-    if (p.K <= 6144) return few_long || (between_one_and_two && (p.K >= 4096 || p.M >= 12)) || (p.M >= 12 && tiles * 2 >= 3ll * cus);
-    return few_long || (tiles > cus && tiles * 2 <= 3ll * cus) || (p.M >= 10 && tiles > cus && tiles <= 3ll * cus);
+    // Single matrix: refitted on a sweep of 900 shapes (N from 1024 to 20480 in steps of 512 and the model widths between,
+    // K from 2048 to 8192, 4 to 16 rows, in a HIP graph, plain | this kernel): the sum over the sweep is 18.9 ms with the
+    // rules before, 18.0 ms with these, 17.98 ms with the better kernel per shape. The persistent x-resident blocks take
+    // the tiles in turn, so a ragged last round costs them nothing, while the plain kernel's blocks fill the CUs unevenly
+    // whenever the tiles are not a whole number of rounds:
+    //  - more tiles than CUs and K >= 4096: this kernel (9216 x 8192 at 4-8 rows 31.1-32.1 -> 27.9-28.5 us, 12544 x 8192 at
+    //    12-16 rows 47.8 -> 37.8 us, 20480 x 5504 at 12-16 rows 56-57 -> 39 us), except, up to 8 rows, on two or four
+    //    whole rounds (8192 and 16384 columns: the plain kernel by 3-9 %);
+    //  - at most one tile per CU: the plain kernel, except long rows on few tiles from 12 rows on (K >= 5504 on at most
+    //    0.7 of the CUs: 5-20 %) and 16 rows on at most half the CUs;
+    //  - K = 3072: from 12 rows on above one tile per CU except between three and four (there the plain kernel wins by
+    //    4-8 %), from 8 rows on above two tiles per CU.
+    const bool even_whole = tiles % (2ll * cus) == 0 && tiles <= 4ll * cus;
+    if (p.K >= 3584) {
+        if (tiles <= cus) return (p.K >= 5504 && p.M >= 12 && tiles * 10 <= 7ll * cus) || (p.M >= 16 && tiles * 2 <= cus);
+        return p.M >= 12 || !even_whole;
+    }
+    if (tiles <= cus) return false;
+    if (p.M >= 12) return !(tiles >= 3ll * cus && tiles < 4ll * cus);
+    return p.M >= 8 && tiles > 2ll * cus && !even_whole;
 }
 
 template <int DT, int MODE>
