@@ -1318,14 +1318,15 @@ void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
 }
 
 // Which kernel takes M <= 3 rows of 16-bit weights. Fitted on a sweep of 342 shapes (single matrix and gated pair, M = 1..3,
-// N = 1376..32000, K = 2048..8192, each timed inside a HIP graph on weights that rotate through more memory than the
+// N = 1376..32000, K = 2048..8192; checked and adjusted on 525 more with other N and K, where it is 1 % off the best choice; each timed inside a HIP graph on weights that rotate through more memory than the
 // caches hold): sum over the sweep 7197 us with the rules before, 6986 us with these, 6948 us with the best kernel per shape.
 //  - a block of W wavefronts owns W output columns (W column pairs of a gated pair) and a CU's share of HBM bandwidth
 //    is what bounds it, so what counts is the most columns any CU gets: ceil(ceil(N / W) / CUs) * W. 16 wavefronts
 //    win when that is no worse than with 8 (N = 5504: 32 against 24 on 256 CUs, 13 % slower) and rows are long enough
 //    to pay for the larger block; 4 wavefronts win on small N where they balance better (N = 2752: 12 against 16);
-//  - 2 rows of long rows (K > 6144 single, K >= 5120 gated pair) on large N go to the MFMA kernels like 3 rows do
-//    (single 8192 x 8192: 24.2 us there, 26.3 us here; pair 5504 x 8192: 29.7 against 33.1 us);
+//  - 2 rows of long rows (K > 6144 single, K >= 5120 gated pair) on 4096 columns or more go to the MFMA kernels like 3
+//    rows do (single 8192 x 8192: 24.2 us there, 26.3 us here; 12800 x 7168: 32.7 against 37.5-41.9 us; pair 5504 x 8192:
+//    29.7 against 33.1 us); a lone row of a long-rowed wide pair goes to the general kernel (12800 x 7168: 55 against 58-66 us);
 //  - gated pairs with 2 rows, 8192 columns or more and K around 4096 go to the general kernel (11008 x 4096: 28.1 against 29.0 us).
 enum RowsPath { ROWS_W4, ROWS_W8, ROWS_W16, ROWS_GENERAL, ROWS_MFMA };
 inline RowsPath pick_rows_path(bool pair, int64_t M, int64_t N, int64_t K, int cus) {
@@ -1334,14 +1335,15 @@ inline RowsPath pick_rows_path(bool pair, int64_t M, int64_t N, int64_t K, int c
     const bool bal16 = most_cols(16) <= most_cols(8) && N >= 2752;
     const bool bal4 = most_cols(4) < most_cols(8) && N < 4096;
     if (!pair) {
-        if (M == 2 && K > 6144) return N >= 4096 && bal16 ? ROWS_MFMA : bal4 ? ROWS_W4 : ROWS_W8;
+        if (M == 2 && K > 6144) return N >= 4096 ? ROWS_MFMA : bal4 ? ROWS_W4 : ROWS_W8;
         if (M == 3) return ROWS_W8;
-        return bal16 && K >= (M == 2 ? 3584 : 3072) ? ROWS_W16 : ROWS_W8;
+        return bal16 && K >= (M == 2 ? 4096 : 3072) ? ROWS_W16 : ROWS_W8;
     }
     const bool near_4096 = K >= 3584 && K <= 4608;
     if (M == 1) {
         if (near_4096 && bal16) return ROWS_W16;
-        return bal4 || (K > 6144 && N >= 2752 && N <= 11008) ? ROWS_W4 : ROWS_W8;
+        if (K > 6144 && N > 11008) return ROWS_GENERAL;
+        return bal4 || (K > 6144 && N >= 2752) ? ROWS_W4 : ROWS_W8;
     }
     if (M == 2) {
         if (K >= 5120 && N >= 4096) return ROWS_MFMA;
@@ -1412,7 +1414,7 @@ inline bool pick_resident(const SkinnyParams &p, int cus) {
     if (p.M > 16 || p.K > 8192) return false;
     if (tuning().skinny_resident != TUNE_UNSET) return tuning().skinny_resident != 0;
     const int64_t tiles = (p.N + (MODE == SK_SWIGLU ? 7 : 15)) / (MODE == SK_SWIGLU ? 8 : 16);
-    if (p.M < 3 || p.K < 3072) return false;
+    if (p.M < (MODE == SK_SWIGLU ? 3 : 2) || p.K < 3072) return false;  // 2 rows of a gated pair: up to 26 % slower here (11008 x 6144)
     if (MODE == SK_SWIGLU) {
         // Refitted on a sweep of 220 pair shapes (N from 1376 to 14336, K from 2048 to 8192, 4 to 16 rows, in a HIP graph,
         // plain 8-column kernel | this one | x staged in LDS). Whole rounds of one tile per CU suit the plain kernel, whose
