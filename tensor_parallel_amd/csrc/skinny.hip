@@ -1463,27 +1463,50 @@ int launch_resident(const SkinnyParams &p, int cus, hipStream_t s) {
     return TPAMD_OK;
 }
 
+// Which of the three int8 kernels takes 2 to 64 rows: the K-split kernel whose wavefronts own columns ("cols": x of the
+// split in LDS, fp32 partial planes, a finishing pass), the older K-split kernel ("split": x in registers) or the unsplit
+// one. Fitted on a sweep of 600 shapes (N 2048-28672, K 2048-16384, 2-64 rows, each kernel forced, inside a HIP graph on
+// weights that rotate through more memory than the caches hold) and checked on 290 random ones: 0.8 % and 0.7 % off the
+// best kernel per shape in the geometric mean (the thresholds on the matrix size that these rules replace: 6.3 % and 5.1 %,
+// up to 80 % on wide matrices with short rows, 11008 x 3072 at 64 rows: 50 us unsplit, 28 us here).
+//  - K >= 4096 and more than 4096 columns: cols, except on one, two or four whole rounds of 16-column tiles per CU
+//    (4096, 8192, 16384 columns on 256 CUs), where the unsplit kernel's blocks fill the CUs evenly and win up to 32 rows
+//    (16384 x 4096 at 16 rows: 18.5 against 21.3 us) unless rows are very long (K > 11008) or there are only 2 of x;
+//    at K = 4096 and 24-32 rows the older split kernel is the faster one off those rounds (11008 x 4096: 5-10 %);
+//  - up to 4096 columns: unsplit, except very long rows (K >= 16384, or K >= 11008 from 48 rows on);
+//  - K < 4096: cols on 18000 columns or more, and from 11008 columns on for 2 rows and from 24 rows on.
+enum W8Path { W8_PLAIN, W8_SPLIT, W8_COLS };
+inline W8Path pick_w8_path(const SkinnyParams &p, int cus) {
+    const int64_t tiles = (p.N + 15) / 16;
+    const bool whole = tiles == cus || (tiles % (2ll * cus) == 0 && tiles <= 4ll * cus);
+    if (p.M < 2) return W8_PLAIN;
+    if (p.K >= 4096) {
+        if (p.N > 4096) {
+            if (!whole || p.M == 2 || p.K > 11008) return p.K < 5120 && p.M >= 24 && p.M <= 32 && !whole ? W8_SPLIT : W8_COLS;
+            if (p.M >= 48) return p.K >= 5120 || p.N >= 16384 ? W8_COLS : W8_SPLIT;
+            return W8_PLAIN;
+        }
+        return p.K >= 16384 || (p.K >= 11008 && p.M >= 48 && p.N >= 3072) ? W8_COLS : W8_PLAIN;
+    }
+    const bool wide = p.N >= 18000 || (p.N >= 11008 && (p.M == 2 || (p.M >= 24 && (!whole || (p.K >= 3072 && p.M >= 48)))));
+    return wide ? W8_COLS : W8_PLAIN;
+}
+
 // int8 weights, K split over blocks: K at least 4096, at most 64 rows and 256 outlier columns.
 // Needs the per-device scratch buffer for the partial sums; without it (first use under stream capture) the
 // caller takes the unsplit kernel.
 template <int DT>
 int launch_w8_split(const SkinnyParams &p, hipStream_t s, bool *done) {
     *done = false;
-    if (tuning().w8_split != TUNE_UNSET) {
-        if (tuning().w8_split == 0) return TPAMD_OK;
-    } else {
-        // Measured (Falcon-40B MLP shard, 16384 x 8192 and 8192 x 16384, and smaller matrices): from 25 rows on it
-        // always pays (32 rows: 57 -> 47 us and 79 -> 49 us, 64 rows: 114 -> 72 us and 156 -> 73 us), from 17 rows
-        // on for matrices of 32 M elements or more, from 12 rows on for 64 M elements or more; below that the
-        // unsplit kernel, with more blocks per CU and no second launch, is as fast or faster.
-        const int64_t elems = static_cast<int64_t>(p.N) * p.K;
-        const bool pays = p.M > 24 || (p.M > 16 && elems >= (1ll << 25)) || (p.M >= 12 && elems >= (1ll << 26));
-        if (!pays) return TPAMD_OK;
-    }
-    if (p.K < 4096 || p.n_out > 256 || p.M > 64) return TPAMD_OK;
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
     if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+    if (tuning().w8_split != TUNE_UNSET) {
+        if (tuning().w8_split == 0) return TPAMD_OK;
+    } else if (pick_w8_path(p, cus) != W8_SPLIT) {
+        return TPAMD_OK;
+    }
+    if (p.K < 4096 || p.n_out > 256 || p.M > 64) return TPAMD_OK;
     // x fragments fill 128 registers: 4 chunks per wavefront (8192 K elements per split) for 16 rows, 2 for 32, 1 for 64
     const int nch = p.M <= 16 ? 4 : p.M <= 32 ? 2 : 1;
     const int splits = (p.K + nch * 2048 - 1) / (nch * 2048);
@@ -1571,17 +1594,13 @@ int launch_w8_cols(const SkinnyParams &p, hipStream_t s, bool *done) {
     *done = false;
     if (tuning().w8_cols == 0) return TPAMD_OK;
     if (p.M > 64 || p.K % 16 != 0 || p.n_out > 256) return TPAMD_OK;
-    if (tuning().w8_cols == TUNE_UNSET) {
-        if (tuning().w8_split != TUNE_UNSET) return TPAMD_OK;  // an explicit choice between the two older kernels
-        // Measured on the Falcon-40B MLP shard (16384 x 8192 and 8192 x 16384, inside a HIP graph, finishing pass included)
-        // against the two older kernels, rows 4 / 8 / 16 / 32 / 64: 30.3 + 34.6 / 34.1 + 37.0 / 37.8 + 40.1 / 46.9 + 50.1 /
-        // 71.5 + 73.9 us -> 29.5 + 30.6 / 31.0 + 31.7 / 34.0 + 34.5 / 39.6 + 39.1 / 54.4 + 52.9 us. Small matrices, where a
-        // block's column range has fewer tiles than wavefronts, stay with the older kernels.
-        if (p.M < 2 || p.K < 4096 || static_cast<int64_t>(p.N) * p.K < (1ll << 25)) return TPAMD_OK;
-    }
     int dev = 0, cus = 256;
     TPAMD_HIP(hipGetDevice(&dev));
     if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
+    if (tuning().w8_cols == TUNE_UNSET) {
+        if (tuning().w8_split != TUNE_UNSET) return TPAMD_OK;  // an explicit choice between the two older kernels
+        if (pick_w8_path(p, cus) != W8_COLS) return TPAMD_OK;
+    }
     if (p.M <= 16) return launch_w8_cols_mt<DT, 1>(p, dev, cus, s, done);
     if (p.M <= 32) return launch_w8_cols_mt<DT, 2>(p, dev, cus, s, done);
     if (p.M <= 48) return launch_w8_cols_mt<DT, 3>(p, dev, cus, s, done);

@@ -189,6 +189,20 @@ def test_k_split_kernel_whose_wavefronts_own_columns(dtype, M, N, K, n_out, tune
     torch.testing.assert_close(got.float(), plain.float(), rtol=2e-2, atol=2e-2 * sigma)
 
 
+@pytest.mark.parametrize("M,N,K", [(2, 11024, 2048), (24, 11024, 3072), (24, 5504, 4096), (16, 8192, 4096), (48, 4352, 5504), (48, 8192, 4096),
+                                   (4, 8192, 11264), (64, 3072, 11008)])
+def test_int8_kernel_chosen_by_shape(M, N, K):
+    """The library's own choice among the three int8 kernels for 2 to 64 rows, on a shape from every branch of the rule
+    (wide matrices with short rows, K = 4096 at 24 rows off and on whole rounds of tiles, few columns with long rows):
+    against the definition."""
+    x, wq, scale, cols, w_out = make_case(M, N, K, 9, torch.bfloat16, seed=6)
+    got = _native.linear_w8(x.to(DEV), torch.from_numpy(wq).to(DEV), torch.from_numpy(scale).to(DEV),
+                            torch.from_numpy(cols.astype(np.int32)).to(DEV), torch.from_numpy(w_out).to(torch.bfloat16).to(DEV))
+    want = oq.linear_w8_f64(x.float().numpy(), wq, scale, cols, w_out)
+    sigma = 0.02 * math.sqrt(K + 400 * 9)
+    torch.testing.assert_close(got.double().cpu(), torch.from_numpy(want), rtol=2e-2, atol=2e-2 * sigma)
+
+
 @pytest.mark.parametrize("knob", ["TPAMD_W8_SPLIT", "TPAMD_W8_COLS"])
 def test_k_split_kernel_inside_a_hip_graph(knob, tune):
     """Either K-split int8 kernel and its finishing pass (two launches sharing the library's scratch buffer) recorded
