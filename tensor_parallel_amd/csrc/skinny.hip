@@ -1324,7 +1324,7 @@ void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
 //    is what bounds it, so what counts is the most columns any CU gets: ceil(ceil(N / W) / CUs) * W. 16 wavefronts
 //    win when that is no worse than with 8 (N = 5504: 32 against 24 on 256 CUs, 13 % slower) and rows are long enough
 //    to pay for the larger block; 4 wavefronts win on small N where they balance better (N = 2752: 12 against 16);
-//  - 2 rows of long rows (K > 6144 single, K >= 5120 gated pair) on 4096 columns or more go to the MFMA kernels like 3
+//  - 2 rows of long rows (K > 6144 single, K >= 7680 gated pair) on 4096 columns or more go to the MFMA kernels like 3
 //    rows do (single 8192 x 8192: 24.2 us there, 26.3 us here; 12800 x 7168: 32.7 against 37.5-41.9 us; pair 5504 x 8192:
 //    29.7 against 33.1 us); a lone row of a long-rowed wide pair goes to the general kernel (12800 x 7168: 55 against 58-66 us);
 //  - gated pairs with 2 rows, 8192 columns or more and K around 4096 go to the general kernel (11008 x 4096: 28.1 against 29.0 us).
@@ -1346,7 +1346,7 @@ inline RowsPath pick_rows_path(bool pair, int64_t M, int64_t N, int64_t K, int c
         return bal4 || (K > 6144 && N >= 2752) ? ROWS_W4 : ROWS_W8;
     }
     if (M == 2) {
-        if (K >= 5120 && N >= 4096) return ROWS_MFMA;
+        if (K >= 5120 && N >= 4096) return K >= 7680 ? ROWS_MFMA : ROWS_GENERAL;  // 7168 x 5120: 24.9 us general, 27.8 us MFMA
         if (K >= 3584 && N >= 8192) return ROWS_GENERAL;
         if (near_4096 && bal16) return ROWS_W16;
         return bal4 ? ROWS_W4 : ROWS_W8;
