@@ -64,6 +64,23 @@ int skinny_row_limit(int64_t N, int64_t K, int64_t *rows) {
     else if (!(K >= 6144 && tiles * 2 <= cus)) *rows = 32;
     return TPAMD_OK;
 }
+// The gated pair with at most one 8-column tile per CU (2048 columns on 256 CUs) and rows of up to 6144 elements stays
+// with the weight-streaming kernel up to 32 rows. Measured inside a HIP graph (us, streaming / tiled) at 17 / 24 / 32 rows:
+//   1376 x 2048   6.6  6.9  7.2 / 10.7 11.5 12.3     2048 x 4096  10.8 10.9 11.6 / 12.2 12.3 12.8
+//   1376 x 4096  10.3 10.3 11.0 / 12.0 12.3 13.1     2048 x 5504  13.7 14.3 15.3 / 14.6 14.9 15.4
+// With more columns the tiled kernels win (2752 x 4096: 17.4 18.4 20.0 / 14.5 14.7 15.1), and on K = 8192 from 1024 columns on.
+int pair_row_limit(int64_t N, int64_t K, int64_t *rows) {
+    *rows = SKINNY_MAX_M;
+    if (tuning().skinny_max_m != TUNE_UNSET) {
+        *rows = tuning().skinny_max_m < 32 ? tuning().skinny_max_m : 32;
+        return TPAMD_OK;
+    }
+    int dev = 0, cus = 256;
+    TPAMD_HIP(hipGetDevice(&dev));
+    if (int rc = device_cus(dev, &cus); rc != TPAMD_OK) return rc;
+    if (K >= 2048 && K <= 6144 && (N + 7) / 8 <= cus) *rows = 32;
+    return TPAMD_OK;
+}
 constexpr int64_t SKINNY_W8_SLAB = 64;
 constexpr int64_t W8_TILED_ABOVE = 128;  // int8 weights: rows from which the tiled MFMA kernel takes over from the slabs
 
@@ -141,7 +158,12 @@ extern "C" int tpamd_swiglu_up(const void *x_dev, const void *wg_dev, const void
     TPAMD_REQUIRE(wu_dev != nullptr, "tpamd_swiglu_up: wu is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool fast = dtype != TPAMD_F32 && mfma_ok(x_dev, wg_dev, wu_dev, nullptr, h_dev, N, K, ldx, ldw, ldh);
-    if (fast && M <= SKINNY_MAX_M)
+    int64_t pair_rows = SKINNY_MAX_M;
+    if (fast && M > SKINNY_MAX_M && M <= 32) {
+        rc = pair_row_limit(N, K, &pair_rows);
+        if (rc != TPAMD_OK) return rc;
+    }
+    if (fast && M <= pair_rows)
         return skinny_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw,
                                ldh, 0, dtype, TPAMD_ACT_NONE, true, false, s);
     return gemm_dispatch(x_dev, wg_dev, wu_dev, nullptr, nullptr, 0, h_dev, M, N, K, ldx, ldw, ldh, dtype, TPAMD_ACT_NONE, true,

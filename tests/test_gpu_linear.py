@@ -459,6 +459,22 @@ def test_gated_pair_with_x_staged_in_lds(dtype, M, N, K, tune):
     torch.testing.assert_close(h.float(), older.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [17, 24, 31, 32])
+@pytest.mark.parametrize("N,K", [(1376, 4096), (2048, 2048), (1000, 2056), (132, 5504)])
+def test_gated_pair_with_few_tiles_at_17_to_32_rows(dtype, M, N, K, tune):
+    """A gated pair with at most one 8-column tile per CU stays on the weight-streaming kernel up to 32 rows (two row
+    tiles of x, the second partly filled; a ragged last K chunk; a column count that is not a multiple of 8): against
+    the oracle's gated hidden state, and against the tiled kernels that take these rows on wider matrices."""
+    x, w, w2 = rnd((M, K), 1, 1.0, dtype).to(DEV), rnd((N, K), 0, 0.02, dtype).to(DEV), rnd((N, K), 5, 0.02, dtype).to(DEV)
+    h = _native.swiglu_up(x, w, w2)
+    sigma = (0.02 * math.sqrt(K)) ** 2
+    torch.testing.assert_close(h.float().cpu(), ofw.gated_mlp_hidden(x.float().cpu(), w.float().cpu(), w2.float().cpu()), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+    tune("TPAMD_SKINNY_MAX_M", "16")
+    tiled = _native.swiglu_up(x, w, w2)
+    torch.testing.assert_close(h.float(), tiled.float(), rtol=RTOL_HALF, atol=RTOL_HALF * sigma)
+
+
 def test_gated_pair_with_x_staged_in_lds_leaves_rows_past_m_and_columns_past_n_alone(tune):
     tune("TPAMD_SKINNY_XLDS", "1")
     M, N, K, ldy = 5, 1001, 4096, 1016
