@@ -1846,7 +1846,7 @@ int configure128(int dev) {
 //  - two stages (two blocks fit a CU): a block that has its CU to itself takes 0.82 per K tile, two blocks sharing a CU
 //    0.98 each (the pace of the CU's global->LDS path), 0.92 when blocks queue for several rounds of two per CU;
 //  - four stages (one block per CU, three K tiles of look-ahead), in rounds of one block per CU: split launches 0.55 per
-//    K tile; unsplit ones 0.66 when there is one row tile (every block streams weights nobody shares, about 25 GB/s
+//    K tile; unsplit ones 0.60 when there is one row tile (every block streams weights nobody shares, about 27 GB/s
 //    per CU), 0.42 with at most half the CUs busy and 0.55 otherwise for a single matrix, 0.62 (two row tiles) / 0.44 and
 //    0.64 for the gated pair;
 //  - no launch streams its weights (tiles_n column tiles of 16 KiB per K tile) faster than 5 TB/s;
@@ -1866,12 +1866,12 @@ inline double estimate128(int64_t tiles, int64_t tiles_m, int64_t tiles_n, int K
         const int64_t units = tiles * sp;
         const double finish = sp > 1 ? 4.6 + units * 0.065536 * valid_rows * 0.39 : 0.0;
         const double per_deep = sp > 1 ? 0.55
-                                : tiles_m == 1 ? 0.66
+                                : tiles_m == 1 ? 0.60
                                 : units * 2 <= cus ? (swiglu ? (tiles_m == 2 ? 0.62 : 0.44) : 0.42)
                                 : (swiglu ? 0.64 : 0.55);
         const double loop_deep = static_cast<double>((units + cus - 1) / cus) * kt * per_deep;
         const double t_deep = (loop_deep > stream ? loop_deep : stream) + finish;
-        if (t_deep < best) { best = t_deep; *splits = sp; *deep = true; }
+        if ((sp == 1 || units <= cus) && t_deep < best) { best = t_deep; *splits = sp; *deep = true; }  // split launches: one round only (measured)
         const double rounds = units <= cus ? 1.0 : static_cast<double>((units + 2 * cus - 1) / (2 * cus));
         const double per_kt = units <= cus ? 0.82 : units <= 2ll * cus ? 0.98 : 0.92;
         const double loop = rounds * kt * per_kt;
@@ -1969,7 +1969,11 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
         const int64_t full = units / cus, last = units % cus;
         return kt * (full * 1.47 + (last == 0 ? 0.0 : last * 4 <= 3ll * cus ? 1.2 : 1.3));
     };
-    double t256 = rounds256(big_tiles, KT);
+    // no launch streams the weights faster than 5 TB/s (what bounds a few rows of a wide matrix: the pair 8192 x 8192 at
+    // 17 rows took 79.8 us on this tiling in four splits, predicted 57 without this term, and 63.8 us on the other)
+    const double stream = static_cast<double>(p.N) * p.K * (swiglu ? 4.0 : 2.0) / 5.0e6;
+    auto floor256 = [&](double loop) { return loop > stream ? loop : stream; };
+    double t256 = floor256(rounds256(big_tiles, KT));
     // ... or split over K while all units still fit one round; the partial tiles cost 9 us + 0.33 us per MB (more than
     // with the small tiles: all blocks finish together, so nothing overlaps the writes and the finishing pass)
     int splits256 = 1;
@@ -1978,7 +1982,7 @@ int gemm_large(GemmParams p, bool swiglu, hipStream_t s) {
         const int kt = (KT + sp - 1) / sp;
         if (kt < 4) break;
         const int64_t units = big_tiles * sp;
-        const double t = rounds256(units, kt) + 9.0 + units * 0.262144 * valid256 * 0.33;
+        const double t = floor256(rounds256(units, kt)) + 9.0 + units * 0.262144 * valid256 * 0.33;
         if (t < t256) { t256 = t; splits256 = sp; }
     }
     if (tuning().gemm_splitk256 != TUNE_UNSET) splits256 = tuning().gemm_splitk256;
