@@ -1330,10 +1330,17 @@ void launch_gemv_rows_m(const SkinnyParams &p, hipStream_t s) {
 //  - gated pairs with 2 rows, 8192 columns or more and K around 4096 go to the general kernel (11008 x 4096: 28.1 against 29.0 us).
 enum RowsPath { ROWS_W4, ROWS_W8, ROWS_W16, ROWS_GENERAL, ROWS_MFMA };
 inline RowsPath pick_rows_path(bool pair, int64_t M, int64_t N, int64_t K, int cus) {
-    if (M == 3 && K >= 3072 && K <= 8192) return ROWS_MFMA;
     auto most_cols = [&](int64_t w) { return ((N + w - 1) / w + cus - 1) / cus * w; };
     const bool bal16 = most_cols(16) <= most_cols(8) && N >= 2752;
     const bool bal4 = most_cols(4) < most_cols(8) && N < 4096;
+    if (M == 3 && K >= 3072 && K <= 8192) {
+        // 3 rows go to the MFMA kernels (Llama-7B MLP shard step: 36.4 us here, 28.3 us there), except a single matrix of at
+        // most 2048 columns (1376 x 6144: 6.5 against 8.4 us, 1024 x 8192: 7.0 against 9.2 us) and, with K near 4096, of at
+        // most 5504 (4096 x 4096: 7.6 against 8.2 us)
+        if (!pair && N <= 2048) return N <= 1024 ? ROWS_W4 : ROWS_W8;
+        if (!pair && K >= 3584 && K <= 4608 && N <= 5504) return bal16 ? ROWS_W16 : ROWS_W8;
+        return ROWS_MFMA;
+    }
     if (!pair) {
         if (M == 2 && K > 6144) return N >= 4096 ? ROWS_MFMA : bal4 ? ROWS_W4 : ROWS_W8;
         if (M == 3) return ROWS_W8;
@@ -1904,7 +1911,7 @@ int skinny_dispatch(const void *x, const void *w, const void *w2, const void *bi
             TPAMD_HIP(hipGetDevice(&dev));
             if (int rc_cus = device_cus(dev, &cus); rc_cus != TPAMD_OK) return rc_cus;
             const int knob = tuning().gemv_rows;  // -1: the MFMA kernels; other values: launch_gemv_rows
-            path = knob == -1 ? ROWS_MFMA : knob != TUNE_UNSET && !(M == 3 && K >= 3072 && K <= 8192) ? ROWS_W8 : pick_rows_path(swiglu, M, N, K, cus);
+            path = knob == -1 ? ROWS_MFMA : knob != TUNE_UNSET ? ROWS_W8 : pick_rows_path(swiglu, M, N, K, cus);
         }
         if (path != ROWS_MFMA) {
             bool done = false;

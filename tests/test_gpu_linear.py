@@ -529,7 +529,7 @@ def test_other_dispatch_paths_inside_a_hip_graph(case, tune):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [1, 2, 3])
-@pytest.mark.parametrize("N,K", [(2048, 512), (2053, 520), (4100, 5504), (6000, 1032), (3000, 8192), (4096, 4096), (8192, 6656), (8200, 4096), (4608, 8192)])
+@pytest.mark.parametrize("N,K", [(2048, 512), (2053, 520), (4100, 5504), (6000, 1032), (3000, 8192), (4096, 4096), (8192, 6656), (8200, 4096), (4608, 8192), (1376, 6144)])
 def test_row_streaming_kernel_on_wide_matrices(dtype, M, N, K):
     """M <= 3 and thousands of output columns (ragged column count, ragged last K step): against the fp32 host
     product, the gated pair against the oracle, the fused sum bit for bit. The shapes reach every choice of the rule
