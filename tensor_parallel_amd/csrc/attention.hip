@@ -628,10 +628,15 @@ int launch(AttnParams p, int cus, hipStream_t s) {
     const bool full_rows = nrows >= 64;
     const int per_cu = (D <= 64 && blocks >= 32) || full_rows ? 2 : 1;
     const int64_t keys_seen = p.causal && p.Sq > 1 ? p.Skv - (p.Sq < p.Skv ? p.Sq : p.Skv) / 2 : p.Skv;  // what a row sees on average
-    if (blocks < static_cast<int64_t>(per_cu) * cus && !(blocks >= cus && keys_seen < 8192) && !(blocks * 2 >= cus && keys_seen <= 512)) {
+    if (blocks < static_cast<int64_t>(per_cu) * cus && !(!full_rows && blocks >= cus && keys_seen < 8192) && !(blocks * 2 >= cus && keys_seen <= 512)) {
         nsplit = static_cast<int>((static_cast<int64_t>(per_cu) * cus + blocks - 1) / blocks);
         int by_keys = static_cast<int>(lroundf(sqrtf(static_cast<float>(keys_seen) / 8.f)));
-        if (full_rows) by_keys = by_keys / 2 < keys_seen / 256 ? by_keys / 2 : static_cast<int>(keys_seen / 256);
+        if (full_rows) {
+            // with a block for every other CU already, a split has to bring 1024 keys or more (224 blocks of 64 rows on 572 keys:
+            // 11.9 us unsplit, 17.6 us in two; 320 blocks on 5936 keys: 88 us unsplit, 68 us in two, 60 us in four)
+            const int64_t min_keys = blocks * 2 >= cus ? 1024 : 256;
+            by_keys = by_keys / 2 < keys_seen / min_keys ? by_keys / 2 : static_cast<int>(keys_seen / min_keys);
+        }
         if (nsplit > by_keys) nsplit = by_keys;
         if (nsplit > 64) nsplit = 64;
         if (nsplit < 1) nsplit = 1;
