@@ -634,7 +634,7 @@ int launch(AttnParams p, int cus, hipStream_t s) {
         if (full_rows) {
             // with a block for every other CU already, a split has to bring 1024 keys or more (224 blocks of 64 rows on 572 keys:
             // 11.9 us unsplit, 17.6 us in two; 320 blocks on 5936 keys: 88 us unsplit, 68 us in two, 60 us in four)
-            const int64_t min_keys = blocks * 2 >= cus ? 1024 : 256;
+            const int64_t min_keys = blocks * 2 >= cus ? 1024 : blocks * 8 < cus ? 128 : 256;  // a handful of blocks: 10 on 692 keys, 10.2 us in two, 8.5 us in four
             by_keys = by_keys / 2 < keys_seen / min_keys ? by_keys / 2 : static_cast<int>(keys_seen / min_keys);
         }
         if (nsplit > by_keys) nsplit = by_keys;
