@@ -1,5 +1,6 @@
-"""Seeded random shapes through the default dispatch of the shard Linears (1 to 70 rows, where the choice of kernel
-depends on M, N and K) against fp32 torch on the host: catches a kernel that is chosen for a shape it mishandles."""
+"""Seeded random shapes through the default dispatch of the shard Linears (1 to 70 rows, and mid-sized problems up to 1500
+rows, where the choice of kernel depends on M, N and K) against fp32 torch on the host: catches a kernel that is chosen for
+a shape it mishandles."""
 import math
 
 import pytest
@@ -50,6 +51,36 @@ def test_gated_pair_random_shape(seed):
     want = ofw.gated_mlp_hidden(x.float(), wg.float(), wu.float())
     sigma = (0.02 * math.sqrt(K)) ** 2
     torch.testing.assert_close(got.float().cpu(), want, rtol=RTOL, atol=RTOL * sigma, msg=lambda m: f"M={M} N={N} K={K} {dtype}: {m}")
+
+
+@pytest.mark.parametrize("seed", range(300, 324))
+def test_mid_sized_random_shape_on_sampled_columns(seed):
+    """17 to 1500 rows of matrices with thousands of columns and long rows: where the tiling (128 x 128 or 256 x 256), the
+    K split, the number of LDS stages and the part of the x tile that is loaded are chosen by cost models. The single
+    matrix (bias, and the fused addend on odd seeds) and the gated pair, on 96 sampled output columns against fp32 on the
+    host (whole matrices of this size would take the host minutes)."""
+    g = torch.Generator().manual_seed(seed)
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    M = [pick(17, 64), pick(65, 300), pick(301, 1500)][pick(0, 2)]
+    N = 64 * pick(16, 224)
+    K = 64 * pick(32, 128)
+    dtype = [torch.bfloat16, torch.float16][pick(0, 1)]
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(dtype)
+    w2 = (torch.randn(N, K, generator=g) * 0.02).to(dtype)
+    b = (torch.randn(N, generator=g) * 0.1).to(dtype)
+    other = torch.randn(M, N, generator=g).to(dtype) if seed % 2 else None
+    cols = torch.randperm(N, generator=g)[:96]
+    xd, wd, w2d = x.to(DEV), w.to(DEV), w2.to(DEV)
+    got = _native.linear(xd, wd, b.to(DEV), addend=None if other is None else other.to(DEV)).float().cpu()[:, cols]
+    want = F.linear(x.float(), w[cols].float(), b[cols].float())
+    if other is not None:
+        want = want.to(dtype).float() + other[:, cols].float()  # the sum is rounded once more, as the fused epilogue does
+    sigma = 0.02 * math.sqrt(K)
+    torch.testing.assert_close(got, want, rtol=RTOL, atol=RTOL * max(sigma, 1.0 if other is not None else 0.0), msg=lambda m: f"linear M={M} N={N} K={K} {dtype}: {m}")
+    pair = _native.swiglu_up(xd, wd, w2d).float().cpu()[:, cols]
+    want = ofw.gated_mlp_hidden(x.float(), w[cols].float(), w2[cols].float())
+    torch.testing.assert_close(pair, want, rtol=RTOL, atol=RTOL * sigma ** 2, msg=lambda m: f"pair M={M} N={N} K={K} {dtype}: {m}")
 
 
 @pytest.mark.parametrize("seed", range(200, 230))
